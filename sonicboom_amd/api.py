@@ -1,0 +1,79 @@
+"""The Python entry point.
+
+Shaped after the reference's C surface (/root/reference/capi/include/sonicboom/capi.h:600-829):
+a model is loaded once (``boom_llm_model_load``), sessions are made from it
+(``boom_llm_session_new``) and own the cache, a session runs steps and
+generation (``boom_llm_prefill`` / ``boom_llm_decode``) with the sampling
+options of ``boom_llm_sampling`` under the same names, and the model's own stop
+tokens are readable (``boom_llm_model_eos``).  Tokens in, tokens out: there is
+no tokenizer here.
+
+    model = Model.load("/path/to/folder", dtype="bfloat16")
+    session = model.session(max_tokens=8192)
+    outs = session.generate([[1, 2, 3], [4, 5]], temperature=0.8, seed=7, max_tokens=32)
+"""
+from __future__ import annotations
+
+from typing import Callable, Iterable, List, Optional, Sequence
+
+from .engine import DecoderModel, Engine, StepEntry, generate
+from .sampling import SamplingParams
+
+
+class Model:
+    def __init__(self, decoder: DecoderModel):
+        self.decoder = decoder
+
+    @classmethod
+    def load(cls, folder: str, dtype: str = "bfloat16", device=None, fast_kernels: bool = True) -> "Model":
+        """Load config.json + safetensors; the model class is chosen by config.json's ``architectures``."""
+        return cls(DecoderModel.from_folder(folder, dtype, device, fast_kernels))
+
+    @classmethod
+    def random(cls, config, seed: int = 0, dtype: str = "bfloat16", device=None,
+               fast_kernels: bool = True) -> "Model":
+        """A model of random weights for a configuration (typed, or a config.json dict)."""
+        return cls(DecoderModel.from_random(config, seed, dtype, device, fast_kernels))
+
+    @property
+    def arch(self) -> str:
+        return self.decoder.spec.architecture
+
+    @property
+    def eos(self) -> tuple:
+        return tuple(self.decoder.spec.stop_tokens)
+
+    @property
+    def vocab_size(self) -> int:
+        return self.decoder.vocab
+
+    def session(self, max_tokens: int, max_slots: Optional[int] = None) -> "Session":
+        """A cache for at most ``max_tokens`` live tokens (each sequence rounded up to 64)."""
+        return Session(self, max_tokens, max_slots)
+
+
+class Session:
+    def __init__(self, model: Model, max_tokens: int, max_slots: Optional[int] = None):
+        self.model = model
+        self.engine = Engine(model.decoder, max_tokens, max_slots)
+
+    def alloc_slot(self) -> int:
+        return self.engine.alloc_slot()
+
+    def free_slot(self, slot: int) -> None:
+        self.engine.free_slot(slot)
+
+    def step(self, entries: Sequence):
+        """entries: (slot, tokens, want) triples or StepEntry; float32 logits [wanted, vocab] on the device."""
+        return self.engine.step([e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries])
+
+    def generate(self, prompts: Sequence[Sequence[int]], temperature: float = 0.0, top_p: float = 1.0,
+                 top_k: int = 0, seed: int = 0, max_tokens: int = 16, min_p: float = 0.0,
+                 repeat_penalty: float = 1.0, repeat_last_n: int = 64, presence_penalty: float = 0.0,
+                 frequency_penalty: float = 0.0, stop_tokens: Optional[Iterable[int]] = None,
+                 max_batch: int = 64, callback: Optional[Callable] = None) -> List[List[int]]:
+        params = SamplingParams(temperature=temperature, top_p=top_p, top_k=top_k, seed=seed,
+                                max_tokens=max_tokens, min_p=min_p, repeat_penalty=repeat_penalty,
+                                repeat_last_n=repeat_last_n, presence_penalty=presence_penalty,
+                                frequency_penalty=frequency_penalty)
+        return generate(self.engine, prompts, params, stop_tokens, max_batch, callback)

@@ -1,0 +1,2 @@
+"""Built-in architectures; importing the package registers them."""
+from . import qwen2  # noqa: F401

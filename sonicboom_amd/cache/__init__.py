@@ -1,0 +1,1 @@
+from .paged import PAGE, CacheError, GroupSpec, PagePool, PagedCache, group_entries, pages_for  # noqa: F401

@@ -1,0 +1,212 @@
+"""The cache: a slot per sequence, paged keys and values per layer, and
+per-sequence state of fixed size.
+
+* A **slot** stands for one live sequence: its length and, per group, the list
+  of physical pages that hold its keys and values.  Slots are handed out by
+  :meth:`PagedCache.alloc_slot`, given back by :meth:`free_slot` and used again.
+* Cache entries (one per mixer that stores keys) with the same needs
+  (kv heads, head size, window) form a **group** with storage and a page pool
+  of its own: ``K, V: [entries, pages, kv_heads, PAGE, head_dim]``.  A group
+  that only reads a window of keys gives pages back as the window leaves them.
+* ``max_tokens`` sizes every pool: the most tokens live sequences hold at any
+  time, each sequence's count rounded up to a whole page (PAGE = 64 tokens).
+* **State**: an entry whose mixer asks for fixed-size state gets a tensor
+  ``[max_slots, *shape]``; a slot's row is zeroed when the slot is handed out,
+  because a recurrence reads its state before it writes it.  Keys and values
+  of a reused page are not cleared: nothing may depend on them.
+
+The reference keeps one sequence per session, position j at row j mod n_slots
+(/root/reference/core/src/planner/kv_cache.h:69-89, :125-170), with per-layer
+specs {kv_heads, head_dim, window} (:96-117) and opaque per-block states
+(:140-152); the batch of slots and the pages are this engine's own.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+
+PAGE = 64
+
+
+class CacheError(RuntimeError):
+    """Out of pages or slots, or a slot used wrongly (unknown, freed twice)."""
+
+
+def pages_for(tokens: int) -> int:
+    return (tokens + PAGE - 1) // PAGE
+
+
+class PagePool:
+    """Free list of physical page numbers; refuses a double free."""
+
+    def __init__(self, n_pages: int):
+        self.n_pages = n_pages
+        self._free = list(range(n_pages - 1, -1, -1))
+        self._held = [False] * n_pages
+
+    @property
+    def free_count(self) -> int:
+        return len(self._free)
+
+    def alloc(self) -> int:
+        if not self._free:
+            raise CacheError("out of cache pages")
+        p = self._free.pop()
+        self._held[p] = True
+        return p
+
+    def free(self, page: int) -> None:
+        if not 0 <= page < self.n_pages or not self._held[page]:
+            raise CacheError(f"page {page} freed while not held")
+        self._held[page] = False
+        self._free.append(page)
+
+
+@dataclass(frozen=True)
+class GroupSpec:
+    kv_heads: int
+    head_dim: int
+    window: int                  # 0: every key is kept
+    entries: Tuple[int, ...]     # cache entry numbers stored in this group
+
+
+@dataclass
+class _Slot:
+    length: int = 0
+    pages: List[List[int]] = field(default_factory=list)   # per group: logical page -> physical or -1
+
+
+class PagedCache:
+    def __init__(self, groups: Sequence[GroupSpec], max_tokens: int, dtype=None, device=None,
+                 state_shapes: Optional[Dict[int, tuple]] = None, max_slots: Optional[int] = None,
+                 allocate: bool = True):
+        if max_tokens <= 0:
+            raise CacheError("max_tokens must be positive")
+        self.groups = list(groups)
+        self.n_pages = pages_for(max_tokens)
+        self.max_slots = max_slots if max_slots is not None else self.n_pages
+        self.pools = [PagePool(self.n_pages) for _ in self.groups]
+        self._slots: Dict[int, _Slot] = {}
+        self._free_slots = list(range(self.max_slots - 1, -1, -1))
+        self.entry_place: Dict[int, Tuple[int, int]] = {}      # entry -> (group, index within group)
+        for g, spec in enumerate(self.groups):
+            for i, e in enumerate(spec.entries):
+                if e in self.entry_place:
+                    raise CacheError(f"cache entry {e} is in two groups")
+                self.entry_place[e] = (g, i)
+        self.k: List = []
+        self.v: List = []
+        self.state: Dict[int, object] = {}
+        self.dtype, self.device = dtype, device
+        if allocate:
+            import torch
+            for spec in self.groups:
+                shape = (len(spec.entries), self.n_pages, spec.kv_heads, PAGE, spec.head_dim)
+                self.k.append(torch.empty(shape, dtype=dtype, device=device))
+                self.v.append(torch.empty(shape, dtype=dtype, device=device))
+            for key, (shape, sdtype) in (state_shapes or {}).items():
+                self.state[key] = torch.zeros((self.max_slots, *shape), dtype=sdtype, device=device)
+
+    # ---- slots -------------------------------------------------------------
+    def alloc_slot(self) -> int:
+        if not self._free_slots:
+            raise CacheError("out of sequence slots")
+        s = self._free_slots.pop()
+        self._slots[s] = _Slot(0, [[] for _ in self.groups])
+        for st in self.state.values():
+            st[s].zero_()
+        return s
+
+    def free_slot(self, slot: int) -> None:
+        sl = self._slots.pop(slot, None)
+        if sl is None:
+            raise CacheError(f"slot {slot} freed while not in use")
+        for g, pages in enumerate(sl.pages):
+            for p in pages:
+                if p >= 0:
+                    self.pools[g].free(p)
+        self._free_slots.append(slot)
+
+    def _slot(self, slot: int) -> _Slot:
+        try:
+            return self._slots[slot]
+        except KeyError:
+            raise CacheError(f"slot {slot} is not in use") from None
+
+    def length(self, slot: int) -> int:
+        return self._slot(slot).length
+
+    @property
+    def live_slots(self) -> List[int]:
+        return sorted(self._slots)
+
+    def held_pages(self, group: int = 0) -> int:
+        return self.n_pages - self.pools[group].free_count
+
+    # ---- a step ------------------------------------------------------------
+    def _first_needed_page(self, g: int, length: int) -> int:
+        """Logical page of the oldest key that a query at position ``length`` still reads."""
+        w = self.groups[g].window
+        if w <= 0:
+            return 0
+        return max(0, length - w + 1) // PAGE
+
+    def reserve(self, slots: Sequence[int], n_new: Sequence[int]) -> None:
+        """Pages for ``n_new[i]`` more tokens of ``slots[i]``, all or nothing."""
+        if len(set(slots)) != len(slots):
+            raise CacheError("a slot appears twice in one step")
+        need = [0] * len(self.groups)
+        for s, n in zip(slots, n_new):
+            if n <= 0:
+                raise CacheError("a step must bring at least one token for every sequence")
+            sl = self._slot(s)
+            for g in range(len(self.groups)):
+                need[g] += pages_for(sl.length + n) - len(sl.pages[g])
+        for g, n in enumerate(need):
+            if n > self.pools[g].free_count:
+                raise CacheError(
+                    f"out of cache pages: the step needs {n} more pages of {PAGE} tokens, "
+                    f"{self.pools[g].free_count} of {self.n_pages} are free")
+        for s, n in zip(slots, n_new):
+            sl = self._slots[s]
+            for g in range(len(self.groups)):
+                while len(sl.pages[g]) < pages_for(sl.length + n):
+                    sl.pages[g].append(self.pools[g].alloc())
+
+    def page_table(self, group: int, slots: Sequence[int], min_width: int = 1) -> np.ndarray:
+        """int32 [len(slots), width]: logical page -> physical page, -1 for none."""
+        rows = [self._slot(s).pages[group] for s in slots]
+        width = max([min_width] + [len(r) for r in rows])
+        t = np.full((len(rows), width), -1, dtype=np.int32)
+        for i, r in enumerate(rows):
+            t[i, :len(r)] = r
+        return t
+
+    def advance(self, slots: Sequence[int], n_new: Sequence[int]) -> None:
+        """The step has run: lengths grow; windowed groups give back pages no later query reads."""
+        for s, n in zip(slots, n_new):
+            sl = self._slot(s)
+            sl.length += n
+            for g in range(len(self.groups)):
+                first = self._first_needed_page(g, sl.length)
+                pages = sl.pages[g]
+                for i in range(min(first, len(pages))):
+                    if pages[i] >= 0:
+                        self.pools[g].free(pages[i])
+                        pages[i] = -1
+
+    # ---- storage -------------------------------------------------------------
+    def entry_views(self, entry: int):
+        """(keys, values) of one cache entry, each [pages, kv_heads, PAGE, head_dim], and its group."""
+        g, i = self.entry_place[entry]
+        return self.k[g][i], self.v[g][i], g
+
+
+def group_entries(specs: Dict[int, Tuple[int, int, int]]) -> List[GroupSpec]:
+    """Group cache entries {entry: (kv_heads, head_dim, window)} by equal needs, in order of first use."""
+    by_need: Dict[Tuple[int, int, int], List[int]] = {}
+    for e in sorted(specs):
+        by_need.setdefault(tuple(specs[e]), []).append(e)
+    return [GroupSpec(k[0], k[1], k[2], tuple(v)) for k, v in by_need.items()]

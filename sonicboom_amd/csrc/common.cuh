@@ -1,0 +1,86 @@
+// Shared device helpers and the host-side error slot of the kernel library.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "sb_hip.h"
+
+typedef uint16_t bf16_t;
+
+// ---- bfloat16 <-> float ----------------------------------------------------
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+  return __uint_as_float(uint32_t(v) << 16);
+}
+// Round to nearest even; a NaN stays a (quiet) NaN.
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return bf16_t((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return bf16_t(u >> 16);
+}
+
+__device__ __forceinline__ float ld_f(const float *p, size_t i) { return p[i]; }
+__device__ __forceinline__ float ld_f(const bf16_t *p, size_t i) { return bf16_to_f32(p[i]); }
+__device__ __forceinline__ void st_f(float *p, size_t i, float v) { p[i] = v; }
+__device__ __forceinline__ void st_f(bf16_t *p, size_t i, float v) { p[i] = f32_to_bf16(v); }
+
+// Value of element i of a buffer whose type is only known at run time.
+__device__ __forceinline__ float ld_dyn(const void *p, int dtype, size_t i) {
+  return dtype == SB_F32 ? ((const float *)p)[i] : bf16_to_f32(((const bf16_t *)p)[i]);
+}
+
+// ---- wave (64 lanes) reductions with a fixed butterfly order -----------------
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+// ---- host side ---------------------------------------------------------------
+namespace sb {
+
+char *error_slot();  // thread-local buffer of SB_ERROR_LEN bytes
+constexpr int kErrorLen = 512;
+
+template <typename... A>
+inline int fail(int code, const char *fmt, A... a) {
+  snprintf(error_slot(), kErrorLen, fmt, a...);
+  return code;
+}
+inline int fail(int code, const char *msg) {
+  snprintf(error_slot(), kErrorLen, "%s", msg);
+  return code;
+}
+
+inline int check_launch(const char *what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(SB_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return SB_OK;
+}
+
+inline bool valid_dtype(int d) { return d == SB_F32 || d == SB_BF16; }
+inline size_t dtype_size(int d) { return d == SB_F32 ? 4 : 2; }
+
+}  // namespace sb
+
+#define SB_REQUIRE(cond, ...)                                  \
+  do {                                                         \
+    if (!(cond)) return sb::fail(SB_ERR_ARGUMENT, __VA_ARGS__); \
+  } while (0)
+#define SB_SUPPORT(cond, ...)                                     \
+  do {                                                            \
+    if (!(cond)) return sb::fail(SB_ERR_UNSUPPORTED, __VA_ARGS__); \
+  } while (0)

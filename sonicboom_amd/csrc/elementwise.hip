@@ -1,0 +1,83 @@
+// SiLU-gated product, residual add, type conversion.
+//
+// silu(g) = g / (1 + expf(-g)) with the full-precision expf, then the product
+// with the up projection (/root/reference/core/src/nn/activation.cpp:41-50,
+// /root/reference/core/src/model/emit.cpp:364-374).
+#include "common.cuh"
+
+namespace {
+
+template <typename TO, typename TI>
+__global__ void silu_mul_kernel(TO *__restrict__ out, const TI *__restrict__ gu, int width,
+                                size_t total) {
+  const size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const size_t row = idx / width;
+  const int col = int(idx - row * width);
+  const TI *g_row = gu + row * size_t(2 * width);
+  const float g = ld_f(g_row, col);
+  const float u = ld_f(g_row, size_t(width) + col);
+  const float act = g / (1.0f + expf(-g));
+  st_f(out, idx, act * u);
+}
+
+template <typename TI>
+__global__ void add_into_kernel(float *__restrict__ resid, const TI *__restrict__ y, size_t n) {
+  const size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx < n) resid[idx] = ld_f(y, idx) + resid[idx];
+}
+
+template <typename TO, typename TI>
+__global__ void cast_kernel(TO *__restrict__ dst, const TI *__restrict__ src, size_t n) {
+  const size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (idx < n) st_f(dst, idx, ld_f(src, idx));
+}
+
+inline unsigned blocks_for(size_t n, int threads) { return unsigned((n + threads - 1) / threads); }
+
+}  // namespace
+
+extern "C" int sb_silu_mul(void *out, int out_dtype, const void *gu, int gu_dtype, int n_rows,
+                           int width, void *stream) {
+  SB_REQUIRE(out && gu, "sb_silu_mul: null pointer");
+  SB_REQUIRE(n_rows >= 0 && width > 0, "sb_silu_mul: bad sizes rows=%d width=%d", n_rows, width);
+  SB_REQUIRE(sb::valid_dtype(out_dtype) && sb::valid_dtype(gu_dtype), "sb_silu_mul: unknown dtype");
+  const size_t total = size_t(n_rows) * width;
+  if (total == 0) return SB_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned nb = blocks_for(total, 256);
+#define SB_GO(TO, TI) silu_mul_kernel<TO, TI><<<nb, 256, 0, s>>>((TO *)out, (const TI *)gu, width, total)
+  if (out_dtype == SB_F32 && gu_dtype == SB_F32) SB_GO(float, float);
+  else if (out_dtype == SB_BF16 && gu_dtype == SB_F32) SB_GO(bf16_t, float);
+  else if (out_dtype == SB_BF16 && gu_dtype == SB_BF16) SB_GO(bf16_t, bf16_t);
+  else SB_GO(float, bf16_t);
+#undef SB_GO
+  return sb::check_launch("sb_silu_mul");
+}
+
+extern "C" int sb_add_into(float *resid, const void *y, int y_dtype, size_t n, void *stream) {
+  SB_REQUIRE(resid && y, "sb_add_into: null pointer");
+  SB_REQUIRE(sb::valid_dtype(y_dtype), "sb_add_into: unknown dtype");
+  if (n == 0) return SB_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned nb = blocks_for(n, 256);
+  if (y_dtype == SB_F32) add_into_kernel<float><<<nb, 256, 0, s>>>(resid, (const float *)y, n);
+  else add_into_kernel<bf16_t><<<nb, 256, 0, s>>>(resid, (const bf16_t *)y, n);
+  return sb::check_launch("sb_add_into");
+}
+
+extern "C" int sb_cast(void *dst, int dst_dtype, const void *src, int src_dtype, size_t n,
+                       void *stream) {
+  SB_REQUIRE(dst && src, "sb_cast: null pointer");
+  SB_REQUIRE(sb::valid_dtype(dst_dtype) && sb::valid_dtype(src_dtype), "sb_cast: unknown dtype");
+  if (n == 0) return SB_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const unsigned nb = blocks_for(n, 256);
+#define SB_GO(TO, TI) cast_kernel<TO, TI><<<nb, 256, 0, s>>>((TO *)dst, (const TI *)src, n)
+  if (dst_dtype == SB_F32 && src_dtype == SB_F32) SB_GO(float, float);
+  else if (dst_dtype == SB_BF16 && src_dtype == SB_F32) SB_GO(bf16_t, float);
+  else if (dst_dtype == SB_BF16 && src_dtype == SB_BF16) SB_GO(bf16_t, bf16_t);
+  else SB_GO(float, bf16_t);
+#undef SB_GO
+  return sb::check_launch("sb_cast");
+}

@@ -1,0 +1,219 @@
+// Token selection on the device: greedy argmax, sampling penalties, and the
+// candidate stage of seeded sampling.
+//
+// Behaviour follows /root/reference/core/src/nn/sampling.cpp: argmax takes the
+// first maximum (:238-244); penalties are v>0 ? v/rp : v*rp, then
+// v -= freq*count + presence, in the float form for the greedy path (:43-70)
+// and the single-rounding fma form for the sampled path (:77-104); candidates
+// are z = l/T as one float division, the 256 largest by (z descending, id
+// ascending) (:257-285).  The filters and the Gumbel draw run on the host.
+#include "common.cuh"
+
+namespace {
+
+constexpr int kSelThreads = 1024;
+constexpr int kSelWaves = kSelThreads / 64;
+constexpr int kMaxCand = 256;
+
+__global__ void __launch_bounds__(kSelThreads)
+argmax_kernel(int32_t *__restrict__ ids, const float *__restrict__ logits, int vocab) {
+  const float *x = logits + size_t(blockIdx.x) * vocab;
+  float best_v = -__builtin_inff();
+  int best_i = 0x7fffffff;
+  for (int i = threadIdx.x; i < vocab; i += kSelThreads) {
+    const float v = x[i];
+    if (best_i == 0x7fffffff || v > best_v) {
+      best_v = v;
+      best_i = i;
+    }
+  }
+  // Larger value wins; equal values go to the lower index.
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ov = __shfl_xor(best_v, off, 64);
+    const int oi = __shfl_xor(best_i, off, 64);
+    if (oi != 0x7fffffff && (best_i == 0x7fffffff || ov > best_v || (ov == best_v && oi < best_i))) {
+      best_v = ov;
+      best_i = oi;
+    }
+  }
+  __shared__ float wv[kSelWaves];
+  __shared__ int wi[kSelWaves];
+  if ((threadIdx.x & 63) == 0) {
+    wv[threadIdx.x >> 6] = best_v;
+    wi[threadIdx.x >> 6] = best_i;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float bv = wv[0];
+    int bi = wi[0];
+    for (int k = 1; k < kSelWaves; ++k) {
+      if (wi[k] != 0x7fffffff && (bi == 0x7fffffff || wv[k] > bv || (wv[k] == bv && wi[k] < bi))) {
+        bv = wv[k];
+        bi = wi[k];
+      }
+    }
+    ids[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
+  }
+}
+
+__global__ void penalize_kernel(float *__restrict__ logits, int vocab,
+                                const int32_t *__restrict__ item_row,
+                                const int32_t *__restrict__ item_token,
+                                const int32_t *__restrict__ item_count, int n_items, float rp,
+                                float presence, float freq, int exact) {
+  const int it = blockIdx.x * blockDim.x + threadIdx.x;
+  if (it >= n_items) return;
+  const int tok = item_token[it];
+  if (tok < 0 || tok >= vocab) return;
+  float *p = logits + size_t(item_row[it]) * vocab + tok;
+  const float c = float(item_count[it]);
+  float v = *p;
+  if (exact) {
+    if (rp != 1.0f) v = v > 0.0f ? __fdiv_rn(v, rp) : __fmul_rn(v, rp);
+    const float adjust = __fmaf_rn(freq, c, presence);
+    v = __fmaf_rn(-1.0f, adjust, v);
+  } else {
+    if (rp != 1.0f) v = v > 0.0f ? __fdiv_rn(v, rp) : __fmul_rn(v, rp);
+    v = __fsub_rn(v, __fadd_rn(__fmul_rn(freq, c), presence));
+  }
+  *p = v;
+}
+
+// Order-preserving map of a float to an unsigned key (larger float, larger key).
+__device__ __forceinline__ uint32_t float_key(float z) {
+  z = z + 0.0f;  // -0 and +0 are one value
+  const uint32_t u = __float_as_uint(z);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_float(uint32_t k) {
+  return __uint_as_float((k & 0x80000000u) ? (k & 0x7fffffffu) : ~k);
+}
+// (z descending, id ascending) as one descending 64-bit order; all keys differ.
+__device__ __forceinline__ uint64_t cand_key(float logit, float temperature, int id) {
+  return (uint64_t(float_key(__fdiv_rn(logit, temperature))) << 32) | uint64_t(0xffffffffu - uint32_t(id));
+}
+
+// One block per row.  Eight radix passes over the 64-bit keys find the key of
+// rank k exactly; every key at or above it is a candidate; a bitonic sort in
+// shared memory orders them.
+__global__ void __launch_bounds__(kSelThreads)
+top_candidates_kernel(int32_t *__restrict__ cand_id, float *__restrict__ cand_z,
+                      const float *__restrict__ logits, int vocab, int k, float temperature) {
+  __shared__ uint32_t hist[kSelWaves][256];
+  __shared__ uint64_t sel[kMaxCand];
+  __shared__ uint64_t prefix_s;
+  __shared__ int remaining_s;
+  __shared__ int count_s;
+  const float *x = logits + size_t(blockIdx.x) * vocab;
+  const int tid = threadIdx.x, wave = tid >> 6;
+  const int want = min(k, vocab);
+  if (tid == 0) {
+    prefix_s = 0;
+    remaining_s = want;
+    count_s = 0;
+  }
+  for (int i = tid; i < kMaxCand; i += kSelThreads) sel[i] = 0;
+
+  for (int pass = 7; pass >= 0; --pass) {
+    const int shift = pass * 8;
+    for (int i = tid; i < kSelWaves * 256; i += kSelThreads) (&hist[0][0])[i] = 0;
+    __syncthreads();
+    const uint64_t prefix = prefix_s;
+    for (int i = tid; i < vocab; i += kSelThreads) {
+      const uint64_t key = cand_key(x[i], temperature, i);
+      if (pass == 7 || (key >> (shift + 8)) == (prefix >> (shift + 8)))
+        atomicAdd(&hist[wave][(key >> shift) & 0xffu], 1u);
+    }
+    __syncthreads();
+    if (tid < 256) {
+      uint32_t total = 0;
+      for (int wv = 0; wv < kSelWaves; ++wv) total += hist[wv][tid];
+      hist[0][tid] = total;
+    }
+    __syncthreads();
+    if (tid == 0) {
+      int remaining = remaining_s;
+      uint32_t above = 0;
+      int chosen = 0;
+      for (int b = 255; b >= 0; --b) {
+        const uint32_t n = hist[0][b];
+        if (above + n >= uint32_t(remaining)) {
+          chosen = b;
+          break;
+        }
+        above += n;
+      }
+      remaining_s = remaining - int(above);
+      prefix_s = prefix | (uint64_t(chosen) << shift);
+    }
+    __syncthreads();
+  }
+
+  const uint64_t kth = prefix_s;
+  for (int i = tid; i < vocab; i += kSelThreads) {
+    const uint64_t key = cand_key(x[i], temperature, i);
+    if (key >= kth) {
+      const int slot = atomicAdd(&count_s, 1);
+      if (slot < kMaxCand) sel[slot] = key;
+    }
+  }
+  __syncthreads();
+
+  // Bitonic sort of 256 keys, descending; empty slots (0) sink to the end.
+  for (int size = 2; size <= kMaxCand; size <<= 1) {
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      if (tid < kMaxCand / 2) {
+        const int lo = ((tid / stride) * stride * 2) + (tid % stride);
+        const int hi = lo + stride;
+        const bool descending = ((lo & size) == 0);
+        const uint64_t a = sel[lo], b = sel[hi];
+        if (descending ? (a < b) : (a > b)) {
+          sel[lo] = b;
+          sel[hi] = a;
+        }
+      }
+      __syncthreads();
+    }
+  }
+  for (int i = tid; i < k; i += kSelThreads) {
+    const uint64_t key = sel[i];
+    const bool real = i < want;
+    cand_id[size_t(blockIdx.x) * k + i] = real ? int32_t(0xffffffffu - uint32_t(key)) : -1;
+    cand_z[size_t(blockIdx.x) * k + i] = real ? key_float(uint32_t(key >> 32)) : 0.0f;
+  }
+}
+
+}  // namespace
+
+extern "C" int sb_argmax(int32_t *ids, const float *logits, int n_rows, int vocab, void *stream) {
+  SB_REQUIRE(ids && logits, "sb_argmax: null pointer");
+  SB_REQUIRE(n_rows >= 0 && vocab > 0, "sb_argmax: bad sizes rows=%d vocab=%d", n_rows, vocab);
+  if (n_rows == 0) return SB_OK;
+  argmax_kernel<<<n_rows, kSelThreads, 0, (hipStream_t)stream>>>(ids, logits, vocab);
+  return sb::check_launch("sb_argmax");
+}
+
+extern "C" int sb_penalize(float *logits, int vocab, const int32_t *item_row, const int32_t *item_token,
+                           const int32_t *item_count, int n_items, float repeat_penalty,
+                           float presence_penalty, float frequency_penalty, int exact, void *stream) {
+  SB_REQUIRE(logits && (n_items == 0 || (item_row && item_token && item_count)), "sb_penalize: null pointer");
+  SB_REQUIRE(n_items >= 0 && vocab > 0, "sb_penalize: bad sizes");
+  if (n_items == 0) return SB_OK;
+  penalize_kernel<<<(n_items + 255) / 256, 256, 0, (hipStream_t)stream>>>(
+      logits, vocab, item_row, item_token, item_count, n_items, repeat_penalty, presence_penalty,
+      frequency_penalty, exact);
+  return sb::check_launch("sb_penalize");
+}
+
+extern "C" int sb_top_candidates(int32_t *cand_id, float *cand_z, const float *logits, int n_rows,
+                                 int vocab, int k, float temperature, void *stream) {
+  SB_REQUIRE(cand_id && cand_z && logits, "sb_top_candidates: null pointer");
+  SB_REQUIRE(n_rows >= 0 && vocab > 0, "sb_top_candidates: bad sizes rows=%d vocab=%d", n_rows, vocab);
+  SB_REQUIRE(temperature > 0.0f, "sb_top_candidates: temperature must be positive");
+  SB_SUPPORT(k >= 1 && k <= kMaxCand, "sb_top_candidates: %d candidates asked, at most %d", k, kMaxCand);
+  if (n_rows == 0) return SB_OK;
+  top_candidates_kernel<<<n_rows, kSelThreads, 0, (hipStream_t)stream>>>(cand_id, cand_z, logits, vocab,
+                                                                         k, temperature);
+  return sb::check_launch("sb_top_candidates");
+}

@@ -1,0 +1,121 @@
+/* C ABI of the sonicboom_amd HIP kernel library (gfx950).
+ *
+ * Conventions, in the manner of the reference's capi.h
+ * (/root/reference/capi/include/sonicboom/capi.h:136-161): every entry point
+ * returns a status, 0 on success; on failure the message of the calling
+ * thread's last error is read with sb_last_error().  No exception crosses
+ * this boundary.  All pointers are device pointers unless said otherwise;
+ * `stream` is a hipStream_t.  Shapes are checked on the host before any
+ * launch; a size that a kernel cannot take is refused with SB_ERR_UNSUPPORTED,
+ * never computed wrongly.
+ *
+ * Element types are named by sb_dtype.  Tensors are row-major and dense unless
+ * a stride is given.  The KV cache is paged: a layer's keys (values) are
+ * [pages][kv_heads][SB_PAGE][head_dim]; `page_table` is int32 [batch][max_pages]
+ * and maps the logical page (position / SB_PAGE) of a sequence to a physical
+ * page, -1 for none.
+ */
+#ifndef SONICBOOM_AMD_SB_HIP_H
+#define SONICBOOM_AMD_SB_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SB_PAGE 64
+
+typedef enum sb_status {
+  SB_OK = 0,
+  SB_ERR_ARGUMENT = 1,    /* null pointer, negative size, inconsistent shapes */
+  SB_ERR_UNSUPPORTED = 2, /* a size or type this kernel does not take */
+  SB_ERR_LAUNCH = 3       /* the HIP runtime refused the launch */
+} sb_status;
+
+typedef enum sb_dtype { SB_F32 = 0, SB_BF16 = 1 } sb_dtype;
+
+/* Message of this thread's last failed call ("" if none). Never NULL. */
+const char *sb_last_error(void);
+/* A JSON object naming the target architecture, the page size and the build flags. */
+const char *sb_build_info(void);
+
+/* out[t,:] = table[ids[t],:]  as f32.  An id outside [0,vocab) yields a NaN row. */
+int sb_embed(float *out, const void *table, int table_dtype, const int32_t *ids,
+             int n_rows, int width, int vocab, void *stream);
+
+/* y[r,:] = (x[src,:] * inv) * w,  inv = 1/sqrt(mean(x[src,:]^2) + eps), src = rows ? rows[r] : r.
+ * x is f32; y is out_dtype; w is w_dtype (NULL = no weight). */
+int sb_rmsnorm(void *y, int out_dtype, const float *x, const void *w, int w_dtype,
+               const int32_t *rows, int n_rows, int width, float eps, void *stream);
+
+/* Y[t,n] = sum_k X[t,k] W[n,k] (+ bias[n]) (+ resid[t,n]).   Plain tiled kernel,
+ * float accumulation in ascending k for every element whatever the batch.
+ * resid is f32 [t,n] and may be the same buffer as Y (when Y is f32). */
+int sb_gemm(void *y, int y_dtype, const void *x, int x_dtype, const void *w, int w_dtype,
+            const void *bias, int bias_dtype, const float *resid,
+            int n_rows, int n_out, int n_in, void *stream);
+
+/* out[t,i] = silu(gu[t,i]) * gu[t,width+i];  gu is [t, 2*width]. */
+int sb_silu_mul(void *out, int out_dtype, const void *gu, int gu_dtype,
+                int n_rows, int width, void *stream);
+
+/* resid[i] += y[i]  (resid f32, y of y_dtype). */
+int sb_add_into(float *resid, const void *y, int y_dtype, size_t n, void *stream);
+
+/* dst[i] = src[i] converted. */
+int sb_cast(void *dst, int dst_dtype, const void *src, int src_dtype, size_t n, void *stream);
+
+/* Rotate the query heads and key heads of a step's qkv rows, write the queries
+ * to q_out and store keys and values into the paged cache.
+ *   qkv        [n_rows, row_stride] of qkv_dtype, read only; a row is
+ *              [heads_q*hd queries | heads_kv*hd keys | heads_kv*hd values]
+ *   q_out      [n_rows, heads_q*hd] of q_dtype
+ *   inv_freq   f32 [rot_dims/2]: angle of pair i at position p is
+ *              float(p)*inv_freq[i], divided by freq_factors[i] when given.
+ *              NULL = no rotation.  Pair i is (i, i + rot_dims/2) of a head.
+ *   row_pos    int32 [n_rows] absolute position;  row_seq int32 [n_rows] index
+ *              of the row's sequence in page_table.
+ *   k_cache/v_cache of cache_dtype; NULL (with heads_kv = 0) for a layer that
+ *              stores nothing.
+ */
+int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int qkv_dtype, int row_stride,
+                     const float *inv_freq, const float *freq_factors, int rot_dims,
+                     const int32_t *row_pos, const int32_t *row_seq, void *k_cache, void *v_cache,
+                     int cache_dtype, const int32_t *page_table, int max_pages, int n_pages_total,
+                     int n_rows, int heads_q, int heads_kv, int head_dim, void *stream);
+
+/* Attention of every row over its sequence's cached keys, position by position:
+ * row r at position p of sequence s sees keys j with j <= p and (window == 0 or
+ * p - j < window).  One wave per (row, query head), 64 keys at a time, online
+ * softmax in f32 whose reduction order depends on key positions only.
+ *   q   [n_rows, q_stride] of act_dtype (heads back to back at the row's start)
+ *   out [n_rows, heads_q*hd] of act_dtype
+ */
+int sb_attention(void *out, const void *q, int act_dtype, int q_stride, const void *k_cache,
+                 const void *v_cache, int cache_dtype, const int32_t *page_table, int max_pages,
+                 int n_pages_total, const int32_t *row_pos, const int32_t *row_seq, int n_rows,
+                 int heads_q, int heads_kv, int head_dim, float scale, int window, void *stream);
+
+/* ids[r] = index of the first maximum of logits[r,:]. */
+int sb_argmax(int32_t *ids, const float *logits, int n_rows, int vocab, void *stream);
+
+/* Sampling penalties on the logits in place, for `n_items` (row, token, count)
+ * triples: v = v>0 ? v/rp : v*rp (when rp != 1), then v -= freq*count + presence.
+ * exact != 0 uses the single-rounding fma form of the sampled path. */
+int sb_penalize(float *logits, int vocab, const int32_t *item_row, const int32_t *item_token,
+                const int32_t *item_count, int n_items, float repeat_penalty,
+                float presence_penalty, float frequency_penalty, int exact, void *stream);
+
+/* The `k` (<= 256) candidates with the largest z = logit / temperature of every
+ * row (ties toward the lower id), ordered by (z descending, id ascending).
+ * cand_id int32 [n_rows,k], cand_z f32 [n_rows,k]; rows with vocab < k are
+ * filled with id -1. */
+int sb_top_candidates(int32_t *cand_id, float *cand_z, const float *logits, int n_rows, int vocab,
+                      int k, float temperature, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,20 @@
+// The error slot and the build description of the kernel library.
+#include "common.cuh"
+
+namespace sb {
+char *error_slot() {
+  static thread_local char slot[kErrorLen] = {0};
+  return slot;
+}
+}  // namespace sb
+
+#ifndef SB_BUILD_FLAGS
+#define SB_BUILD_FLAGS ""
+#endif
+
+extern "C" const char *sb_last_error(void) { return sb::error_slot(); }
+
+extern "C" const char *sb_build_info(void) {
+  return "{\"library\": \"sonicboom_amd\", \"target\": \"gfx950\", \"wave\": 64, "
+         "\"page\": 64, \"flags\": \"" SB_BUILD_FLAGS "\"}";
+}

@@ -1,0 +1,141 @@
+"""The step function: a batch of sequences, the tokens each brings, logits back.
+
+A step carries, for every sequence, either its whole prompt (all sequences of
+the batch start together, lengths differ) or one more token.  The rows of all
+sequences are laid end to end — there is no padding — and run as one batch
+through the model from the cache that earlier steps left: row r of sequence s
+sits at position ``length(s) + r``, stores its key and value there, and sees
+the keys at or before its own position.  The logits come back only for the
+rows that were asked for, in the order of the entries and of their ``want``.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache.paged import CacheError, PagedCache
+from .model import DecoderModel
+
+
+class StepError(ValueError):
+    """A step that cannot run: unknown slot, token outside the vocabulary, no room in the cache."""
+
+
+@dataclass
+class StepEntry:
+    slot: int
+    tokens: Sequence[int]
+    want: Sequence[int] = ()        # indices into ``tokens`` whose logits are wanted
+
+
+class StepContext:
+    """Row and sequence bookkeeping of one step, on the host and on the device.
+
+    Device tensors (int32): ``ids`` [rows], ``row_pos`` [rows] absolute
+    positions, ``row_seq`` [rows] index of the row's sequence in the batch,
+    ``cu_rows`` [seqs+1] first row of every sequence, ``len_before`` [seqs]
+    cached length before the step, ``slots`` [seqs] (rows of the state
+    tensors), ``want_rows`` [wanted]; ``page_table(group)`` [seqs, pages].
+    Host: ``n_rows``, ``n_seqs``, ``n_new`` list, ``lengths_before`` list,
+    ``is_decode`` (every sequence brings one token), ``max_new``,
+    ``max_len_after``.
+    """
+
+    def __init__(self, cache: PagedCache, entries: Sequence[StepEntry], device):
+        self.n_seqs = len(entries)
+        self.n_new = [len(e.tokens) for e in entries]
+        self.slot_list = [e.slot for e in entries]
+        self.lengths_before = [cache.length(s) for s in self.slot_list]
+        self.n_rows = sum(self.n_new)
+        self.is_decode = all(n == 1 for n in self.n_new)
+        self.max_new = max(self.n_new)
+        self.max_len_after = max(l + n for l, n in zip(self.lengths_before, self.n_new))
+        cu = np.zeros(self.n_seqs + 1, dtype=np.int32)
+        cu[1:] = np.cumsum(self.n_new)
+        ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries]).astype(np.int32)
+        row_seq = np.repeat(np.arange(self.n_seqs, dtype=np.int32), self.n_new)
+        row_pos = (np.arange(self.n_rows, dtype=np.int32) - cu[row_seq]
+                   + np.asarray(self.lengths_before, dtype=np.int32)[row_seq]).astype(np.int32)
+        want = [int(cu[i]) + int(w) for i, e in enumerate(entries) for w in e.want]
+        self.n_wanted = len(want)
+        tables = [cache.page_table(g, self.slot_list) for g in range(len(cache.groups))]
+        parts = [ids, row_pos, row_seq, cu, np.asarray(self.lengths_before, dtype=np.int32),
+                 np.asarray(self.slot_list, dtype=np.int32), np.asarray(want, dtype=np.int32)]
+        parts += [t.reshape(-1) for t in tables]
+        sizes = [p.size for p in parts]
+        # One pinned staging buffer, one copy to the device, views into it.
+        host = torch.empty(sum(sizes), dtype=torch.int32, pin_memory=(torch.device(device).type == "cuda"))
+        host.numpy()[:] = np.concatenate(parts) if parts else np.zeros(0, np.int32)
+        dev = host.to(device, non_blocking=True)
+        self._host = host
+        views, off = [], 0
+        for n in sizes:
+            views.append(dev[off:off + n])
+            off += n
+        (self.ids, self.row_pos, self.row_seq, self.cu_rows, self.len_before, self.slots,
+         self.want_rows) = views[:7]
+        self._tables = [v.view(t.shape) for v, t in zip(views[7:], tables)]
+        self.host_row_pos = row_pos
+
+    def page_table(self, group: int) -> torch.Tensor:
+        return self._tables[group]
+
+
+class Engine:
+    """A model with its cache: slots, the step function, and the device."""
+
+    def __init__(self, model: DecoderModel, max_tokens: int, max_slots: Optional[int] = None):
+        self.model = model
+        self.device = model.rt.device
+        self.cache = model.new_cache(max_tokens, max_slots)
+        self.bindings = model.bindings(self.cache)
+
+    # ---- slots -----------------------------------------------------------------
+    def alloc_slot(self) -> int:
+        return self.cache.alloc_slot()
+
+    def free_slot(self, slot: int) -> None:
+        self.cache.free_slot(slot)
+
+    def length(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    # ---- the step ----------------------------------------------------------------
+    def _check(self, entries: Sequence[StepEntry]) -> None:
+        if not entries:
+            raise StepError("a step needs at least one sequence")
+        vocab = self.model.vocab
+        for e in entries:
+            n = len(e.tokens)
+            if n == 0:
+                raise StepError(f"slot {e.slot}: a step must bring at least one token")
+            lo, hi = min(e.tokens), max(e.tokens)
+            if lo < 0 or hi >= vocab:
+                raise StepError(f"slot {e.slot}: token id {hi if hi >= vocab else lo} is outside the vocabulary of {vocab}")
+            for w in e.want:
+                if not 0 <= w < n:
+                    raise StepError(f"slot {e.slot}: wanted row {w} is not among the {n} tokens of this step")
+
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run the entries' tokens; float32 logits [wanted rows, vocab] on the device."""
+        entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        try:
+            self._check(entries)
+            slots = [e.slot for e in entries]
+            n_new = [len(e.tokens) for e in entries]
+            self.cache.reserve(slots, n_new)
+        except CacheError as e:
+            raise StepError(str(e)) from None
+        model = self.model
+        ctx = StepContext(self.cache, entries, self.device)
+        x = model.embedding.forward(ctx.ids)
+        for i, e in enumerate(model.order):
+            model.blocks[e.block].forward(x, ctx, self.bindings[i])
+        self.cache.advance(slots, n_new)
+        if ctx.n_wanted == 0:
+            return torch.empty((0, model.vocab), dtype=torch.float32, device=self.device)
+        h = model.final_norm.forward(x, model.rt.act_dtype, rows=ctx.want_rows)
+        return model.head.forward(h)

@@ -1,0 +1,268 @@
+"""Python faces of the HIP kernels.
+
+Each function checks on the host that the operands have the shapes, types and
+placement its kernel and grid assume, then launches on torch's current stream.
+Tensors are torch tensors on a HIP device; torch is used for memory and
+streams only.  Nothing here falls back to the CPU or to a library routine:
+a missing library or a refused size raises
+:class:`~sonicboom_amd.ops.library.KernelLibraryError`.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import library
+from .library import KernelLibraryError, check
+
+PAGE = 64          # tokens per cache page; SB_PAGE of csrc/sb_hip.h
+MAX_CANDIDATES = 256
+
+_DT = {torch.float32: 0, torch.bfloat16: 1}
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise KernelLibraryError(f"kernels take float32 and bfloat16 tensors, not {t.dtype}") from None
+
+
+def _dev(*ts) -> None:
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise KernelLibraryError("kernel operands must live on the GPU (there is no CPU path)")
+        if not t.is_contiguous():
+            raise KernelLibraryError("kernel operands must be contiguous")
+
+
+def _i32(t: torch.Tensor, n: int, what: str) -> None:
+    if t.dtype != torch.int32 or t.numel() < n:
+        raise KernelLibraryError(f"{what} must be int32 with at least {n} elements")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _p(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+# --------------------------------------------------------------------------
+def embed(table: torch.Tensor, ids: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Rows of ``table`` [vocab, width] named by int32 ``ids`` [n], as float32."""
+    _dev(table, ids, out)
+    if table.dim() != 2:
+        raise KernelLibraryError("embedding table must be [vocab, width]")
+    n = ids.numel()
+    _i32(ids, n, "token ids")
+    vocab, width = table.shape
+    if out is None:
+        out = torch.empty((n, width), dtype=torch.float32, device=table.device)
+    elif out.dtype != torch.float32 or out.numel() != n * width:
+        raise KernelLibraryError("embedding output must be float32 [n, width]")
+    lib = library.core()
+    check(lib.sb_embed(_p(out), _p(table), _dt(table), _p(ids), n, width, vocab, _stream()))
+    return out
+
+
+def rmsnorm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out_dtype: torch.dtype,
+            rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """RMS norm of float32 rows ``x`` [n, width]; ``rows`` (int32) picks and orders source rows."""
+    _dev(x, weight, rows)
+    if x.dtype != torch.float32 or x.dim() != 2:
+        raise KernelLibraryError("rmsnorm input must be float32 [rows, width]")
+    width = x.shape[1]
+    if weight is not None and weight.numel() != width:
+        raise KernelLibraryError(f"rmsnorm weight has {weight.numel()} elements, the rows have {width}")
+    n = x.shape[0] if rows is None else rows.numel()
+    if rows is not None:
+        _i32(rows, n, "row index")
+    y = torch.empty((n, width), dtype=out_dtype, device=x.device)
+    lib = library.core()
+    check(lib.sb_rmsnorm(_p(y), _dt(y), _p(x), _p(weight), _dt(weight) if weight is not None else 0,
+                         _p(rows), n, width, float(eps), _stream()))
+    return y
+
+
+def gemm_plain(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], resid: Optional[torch.Tensor],
+               out_dtype: torch.dtype, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y = x w^T (+bias) (+resid) by the plain tiled kernel; any sizes, f32 or bf16 operands."""
+    _dev(x, w, bias, resid, out)
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
+        raise KernelLibraryError(f"gemm shapes do not match: x {tuple(x.shape)}, w {tuple(w.shape)}")
+    t, k = x.shape
+    n = w.shape[0]
+    if bias is not None and bias.numel() != n:
+        raise KernelLibraryError(f"bias has {bias.numel()} elements, the product has {n} columns")
+    if resid is not None and (resid.dtype != torch.float32 or tuple(resid.shape) != (t, n)):
+        raise KernelLibraryError("the residual must be float32 and shaped like the product")
+    if out is None:
+        out = torch.empty((t, n), dtype=out_dtype, device=x.device)
+    elif out.dtype != out_dtype or tuple(out.shape) != (t, n):
+        raise KernelLibraryError("gemm output buffer has the wrong shape or type")
+    lib = library.core()
+    check(lib.sb_gemm(_p(out), _dt(out), _p(x), _dt(x), _p(w), _dt(w), _p(bias),
+                      _dt(bias) if bias is not None else 0, _p(resid), t, n, k, _stream()))
+    return out
+
+
+def silu_mul(gu: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """silu(gu[:, :w]) * gu[:, w:] for gu [n, 2w]."""
+    _dev(gu)
+    if gu.dim() != 2 or gu.shape[1] % 2:
+        raise KernelLibraryError("silu_mul input must be [rows, 2*width]")
+    n, w2 = gu.shape
+    out = torch.empty((n, w2 // 2), dtype=out_dtype, device=gu.device)
+    lib = library.core()
+    check(lib.sb_silu_mul(_p(out), _dt(out), _p(gu), _dt(gu), n, w2 // 2, _stream()))
+    return out
+
+
+def add_into(resid: torch.Tensor, y: torch.Tensor) -> None:
+    """resid += y (resid float32)."""
+    _dev(resid, y)
+    if resid.dtype != torch.float32 or resid.numel() != y.numel():
+        raise KernelLibraryError("add_into needs a float32 residual and an addend of the same size")
+    lib = library.core()
+    check(lib.sb_add_into(_p(resid), _p(y), _dt(y), resid.numel(), _stream()))
+
+
+def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    _dev(x)
+    if x.dtype == dtype:
+        return x
+    out = torch.empty(x.shape, dtype=dtype, device=x.device)
+    lib = library.core()
+    check(lib.sb_cast(_p(out), _dt(out), _p(x), _dt(x), x.numel(), _stream()))
+    return out
+
+
+def _check_cache(k_cache, v_cache, heads_kv, head_dim):
+    if k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (heads_kv, PAGE, head_dim) or k_cache.shape != v_cache.shape \
+            or k_cache.dtype != v_cache.dtype:
+        raise KernelLibraryError(
+            f"cache must be [pages, {heads_kv}, {PAGE}, {head_dim}] for keys and values alike, "
+            f"found {tuple(k_cache.shape)} and {tuple(v_cache.shape)}")
+
+
+def _check_rows(row_pos, row_seq, page_table, n_rows):
+    _i32(row_pos, n_rows, "row positions")
+    _i32(row_seq, n_rows, "row sequence index")
+    if page_table.dtype != torch.int32 or page_table.dim() != 2:
+        raise KernelLibraryError("page table must be int32 [sequences, pages]")
+
+
+def rope_kv_store(qkv: torch.Tensor, q_dtype: torch.dtype, inv_freq: Optional[torch.Tensor],
+                  freq_factors: Optional[torch.Tensor], rot_dims: int, row_pos: torch.Tensor,
+                  row_seq: torch.Tensor, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                  page_table: Optional[torch.Tensor], heads_q: int, heads_kv: int, head_dim: int) -> torch.Tensor:
+    """Rotate queries and keys of ``qkv`` [n, (hq+2hkv)*hd], return the queries
+    [n, hq*hd] in ``q_dtype`` and store keys and values in the paged cache.
+    ``heads_kv`` = 0 (and no cache) for a layer that stores nothing."""
+    _dev(qkv, inv_freq, freq_factors, row_pos, row_seq, k_cache, v_cache, page_table)
+    n = qkv.shape[0]
+    need = (heads_q + 2 * heads_kv) * head_dim
+    if qkv.dim() != 2 or qkv.shape[1] < need:
+        raise KernelLibraryError(f"qkv rows have {qkv.shape[1]} elements, {need} are needed")
+    if inv_freq is not None:
+        if inv_freq.dtype != torch.float32 or inv_freq.numel() != rot_dims // 2:
+            raise KernelLibraryError("inv_freq must be float32 [rot_dims/2]")
+        if freq_factors is not None and (freq_factors.dtype != torch.float32 or freq_factors.numel() < rot_dims // 2):
+            raise KernelLibraryError("freq_factors must be float32 [rot_dims/2]")
+    _i32(row_pos, n, "row positions")
+    max_pages = n_pages = 0
+    if heads_kv > 0:
+        _check_cache(k_cache, v_cache, heads_kv, head_dim)
+        _check_rows(row_pos, row_seq, page_table, n)
+        max_pages, n_pages = page_table.shape[1], k_cache.shape[0]
+    q = torch.empty((n, heads_q * head_dim), dtype=q_dtype, device=qkv.device)
+    lib = library.core()
+    check(lib.sb_rope_kv_store(
+        _p(q), _dt(q), _p(qkv), _dt(qkv), qkv.shape[1], _p(inv_freq), _p(freq_factors), rot_dims,
+        _p(row_pos), _p(row_seq), _p(k_cache), _p(v_cache), _dt(k_cache) if k_cache is not None else 0,
+        _p(page_table), max_pages, n_pages, n, heads_q, heads_kv, head_dim, _stream()))
+    return q
+
+
+def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor,
+                    row_pos: torch.Tensor, row_seq: torch.Tensor, heads_q: int, heads_kv: int, head_dim: int,
+                    scale: float, window: int) -> torch.Tensor:
+    """Attention of rows ``q`` [n, hq*hd] over the cache, by the plain kernel."""
+    _dev(q, k_cache, v_cache, page_table, row_pos, row_seq)
+    n = q.shape[0]
+    if q.dim() != 2 or q.shape[1] != heads_q * head_dim:
+        raise KernelLibraryError(f"queries must be [rows, {heads_q * head_dim}]")
+    _check_cache(k_cache, v_cache, heads_kv, head_dim)
+    _check_rows(row_pos, row_seq, page_table, n)
+    out = torch.empty((n, heads_q * head_dim), dtype=q.dtype, device=q.device)
+    lib = library.core()
+    check(lib.sb_attention(_p(out), _p(q), _dt(q), q.shape[1], _p(k_cache), _p(v_cache), _dt(k_cache),
+                           _p(page_table), page_table.shape[1], k_cache.shape[0], _p(row_pos), _p(row_seq),
+                           n, heads_q, heads_kv, head_dim, float(scale), int(window), _stream()))
+    return out
+
+
+def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """First maximum of every row of float32 ``logits`` [n, vocab], int32 [n]."""
+    _dev(logits, out)
+    if logits.dtype != torch.float32 or logits.dim() != 2:
+        raise KernelLibraryError("logits must be float32 [rows, vocab]")
+    n, vocab = logits.shape
+    if out is None:
+        out = torch.empty((n,), dtype=torch.int32, device=logits.device)
+    else:
+        _i32(out, n, "argmax output")
+    lib = library.core()
+    check(lib.sb_argmax(_p(out), _p(logits), n, vocab, _stream()))
+    return out
+
+
+def penalize(logits: torch.Tensor, item_row: torch.Tensor, item_token: torch.Tensor, item_count: torch.Tensor,
+             repeat_penalty: float, presence_penalty: float, frequency_penalty: float, exact: bool) -> None:
+    """Apply sampling penalties in place for (row, token, count) triples."""
+    _dev(logits, item_row, item_token, item_count)
+    if logits.dtype != torch.float32 or logits.dim() != 2:
+        raise KernelLibraryError("logits must be float32 [rows, vocab]")
+    n = item_row.numel()
+    for t, what in ((item_row, "item rows"), (item_token, "item tokens"), (item_count, "item counts")):
+        _i32(t, n, what)
+    lib = library.core()
+    check(lib.sb_penalize(_p(logits), logits.shape[1], _p(item_row), _p(item_token), _p(item_count), n,
+                          float(repeat_penalty), float(presence_penalty), float(frequency_penalty),
+                          1 if exact else 0, _stream()))
+
+
+def top_candidates(logits: torch.Tensor, temperature: float, k: int = MAX_CANDIDATES):
+    """The ``k`` best candidates of every row by z = logit / temperature:
+    (ids int32 [n,k], z float32 [n,k]) ordered by (z descending, id ascending)."""
+    _dev(logits)
+    if logits.dtype != torch.float32 or logits.dim() != 2:
+        raise KernelLibraryError("logits must be float32 [rows, vocab]")
+    n, vocab = logits.shape
+    ids = torch.empty((n, k), dtype=torch.int32, device=logits.device)
+    z = torch.empty((n, k), dtype=torch.float32, device=logits.device)
+    lib = library.core()
+    check(lib.sb_top_candidates(_p(ids), _p(z), _p(logits), n, vocab, k, float(temperature), _stream()))
+    return ids, z
+
+
+# --------------------------------------------------------------------------
+# dispatch between the plain kernels and the MFMA kernels
+# --------------------------------------------------------------------------
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], resid: Optional[torch.Tensor],
+              out_dtype: torch.dtype, out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """bfloat16 product by an MFMA kernel, or None when no such kernel takes these sizes."""
+    return None
+
+
+def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor, ctx,
+              heads_q: int, heads_kv: int, head_dim: int, scale: float, window: int,
+              fast: bool = True) -> torch.Tensor:
+    """Attention of a step's rows over the cache; ``ctx`` is the step's context."""
+    return attention_plain(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_seq, heads_q, heads_kv,
+                           head_dim, scale, window)

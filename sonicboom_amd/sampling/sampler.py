@@ -1,0 +1,112 @@
+"""Choosing the next token of every sequence of a step.
+
+The order of stages is the reference's
+(/root/reference/core/include/sonicboom/nn/sampling.h:93-98): penalties over the
+last ``repeat_last_n`` tokens of the history, then either the argmax
+(temperature 0, ties to the lowest id) or: the 256 best candidates by
+z = logit / temperature, a window of 30 below the best, top-k, min-p, top-p,
+and a Gumbel-max draw with a Philox4x32-10 word keyed by (seed, position of
+the token being produced, candidate id).  Penalties, argmax and the candidate
+selection run on the device over the whole batch; the filters and the draw
+work on 256 numbers per sequence and run on the host in float64, as the
+reference's do (/root/reference/core/src/nn/sampling.cpp:157-203, :287-312).
+Every sequence draws from its own (seed, position) stream, so its tokens do
+not depend on what else is in the batch.
+"""
+from __future__ import annotations
+
+from typing import List, Sequence
+
+import numpy as np
+import torch
+
+from .. import ops
+from .params import SamplingParams
+from .philox import philox4x32_10
+
+LOGIT_WINDOW = np.float32(30.0)     # /root/reference/core/include/sonicboom/nn/sampling.h:61
+CANDIDATES = 256                    # /root/reference/core/include/sonicboom/nn/sampling.h:68
+
+
+def penalty_items(histories: Sequence[Sequence[int]], last_n: int, vocab: int):
+    """(row, token, count) triples of the tokens in each history's trailing window."""
+    rows, toks, counts = [], [], []
+    for r, h in enumerate(histories):
+        window = min(len(h), last_n)
+        if window == 0:
+            continue
+        seen = {}
+        for t in h[len(h) - window:]:
+            if 0 <= t < vocab:
+                seen[t] = seen.get(t, 0) + 1
+        for t, c in seen.items():
+            rows.append(r)
+            toks.append(t)
+            counts.append(c)
+    return rows, toks, counts
+
+
+def filter_candidates(ids: np.ndarray, z: np.ndarray, p: SamplingParams):
+    """Window, top-k, min-p and nucleus over candidates ordered (z descending, id ascending)."""
+    if ids.size == 0:
+        return ids, z
+    m = z[0]
+    keep = int(np.count_nonzero(z >= np.float32(m - LOGIT_WINDOW)))
+    if p.top_k > 0:
+        keep = min(keep, p.top_k)
+    ids, z = ids[:keep], z[:keep]
+    if p.min_p > 0.0:
+        cutoff = np.float32(m + np.log(np.float32(p.min_p)))
+        ok = ~(z < cutoff)
+        ids, z = ids[ok], z[ok]
+    if 0.0 < p.top_p < 1.0 and ids.size:
+        e = np.exp(z.astype(np.float64) - np.float64(m))
+        acc = np.cumsum(e)            # sequential, like the reference's running sums
+        total = acc[-1]
+        if total > 0.0:
+            reached = np.nonzero(acc / total >= np.float64(np.float32(p.top_p)))[0]
+            n = int(reached[0]) + 1 if reached.size else ids.size
+            ids, z = ids[:max(n, 1)], z[:max(n, 1)]
+    return ids, z
+
+
+def gumbel_draw(ids: np.ndarray, z: np.ndarray, seed: int, position: int) -> int:
+    """The candidate with the largest z + g, g = -ln(-ln u), u from Philox word 0
+    of counter (position lo, position hi, id, 0); ties go to the lower id."""
+    if ids.size == 0:
+        return -1
+    w0, _, _, _ = philox4x32_10(position & 0xFFFFFFFF, (position >> 32) & 0xFFFFFFFF, ids.astype(np.uint64), 0, seed)
+    u = (w0.astype(np.float64) + 0.5) / 4294967296.0
+    score = z.astype(np.float64) - np.log(-np.log(u))
+    best = score.max()
+    return int(ids[score == best].min())
+
+
+class Sampler:
+    def __init__(self, params: SamplingParams):
+        self.params = params.validated()
+
+    def pick(self, logits: torch.Tensor, positions: Sequence[int], histories: Sequence[Sequence[int]]) -> List[int]:
+        """One token per row of float32 ``logits`` [rows, vocab] (modified in place when
+        penalties apply).  ``positions[r]`` is the absolute position the new token of row r
+        will take; ``histories[r]`` its prompt and generated tokens so far."""
+        p = self.params
+        n, vocab = logits.shape
+        sampled = p.temperature > 0.0
+        if p.has_penalties:
+            rows, toks, counts = penalty_items(histories, p.repeat_last_n, vocab)
+            if rows:
+                dev = logits.device
+                items = torch.tensor([rows, toks, counts], dtype=torch.int32).to(dev)
+                ops.penalize(logits, items[0].contiguous(), items[1].contiguous(), items[2].contiguous(),
+                             p.repeat_penalty, p.presence_penalty, p.frequency_penalty, exact=sampled)
+        if not sampled:
+            return ops.argmax(logits).tolist()
+        k = min(CANDIDATES, vocab)
+        ids_d, z_d = ops.top_candidates(logits, p.temperature, k)
+        ids_h, z_h = ids_d.cpu().numpy(), z_d.cpu().numpy()
+        out = []
+        for r in range(n):
+            ids, z = filter_candidates(ids_h[r], z_h[r], p)
+            out.append(gumbel_draw(ids, z, p.seed, int(positions[r])))
+        return out

@@ -1,0 +1,145 @@
+"""The cache's bookkeeping: slots, pages, windows (CPU, no storage)."""
+import random
+
+import numpy as np
+import pytest
+
+from sonicboom_amd.cache import PAGE, CacheError, GroupSpec, PagedCache, PagePool, group_entries, pages_for
+
+
+def make(max_tokens=64 * 8, window=0, max_slots=None):
+    groups = [GroupSpec(2, 16, 0, (0, 1))]
+    if window:
+        groups.append(GroupSpec(1, 32, window, (2,)))
+    return PagedCache(groups, max_tokens, allocate=False, max_slots=max_slots)
+
+
+def check_invariants(c: PagedCache):
+    """No page lost or held twice: every page is either free or in exactly one slot's list."""
+    for g, pool in enumerate(c.pools):
+        held = [p for s in c.live_slots for p in c._slots[s].pages[g] if p >= 0]
+        assert len(held) == len(set(held)), "a page is held twice"
+        assert len(held) + pool.free_count == c.n_pages, "a page is lost"
+        assert set(held).isdisjoint(pool._free)
+    assert len(c.live_slots) + len(c._free_slots) == c.max_slots
+    assert set(c.live_slots).isdisjoint(c._free_slots)
+
+
+def test_page_pool_refuses_double_free():
+    p = PagePool(3)
+    a, b = p.alloc(), p.alloc()
+    p.free(a)
+    with pytest.raises(CacheError):
+        p.free(a)
+    with pytest.raises(CacheError):
+        p.free(7)
+    p.alloc(), p.alloc()
+    with pytest.raises(CacheError, match="out of cache pages"):
+        p.alloc()
+
+
+def test_slots_are_given_back_and_used_again():
+    c = make(max_slots=2)
+    a, b = c.alloc_slot(), c.alloc_slot()
+    with pytest.raises(CacheError, match="out of sequence slots"):
+        c.alloc_slot()
+    c.reserve([a, b], [70, 1])
+    c.advance([a, b], [70, 1])
+    assert (c.length(a), c.length(b)) == (70, 1) and c.held_pages() == 3
+    c.free_slot(a)
+    with pytest.raises(CacheError, match="freed while not in use"):
+        c.free_slot(a)
+    with pytest.raises(CacheError, match="not in use"):
+        c.length(a)
+    assert c.held_pages() == 1
+    a2 = c.alloc_slot()
+    assert a2 == a and c.length(a2) == 0       # the same slot again, empty
+    check_invariants(c)
+
+
+def test_max_tokens_counts_each_sequence_rounded_up_to_a_page():
+    c = make(max_tokens=64 * 3)
+    s = [c.alloc_slot() for _ in range(3)]
+    c.reserve(s, [1, 64, 5])                  # 1 + 1 + 1 pages
+    c.advance(s, [1, 64, 5])
+    with pytest.raises(CacheError, match="out of cache pages"):
+        c.reserve([s[1]], [1])                # position 64 needs a second page
+    c.reserve([s[0]], [63])                   # still inside its first page
+    c.advance([s[0]], [63])
+    check_invariants(c)
+
+
+def test_reserve_is_all_or_nothing():
+    c = make(max_tokens=64 * 4)
+    a, b = c.alloc_slot(), c.alloc_slot()
+    with pytest.raises(CacheError):
+        c.reserve([a, b], [128, 200])         # 2 + 4 pages > 4
+    assert c.held_pages() == 0
+    with pytest.raises(CacheError, match="twice"):
+        c.reserve([a, a], [1, 1])
+    with pytest.raises(CacheError, match="at least one token"):
+        c.reserve([a], [0])
+    check_invariants(c)
+
+
+def test_page_table_maps_positions_to_pages():
+    c = make()
+    a, b = c.alloc_slot(), c.alloc_slot()
+    c.reserve([a, b], [130, 3])
+    t = c.page_table(0, [b, a])
+    assert t.dtype == np.int32 and t.shape == (2, 3)
+    assert (t[0, 1:] == -1).all() and (t[1] >= 0).all() and len(set(t[1]) | {t[0, 0]}) == 4
+
+
+def test_windowed_group_gives_pages_back():
+    c = make(max_tokens=64 * 16, window=100)
+    s = c.alloc_slot()
+    c.reserve([s], [300])
+    assert c.held_pages(0) == 5 and c.held_pages(1) == 5      # a long prompt needs all its pages in the step
+    c.advance([s], [300])
+    # next query at 300 reads keys 201..300: pages 3.. stay, 0..2 go back
+    assert c.held_pages(0) == 5 and c.held_pages(1) == 2
+    t = c.page_table(1, [s])
+    assert (t[0, :3] == -1).all() and (t[0, 3:5] >= 0).all()
+    for _ in range(200):
+        c.reserve([s], [1])
+        c.advance([s], [1])
+        assert c.held_pages(1) <= pages_for(100) + 1
+    check_invariants(c)
+    c.free_slot(s)
+    assert c.held_pages(0) == 0 and c.held_pages(1) == 0
+
+
+def test_random_traffic_keeps_the_books():
+    rnd = random.Random(7)
+    c = make(max_tokens=64 * 40, window=70, max_slots=6)
+    live = {}
+    for _ in range(600):
+        r = rnd.random()
+        if r < 0.25 and len(live) < 6:
+            live[c.alloc_slot()] = 0
+        elif r < 0.4 and live:
+            s = rnd.choice(list(live))
+            c.free_slot(s)
+            del live[s]
+        elif live:
+            chosen = rnd.sample(list(live), rnd.randint(1, len(live)))
+            n = [rnd.choice([1, 1, 1, 17, 64, 90]) for _ in chosen]
+            try:
+                c.reserve(chosen, n)
+            except CacheError:
+                check_invariants(c)
+                continue
+            c.advance(chosen, n)
+            for s, k in zip(chosen, n):
+                live[s] += k
+        check_invariants(c)
+        assert all(c.length(s) == n for s, n in live.items())
+
+
+def test_groups_by_need():
+    g = group_entries({0: (2, 16, 0), 1: (2, 16, 0), 2: (2, 16, 128), 3: (4, 16, 0)})
+    assert [(x.kv_heads, x.head_dim, x.window, x.entries) for x in g] == [
+        (2, 16, 0, (0, 1)), (2, 16, 128, (2,)), (4, 16, 0, (3,))]
+    with pytest.raises(CacheError, match="two groups"):
+        PagedCache([GroupSpec(1, 16, 0, (0,)), GroupSpec(1, 16, 4, (0,))], 64, allocate=False)
