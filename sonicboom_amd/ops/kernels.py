@@ -254,10 +254,44 @@ def top_candidates(logits: torch.Tensor, temperature: float, k: int = MAX_CANDID
 # --------------------------------------------------------------------------
 # dispatch between the plain kernels and the MFMA kernels
 # --------------------------------------------------------------------------
+SKINNY_MAX_ROWS = 64
+
+
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], resid: Optional[torch.Tensor],
-              out_dtype: torch.dtype, out: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
-    """bfloat16 product by an MFMA kernel, or None when no such kernel takes these sizes."""
-    return None
+              out_dtype: torch.dtype, out: Optional[torch.Tensor] = None, gated: bool = False
+              ) -> Optional[torch.Tensor]:
+    """bfloat16 product on the matrix cores: y = x w^T (+bias) (+resid), or with ``gated``
+    y = silu(x wg^T) * (x wu^T) for w = [wg; wu].  Up to 64 rows go to the weight-streaming
+    kernel, more to the tiled one.  Returns None when the sizes fit neither (an inner size
+    that is not a multiple of 8): the caller then takes the plain kernel."""
+    _dev(x, w, bias, resid, out)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        return None
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
+        raise KernelLibraryError(f"gemm shapes do not match: x {tuple(x.shape)}, w {tuple(w.shape)}")
+    t, k = x.shape
+    n = w.shape[0] // 2 if gated else w.shape[0]
+    if k % 8 or x.data_ptr() % 16 or w.data_ptr() % 16 or (gated and w.shape[0] % 2):
+        return None
+    if bias is not None and bias.numel() != n:
+        raise KernelLibraryError(f"bias has {bias.numel()} elements, the product has {n} columns")
+    if resid is not None and (resid.dtype != torch.float32 or tuple(resid.shape) != (t, n)):
+        raise KernelLibraryError("the residual must be float32 and shaped like the product")
+    if out is None:
+        out = torch.empty((t, n), dtype=out_dtype, device=x.device)
+    elif out.dtype != out_dtype or tuple(out.shape) != (t, n):
+        raise KernelLibraryError("gemm output buffer has the wrong shape or type")
+    lib = library.core()
+    bdt = _dt(bias) if bias is not None else 0
+    if t <= SKINNY_MAX_ROWS:
+        need = lib.sb_gemm_skinny_scratch(t, n, k, 1 if gated else 0)
+        scratch = torch.empty((need,), dtype=torch.float32, device=x.device) if need else None
+        check(lib.sb_gemm_skinny_bf16(_p(out), _dt(out), _p(x), _p(w), _p(bias), bdt, _p(resid), t, n, k,
+                                      1 if gated else 0, _p(scratch), need, _stream()))
+    else:
+        check(lib.sb_gemm_mfma_bf16(_p(out), _dt(out), _p(x), _p(w), _p(bias), bdt, _p(resid), t, n, k,
+                                    1 if gated else 0, _stream()))
+    return out
 
 
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor, ctx,

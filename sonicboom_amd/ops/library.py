@@ -33,7 +33,7 @@ _CORE_SIGNATURES = {
 }
 # Entry points of later kernels; declared when the library has them.
 _OPTIONAL_SIGNATURES = {
-    "sb_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P],
+    "sb_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P, _Z, _P],
     "sb_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P],
 }
 _ATTN_SIGNATURES = {
@@ -73,6 +73,8 @@ def core():
                 lib.sb_build_info.restype = c_char_p
                 _declare(lib, _CORE_SIGNATURES)
                 _declare(lib, _OPTIONAL_SIGNATURES, optional=True)
+                lib.sb_gemm_skinny_scratch.argtypes = [_I, _I, _I, _I]
+                lib.sb_gemm_skinny_scratch.restype = c_size_t
                 lib._sb_path = path
                 _core = lib
     return _core

@@ -45,6 +45,5 @@ class GatedDenseFFN(Part):
         self.down = Linear(tensors["down_weight"], None, rt.fast_kernels)
 
     def forward(self, h, x, ctx) -> None:
-        gu = self.gate_up(h, torch.float32)
-        mid = ops.silu_mul(gu, self.rt.act_dtype)
+        mid = self.gate_up.gated(h, self.rt.act_dtype)
         self.down(mid, torch.float32, resid=x, out=x)

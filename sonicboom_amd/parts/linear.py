@@ -38,3 +38,13 @@ class Linear:
             if y is not None:
                 return y
         return ops.gemm_plain(x, w, self.bias, resid, out_dtype, out)
+
+    def gated(self, x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        """silu(x Wg^T) * (x Wu^T) for a stacked weight [Wg; Wu]: one fused kernel on the
+        matrix cores when the sizes allow, else the product in float32 and the activation kernel."""
+        w = self.weight
+        if self.fast and w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
+            y = ops.gemm_bf16(x, w, None, None, out_dtype, gated=True)
+            if y is not None:
+                return y
+        return ops.silu_mul(self(x, torch.float32), out_dtype)

@@ -173,6 +173,45 @@ def swiglu(f: np.ndarray, w_gate, w_up, w_down) -> np.ndarray:
     return linear((g * u).astype(F32), w_down)
 
 
+def rope_scaling(cfg: dict):
+    """(freq_factors or None, multiplier of the attention scores) from config.json's
+    ``rope_scaling`` {type|rope_type, factor, original_max_position_embeddings,
+    beta_fast, beta_slow, attention_factor}.
+
+    core/src/model/loader.cpp:226-311: theta(i) = pos * base^(-2i/d) / ff[i] with
+    ff[i] = 1/alpha(i); linear: alpha = 1/factor; YaRN: alpha = fs (1 - ramp) + ramp
+    with ramp(i) = 1 - clamp((i - lo) / max(0.001, hi - lo), 0, 1),
+    corr(beta) = d ln(orig / (2 pi beta)) / (2 ln base), lo = max(0, floor(corr(beta_fast))),
+    hi = min(d - 1, ceil(corr(beta_slow))); YaRN multiplies the scores by m^2,
+    m = (1 + 0.1 ln factor) * attention_factor for factor > 1.
+    """
+    rs = cfg.get("rope_scaling")
+    if not rs:
+        return None, 1.0
+    kind = rs.get("rope_type", rs.get("type"))
+    if kind in (None, "none", "default"):
+        return None, 1.0
+    d = cfg["_head_dim"]
+    base = float(cfg["rope_theta"])
+    factor = float(rs["factor"])
+    fs = 1.0 / factor
+    ff = []
+    if kind == "linear":
+        return [F32(factor)] * (d // 2), 1.0
+    assert kind == "yarn", kind
+    orig = rs.get("original_max_position_embeddings", cfg.get("max_position_embeddings"))
+    corr = lambda beta: d * math.log(orig / (beta * 2.0 * math.pi)) / (2.0 * math.log(base))  # noqa: E731
+    lo = max(0.0, math.floor(corr(float(rs.get("beta_fast", 32.0)))))
+    hi = min(d - 1.0, math.ceil(corr(float(rs.get("beta_slow", 1.0)))))
+    for i in range(d // 2):
+        y = (i - lo) / max(0.001, hi - lo)
+        ramp = 1.0 - min(1.0, max(0.0, y))
+        alpha = fs * (1.0 - ramp) + ramp
+        ff.append(F32(1.0 / alpha))
+    m = (1.0 if factor <= 1.0 else 1.0 + 0.1 * math.log(factor)) * float(rs.get("attention_factor", 1.0))
+    return ff, float(F32(m * m))
+
+
 def self_attention(h: np.ndarray, positions, w: dict, prefix: str, cfg: dict) -> np.ndarray:
     """q = Wq h + bq, rotated; k = Wk h + bk, rotated; v = Wv h + bv;
     causal GQA with scale 1/sqrt(head_dim); o = Wo attn (no bias).
@@ -180,16 +219,18 @@ def self_attention(h: np.ndarray, positions, w: dict, prefix: str, cfg: dict) ->
     core/src/model/emit.cpp:255-308 (both matmuls, both biases, the bias
     precedes the rotation, V is not rotated, the output projection has no
     bias for Qwen2), core/src/model/recipe.cpp:65-70 and :153-167 (q/k/v bias,
-    score scale 1/sqrt(head_dim)), core/src/model/loader.cpp:656-671 (head_dim
+    score scale 1/sqrt(head_dim)), core/src/model/loader.cpp:656-671, :945 (head_dim
     = width / heads, every layer global: no window).
     """
     hq, hkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["_head_dim"]
     q = linear(h, w[prefix + "q_proj.weight"], w[prefix + "q_proj.bias"])
     k = linear(h, w[prefix + "k_proj.weight"], w[prefix + "k_proj.bias"])
     v = linear(h, w[prefix + "v_proj.weight"], w[prefix + "v_proj.bias"])
-    q = rope_neox(q, positions, hd, cfg["rope_theta"])
-    k = rope_neox(k, positions, hd, cfg["rope_theta"])
-    scale = F32(1.0) / np.sqrt(F32(hd))
+    ff, score_mult = rope_scaling(cfg)
+    q = rope_neox(q, positions, hd, cfg["rope_theta"], freq_factors=ff)
+    k = rope_neox(k, positions, hd, cfg["rope_theta"], freq_factors=ff)
+    # core/src/model/recipe.cpp:165-167: the architecture's 1/sqrt(head_dim) times YaRN's magnitude term
+    scale = F32(F32(1.0) / np.sqrt(F32(hd))) * F32(score_mult)
     a = attention(q, k, v, positions, positions, hq, hkv, hd, float(scale),
                   causal=True, window=0)
     return linear(a, w[prefix + "o_proj.weight"])

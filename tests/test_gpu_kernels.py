@@ -1,0 +1,367 @@
+"""Each kernel alone against a plain reference of the same operation, at sizes other
+than the engine's tiny configurations: widths that are no power of two, ragged row
+counts, head sizes in steps of 16, any number of heads and groups."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from plain import qwen2_plain as plain
+from plain import sampling_plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+BF16, F32 = torch.bfloat16, torch.float32
+
+
+def randn(*shape, dtype=F32, scale=1.0, seed=0):
+    g = torch.Generator().manual_seed(seed + sum(shape))
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+def close(got, want, atol, rtol, what=""):
+    got = got.detach().float().cpu().double()
+    want = torch.as_tensor(want).double()
+    assert got.shape == want.shape, f"{what}: {tuple(got.shape)} vs {tuple(want.shape)}"
+    assert torch.isfinite(got).all(), f"{what}: not finite"
+    err = (got - want).abs()
+    bound = atol + rtol * want.abs()
+    assert (err <= bound).all(), f"{what}: max |diff| {err.max():.3g} (worst excess {(err - bound).max():.3g})"
+
+
+# -------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_embed(dtype):
+    from sonicboom_amd import ops
+    table = randn(301, 72, dtype=dtype)
+    ids = torch.tensor([0, 300, 7, 7, 150], dtype=torch.int32)
+    got = ops.embed(table.to(DEV), ids.to(DEV))
+    assert got.dtype == F32 and torch.equal(got.cpu(), table.float()[ids.long()])
+    bad = ops.embed(table.to(DEV), torch.tensor([301, -1], dtype=torch.int32, device=DEV))
+    assert torch.isnan(bad).all()          # an id outside the table never reads memory it does not own
+
+
+@pytest.mark.parametrize("width", [64, 201, 338, 3584])
+@pytest.mark.parametrize("out_dtype, w_dtype", [(F32, F32), (BF16, BF16), (BF16, F32)])
+def test_rmsnorm(width, out_dtype, w_dtype):
+    from sonicboom_amd import ops
+    x = randn(7, width, scale=3.0)
+    w = (1.0 + randn(width, scale=0.1)).to(w_dtype)
+    eps = 1e-5
+    want = plain.rms_norm(x.numpy(), w.float().numpy(), eps)
+    got = ops.rmsnorm(x.to(DEV), w.to(DEV), eps, out_dtype)
+    tol = dict(atol=1e-6, rtol=2e-6) if out_dtype == F32 else dict(atol=1e-2, rtol=8e-3)
+    close(got, want, what="rmsnorm", **tol)
+    rows = torch.tensor([5, 0, 5], dtype=torch.int32)
+    picked = ops.rmsnorm(x.to(DEV), w.to(DEV), eps, out_dtype, rows.to(DEV))
+    assert torch.equal(picked.cpu(), got.cpu()[rows.long()])
+
+
+def test_rmsnorm_reference_vectors():
+    """/root/reference/tests/core/test_nn.cpp:172-219."""
+    from sonicboom_amd import ops
+    x = torch.tensor([[2.0, 2.0, 2.0, 2.0]], device=DEV)
+    assert torch.allclose(ops.rmsnorm(x, None, 0.0, F32).cpu(), torch.ones(1, 4), atol=1e-6)
+    w3 = torch.full((4,), 3.0, device=DEV)
+    assert torch.allclose(ops.rmsnorm(x, w3, 0.0, F32).cpu(), torch.full((1, 4), 3.0), atol=1e-6)
+    e = torch.tensor([[1.0, 0.0, 0.0, 0.0]], device=DEV)
+    assert torch.equal(ops.rmsnorm(e, None, 0.75, F32).cpu(), torch.tensor([[1.0, 0.0, 0.0, 0.0]]))
+
+
+def ref_gemm(x, w, bias=None, resid=None):
+    y = x.double() @ w.double().T
+    if bias is not None:
+        y = y + bias.double()
+    if resid is not None:
+        y = y + resid.double()
+    return y
+
+
+@pytest.mark.parametrize("t, n, k", [(1, 100, 96), (5, 224, 200), (64, 64, 64), (130, 97, 51), (3, 1000, 3584)])
+@pytest.mark.parametrize("xd, wd", [(F32, F32), (BF16, BF16), (BF16, F32), (F32, BF16)])
+def test_gemm_plain(t, n, k, xd, wd):
+    from sonicboom_amd import ops
+    x, w = randn(t, k, dtype=xd), randn(n, k, dtype=wd, scale=0.05)
+    bias, resid = randn(n, scale=0.1), randn(t, n)
+    want = ref_gemm(x, w, bias, resid)
+    got = ops.gemm_plain(x.to(DEV), w.to(DEV), bias.to(DEV), resid.to(DEV), F32)
+    close(got, want, atol=2e-5 * math.sqrt(k), rtol=1e-5, what="gemm_plain")
+    # in place on the residual, and without the extras
+    r = resid.to(DEV)
+    ops.gemm_plain(x.to(DEV), w.to(DEV), None, r, F32, out=r)
+    close(r, ref_gemm(x, w, None, resid), atol=2e-5 * math.sqrt(k), rtol=1e-5, what="gemm_plain in place")
+
+
+def test_gemm_plain_does_not_depend_on_the_batch():
+    """The same row gives the same bits alone and among 200 others."""
+    from sonicboom_amd import ops
+    x, w = randn(200, 333).to(DEV), randn(150, 333, scale=0.05).to(DEV)
+    whole = ops.gemm_plain(x, w, None, None, F32)
+    for r in (0, 63, 64, 199):
+        alone = ops.gemm_plain(x[r:r + 1].contiguous(), w, None, None, F32)
+        assert torch.equal(alone[0], whole[r])
+
+
+@pytest.mark.parametrize("t", [1, 5, 16, 17, 33, 64, 65, 128, 300])
+@pytest.mark.parametrize("n, k", [(96, 64), (100, 96), (224, 200), (3584, 512), (1000, 3584), (72, 18944 // 8)])
+def test_gemm_bf16_matrix_cores(t, n, k):
+    from sonicboom_amd import ops
+    x, w = randn(t, k, dtype=BF16), randn(n, k, dtype=BF16, scale=0.05)
+    bias, resid = randn(n, scale=0.1), randn(t, n)
+    want = ref_gemm(x, w, bias, resid)
+    got = ops.gemm_bf16(x.to(DEV), w.to(DEV), bias.to(DEV), resid.to(DEV), F32)
+    assert got is not None
+    close(got, want, atol=3e-5 * math.sqrt(k), rtol=1e-5, what=f"gemm_bf16 t={t}")
+    got16 = ops.gemm_bf16(x.to(DEV), w.to(DEV), None, None, BF16)
+    close(got16, ref_gemm(x, w), atol=2e-2, rtol=8e-3, what=f"gemm_bf16 bf16 out t={t}")
+    r = resid.to(DEV)
+    ops.gemm_bf16(x.to(DEV), w.to(DEV), None, r, F32, out=r)
+    close(r, ref_gemm(x, w, None, resid), atol=3e-5 * math.sqrt(k), rtol=1e-5, what="in place")
+
+
+@pytest.mark.parametrize("t", [1, 8, 40, 64, 65, 200])
+@pytest.mark.parametrize("inner, k", [(100, 96), (224, 200), (18944 // 4, 512)])
+def test_gemm_bf16_gated(t, inner, k):
+    from sonicboom_amd import ops
+    x, w = randn(t, k, dtype=BF16), randn(2 * inner, k, dtype=BF16, scale=0.1)
+    gu = x.double() @ w.double().T
+    g, u = gu[:, :inner], gu[:, inner:]
+    want = g / (1.0 + torch.exp(-g)) * u
+    got = ops.gemm_bf16(x.to(DEV), w.to(DEV), None, None, F32, gated=True)
+    close(got, want, atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"gated t={t}")
+
+
+def test_gemm_bf16_refuses_what_it_cannot_take():
+    from sonicboom_amd import ops
+    x, w = randn(4, 100, dtype=BF16).to(DEV), randn(8, 100, dtype=BF16).to(DEV)
+    assert ops.gemm_bf16(x, w, None, None, F32) is None          # inner size not a multiple of 8
+    want = ref_gemm(x.cpu(), w.cpu())
+    close(ops.gemm_plain(x, w, None, None, F32), want, atol=1e-3, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_silu_mul_add_cast(dtype):
+    from sonicboom_amd import ops
+    gu = randn(9, 2 * 77, scale=3.0)
+    gu[0, 0], gu[0, 1], gu[0, 2] = 0.0, 1.0, -100.0
+    want = plain.silu(gu[:, :77].numpy()) * gu[:, 77:].numpy()
+    got = ops.silu_mul(gu.to(DEV), dtype)
+    close(got, want, atol=1e-6 if dtype == F32 else 2e-2, rtol=1e-6 if dtype == F32 else 8e-3)
+    # silu(0) = 0, silu(1) = 0.7310586 (/root/reference/tests/core/test_nn.cpp:52-66)
+    one = ops.silu_mul(torch.tensor([[0.0, 1.0, 1.0, 1.0]], device=DEV), F32).cpu()
+    assert one[0, 0] == 0.0 and abs(one[0, 1].item() - 0.7310586) < 1e-6
+    resid = randn(5, 33)
+    y = randn(5, 33, dtype=dtype, seed=3)
+    r = resid.to(DEV)
+    ops.add_into(r, y.to(DEV))
+    assert torch.equal(r.cpu(), resid + y.float())
+    c = ops.cast(resid.to(DEV), BF16)
+    assert torch.equal(c.cpu(), resid.to(BF16))
+
+
+def make_cache(n_pages, heads_kv, head_dim, dtype, fill=float("nan")):
+    k = torch.full((n_pages, heads_kv, 64, head_dim), fill, dtype=dtype, device=DEV)
+    return k, k.clone()
+
+
+@pytest.mark.parametrize("hq, hkv, hd, rot", [(4, 2, 16, 0), (3, 1, 32, 0), (5, 5, 48, 0), (2, 1, 64, 32), (8, 2, 128, 0)])
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_rope_kv_store(hq, hkv, hd, rot, dtype):
+    """Rotation against the plain rope; keys and values land where the page table says."""
+    from sonicboom_amd import ops
+    base = 10000.0
+    n = 11
+    qkv = randn(n, (hq + 2 * hkv) * hd)
+    pos = torch.tensor([0, 1, 2, 63, 64, 65, 130, 7, 200, 1000, 5], dtype=torch.int32)
+    seq = torch.tensor([0, 0, 0, 0, 0, 0, 0, 1, 1, 1, 1], dtype=torch.int32)   # row -> sequence
+    pos[7:] = torch.tensor([3, 64, 127, 128])
+    # scattered physical pages, different per sequence
+    table = torch.tensor([[5, 2, 7], [1, 6, 3]], dtype=torch.int32)
+    kc, vc = make_cache(8, hkv, hd, dtype)
+    dims = rot or hd
+    ff = (1.0 + torch.arange(dims // 2, dtype=F32) / 7.0) if rot else None
+    log_base = np.log(np.float32(base)).astype(np.float32)
+    inv = np.exp((np.float32(-2.0) * np.arange(dims // 2, dtype=np.float32) / np.float32(dims)).astype(np.float32)
+                 * log_base).astype(np.float32)
+    q = ops.rope_kv_store(qkv.to(DEV), dtype, torch.from_numpy(inv).to(DEV), None if ff is None else ff.to(DEV),
+                          dims, pos.to(DEV), seq.to(DEV), kc, vc, table.to(DEV), hq, hkv, hd)
+    qw, kvw = hq * hd, hkv * hd
+    ffn = None if ff is None else ff.numpy()
+    want_q = plain.rope_neox(qkv[:, :qw].numpy(), pos.numpy(), hd, base, rot, ffn)
+    want_k = plain.rope_neox(qkv[:, qw:qw + kvw].numpy(), pos.numpy(), hd, base, rot, ffn)
+    tol = dict(atol=2e-6, rtol=1e-5) if dtype == F32 else dict(atol=2e-2, rtol=8e-3)
+    close(q, want_q, what="q", **tol)
+    for r in range(n):
+        page = table[seq[r], pos[r] // 64]
+        got_k = kc[page, :, pos[r] % 64, :].reshape(-1)
+        got_v = vc[page, :, pos[r] % 64, :].reshape(-1)
+        close(got_k, want_k[r], what=f"k row {r}", **tol)
+        close(got_v, qkv[r, qw + kvw:].to(dtype).float(), atol=0, rtol=0, what=f"v row {r}")
+    # nothing else was written
+    assert torch.isnan(kc.float()).sum().item() == kc.numel() - n * kvw
+
+
+def test_rope_reference_vectors():
+    """/root/reference/tests/core/test_nn.cpp:221-290: position 0 is the identity; with
+    head size 2 and an angle of pi/2, [1,0] turns into [0,1]; pairs are (i, i+half)."""
+    from sonicboom_amd import ops
+    kc, vc = make_cache(1, 1, 4, F32)
+    table = torch.zeros((1, 1), dtype=torch.int32, device=DEV)
+    z = torch.zeros(1, dtype=torch.int32, device=DEV)
+    x = torch.tensor([[0.5, -1.25, 2.0, 3.5] * 3], device=DEV)
+    inv = torch.tensor([1.0, 0.01], device=DEV)
+    q = ops.rope_kv_store(x, F32, inv, None, 4, z, z, kc, vc, table, 1, 1, 4)
+    assert torch.equal(q.cpu(), x[:, :4].cpu())
+    # angle pi/2 for both pairs at position 1: (x0, x2) -> (-x2, x0), (x1, x3) -> (-x3, x1)
+    inv = torch.full((2,), math.pi / 2, device=DEV)
+    one = torch.ones(1, dtype=torch.int32, device=DEV)
+    x = torch.tensor([[1.0, 0.0, 2.0, 3.0] * 3], device=DEV)
+    q = ops.rope_kv_store(x, F32, inv, None, 4, one, z, kc, vc, table, 1, 1, 4).cpu()
+    assert torch.allclose(q, torch.tensor([[-2.0, -3.0, 1.0, 0.0]]), atol=1e-6)
+    # freq_factors: a huge divisor freezes its pair (test_nn.cpp:272-289)
+    ff = torch.tensor([1.0, 1e30], device=DEV)
+    q = ops.rope_kv_store(x, F32, inv, ff, 4, one, z, kc, vc, table, 1, 1, 4).cpu()
+    assert torch.allclose(q, torch.tensor([[-2.0, 0.0, 1.0, 3.0]]), atol=1e-5)
+
+
+def fill_cache_from(keys, values, table, dtype):
+    """keys/values: list per sequence of [len, hkv, hd] float tensors -> paged caches."""
+    hkv, hd = keys[0].shape[1:]
+    n_pages = int(table.max()) + 1
+    kc, vc = make_cache(n_pages, hkv, hd, dtype)
+    for s, (k, v) in enumerate(zip(keys, values)):
+        for p in range(k.shape[0]):
+            page = table[s, p // 64]
+            kc[page, :, p % 64, :] = k[p].to(dtype)
+            vc[page, :, p % 64, :] = v[p].to(dtype)
+    return kc, vc
+
+
+ATTN_SHAPES = [(4, 2, 16), (3, 1, 32), (5, 5, 48), (6, 2, 80), (8, 2, 128), (2, 1, 256)]
+
+
+@pytest.mark.parametrize("hq, hkv, hd", ATTN_SHAPES)
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("window", [0, 70])
+def test_attention_plain_kernel(hq, hkv, hd, dtype, window):
+    from sonicboom_amd import ops
+    lens = [150, 3]
+    table = torch.tensor([[4, 0, 2], [1, 3, 5]], dtype=torch.int32)
+    keys = [randn(n, hkv, hd, seed=s).to(dtype).float() for s, n in enumerate(lens)]
+    vals = [randn(n, hkv, hd, seed=9 + s).to(dtype).float() for s, n in enumerate(lens)]
+    kc, vc = fill_cache_from(keys, vals, table, dtype)
+    # rows: a few positions of sequence 0 (first, page edges, last), all of sequence 1
+    rows = [(0, 0), (0, 63), (0, 64), (0, 100), (0, 149), (1, 0), (1, 1), (1, 2)]
+    q = randn(len(rows), hq * hd, seed=5).to(dtype)
+    scale = 1.0 / math.sqrt(hd)
+    pos = torch.tensor([p for _, p in rows], dtype=torch.int32)
+    seq = torch.tensor([s for s, _ in rows], dtype=torch.int32)
+    got = ops.attention_plain(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), seq.to(DEV), hq, hkv, hd, scale, window)
+    for r, (s, p) in enumerate(rows):
+        n = lens[s]
+        want = plain.attention(q[r:r + 1].float().numpy(), keys[s].reshape(n, -1).numpy(),
+                               vals[s].reshape(n, -1).numpy(), [p], np.arange(n), hq, hkv, hd, scale,
+                               causal=True, window=window)
+        tol = dict(atol=3e-6, rtol=2e-5) if dtype == F32 else dict(atol=2e-2, rtol=1e-2)
+        close(got[r:r + 1], want, what=f"row {r} (seq {s}, pos {p})", **tol)
+
+
+def test_attention_reference_vectors():
+    """/root/reference/tests/core/test_nn.cpp:402-495: one key copies its value; causal
+    2x2 gives [2, 3]; GQA maps 4 query heads onto 2 kv heads; window 2 drops key 0;
+    scale 1 and 0.5 give 1.0360 and 1.2384."""
+    from sonicboom_amd import ops
+
+    def run(q, k, v, hq, hkv, hd, scale, window=0):
+        n = len(k)
+        keys = [torch.tensor(k, dtype=F32).reshape(n, hkv, hd)]
+        vals = [torch.tensor(v, dtype=F32).reshape(n, hkv, hd)]
+        table = torch.zeros((1, 1), dtype=torch.int32)
+        # pad the head to the kernels' smallest size by zero columns: scores are unchanged
+        kc, vc = fill_cache_from(keys, vals, table, F32)
+        qt = torch.tensor(q, dtype=F32).reshape(-1, hq * hd)
+        pos = torch.arange(qt.shape[0], dtype=torch.int32)
+        seq = torch.zeros(qt.shape[0], dtype=torch.int32)
+        return ops.attention_plain(qt.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), seq.to(DEV), hq, hkv, hd,
+                                   scale, window).cpu()
+
+    assert torch.allclose(run([[1.0, 0, 0, 0]], [[1.0, 0, 0, 0]], [[1.0, 2, 3, 4]], 1, 1, 4, 1.0),
+                          torch.tensor([[1.0, 2, 3, 4]]), atol=1e-6)
+    out = run([[1.0], [1.0]], [[1.0], [1.0]], [[2.0], [4.0]], 1, 1, 1, 1.0)
+    assert torch.allclose(out.flatten(), torch.tensor([2.0, 3.0]), atol=1e-6)
+    out = run([[1.0, 1, 1, 1]], [[1.0, 1.0]], [[1.0, 2.0]], 4, 2, 1, 1.0)
+    assert torch.allclose(out.flatten(), torch.tensor([1.0, 1.0, 2.0, 2.0]), atol=1e-6)
+    out = run([[1.0], [1.0], [1.0]], [[1.0], [1.0], [1.0]], [[1.0], [2.0], [4.0]], 1, 1, 1, 1.0, window=2)
+    assert abs(out[2, 0].item() - 3.0) < 1e-6
+    # q = 2 at the position of the second key; keys [2, 0], values [1, 3]
+    for scale, want in ((1.0, 1.0360), (0.5, 1.2384)):
+        out = run([[0.0], [2.0]], [[2.0], [0.0]], [[1.0], [3.0]], 1, 1, 1, scale)
+        assert abs(out[1, 0].item() - want) < 1e-3
+
+
+def test_a_far_key_among_hundreds_is_found():
+    """One key far back is made to dominate: the output must be its value, whatever page it is on."""
+    from sonicboom_amd import ops
+    hq, hkv, hd, n = 4, 2, 32, 700
+    keys = [randn(n, hkv, hd, scale=0.1)]
+    vals = [randn(n, hkv, hd, seed=2)]
+    q = randn(1, hq * hd, seed=4)
+    table = torch.tensor([list(reversed(range(11)))], dtype=torch.int32)
+    for far in (0, 63, 64, 389, 699):
+        k = [keys[0].clone()]
+        for h in range(hq):
+            k[0][far, h // 2] = q[0, h * hd:(h + 1) * hd] * 40.0 if h % 2 == 0 else k[0][far, h // 2]
+        kc, vc = fill_cache_from(k, vals, table, F32)
+        out = ops.attention_plain(q.to(DEV), kc, vc, table.to(DEV), torch.tensor([n - 1], dtype=torch.int32, device=DEV),
+                                  torch.zeros(1, dtype=torch.int32, device=DEV), hq, hkv, hd, 1.0, 0).cpu()
+        for h in (0, 2):
+            assert torch.allclose(out[0, h * hd:(h + 1) * hd], vals[0][far, h // 2], atol=1e-4), (far, h)
+
+
+@pytest.mark.parametrize("vocab", [5, 256, 1000, 152064])
+def test_argmax_first_maximum(vocab):
+    from sonicboom_amd import ops
+    x = randn(6, vocab)
+    x[0, :] = 0.5                                   # all equal: id 0
+    x[1, vocab - 1] = 50.0
+    x[2, 3] = 60.0
+    if vocab > 4:
+        x[2, 4] = 60.0                              # a tie: the lower id
+    x[3, :] = float("-inf")
+    got = ops.argmax(x.to(DEV)).cpu().tolist()
+    want = [plain.argmax(r.numpy()) for r in x]
+    assert got == want and got[:3] == [0, vocab - 1, 3]
+
+
+@pytest.mark.parametrize("vocab", [7, 256, 300, 5000, 152064])
+@pytest.mark.parametrize("temperature", [1.0, 0.7])
+def test_top_candidates(vocab, temperature):
+    from sonicboom_amd import ops
+    x = randn(4, vocab, scale=2.0)
+    x[1] = torch.round(x[1])                        # many ties: ordered by id
+    x[2, :] = 1.25                                  # all equal
+    x[3, ::3] = -0.0
+    x[3, 1::3] = 0.0                                # signed zeros are one value
+    k = min(256, vocab)
+    ids, z = ops.top_candidates(x.to(DEV), temperature, k)
+    ids, z = ids.cpu().numpy(), z.cpu().numpy()
+    for r in range(4):
+        want = sampling_plain.select_candidates(x[r].numpy(), temperature)
+        assert [c[0] for c in want] == ids[r].tolist(), f"row {r}"
+        assert np.array_equal(np.array([c[1] for c in want], dtype=np.float32), z[r]), f"row {r}"
+
+
+@pytest.mark.parametrize("exact", [False, True])
+def test_penalize(exact):
+    from sonicboom_amd import ops
+    logits = randn(3, 50)
+    hist = [[1, 2, 2, 49], [], [7] * 10]
+    rows, toks, counts = [0, 0, 0, 2], [1, 2, 49, 7], [1, 2, 1, 10]
+    dev = logits.to(DEV)
+    ops.penalize(dev, *(torch.tensor(v, dtype=torch.int32, device=DEV) for v in (rows, toks, counts)),
+                 1.3, 0.2, 0.1, exact)
+    for r in range(3):
+        want = sampling_plain.penalize(logits[r].numpy(), exact, 1.3, 64, 0.2, 0.1, hist[r])
+        assert np.array_equal(dev[r].cpu().numpy(), want), f"row {r}"
