@@ -6,7 +6,8 @@ per-sequence state of fixed size.
   :meth:`PagedCache.alloc_slot`, given back by :meth:`free_slot` and used again.
 * Cache entries (one per mixer that stores keys) with the same needs
   (kv heads, head size, window) form a **group** with storage and a page pool
-  of its own: ``K, V: [entries, pages, kv_heads, PAGE, head_dim]``.  A group
+  of its own: ``K: [entries, pages, kv_heads, PAGE, head_dim]`` and ``V`` with
+  the last two axes swapped.  A group
   that only reads a window of keys gives pages back as the window leaves them.
 * ``max_tokens`` sizes every pool: the most tokens live sequences hold at any
   time, each sequence's count rounded up to a whole page (PAGE = 64 tokens).
@@ -103,9 +104,12 @@ class PagedCache:
         if allocate:
             import torch
             for spec in self.groups:
-                shape = (len(spec.entries), self.n_pages, spec.kv_heads, PAGE, spec.head_dim)
-                self.k.append(torch.empty(shape, dtype=dtype, device=device))
-                self.v.append(torch.empty(shape, dtype=dtype, device=device))
+                # keys [.., position, d]; values transposed [.., d, position] (see csrc/sb_hip.h)
+                n = len(spec.entries)
+                self.k.append(torch.zeros((n, self.n_pages, spec.kv_heads, PAGE, spec.head_dim),
+                                          dtype=dtype, device=device))
+                self.v.append(torch.zeros((n, self.n_pages, spec.kv_heads, spec.head_dim, PAGE),
+                                          dtype=dtype, device=device))
             for key, (shape, sdtype) in (state_shapes or {}).items():
                 self.state[key] = torch.zeros((self.max_slots, *shape), dtype=sdtype, device=device)
 
@@ -199,7 +203,8 @@ class PagedCache:
 
     # ---- storage -------------------------------------------------------------
     def entry_views(self, entry: int):
-        """(keys, values) of one cache entry, each [pages, kv_heads, PAGE, head_dim], and its group."""
+        """(keys [pages, kv_heads, PAGE, head_dim], values [pages, kv_heads, head_dim, PAGE]) of one
+        cache entry, and its group."""
         g, i = self.entry_place[entry]
         return self.k[g][i], self.v[g][i], g
 

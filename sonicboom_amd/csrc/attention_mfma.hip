@@ -1,0 +1,396 @@
+// bf16 attention over the paged cache on the matrix cores, for one head size
+// (compiled with -DSB_HEAD_DIM=N, N a multiple of 16 up to 256): a prefill
+// kernel (many rows per sequence, causal) and a decode kernel (one row per
+// sequence, keys split over blocks, the query heads of a kv head sharing its
+// keys and values).
+//
+// Formula: /root/reference/core/src/nn/attention.cpp:26-105, :121-181 — query
+// head h reads kv head h / group, s = dot(q, k) * scale, key j visible from
+// position p when j <= p and (window == 0 or p - j < window), softmax with the
+// maximum subtracted, in float32; probabilities are rounded to bf16 only as
+// the operand of the P V product, which accumulates in float32.
+//
+// One wave owns 16 query columns (16 positions of one head in prefill, the
+// heads of one kv head in decode) and walks its keys 32 at a time:
+//   S^T[key][col] = K[key][:] . Q[col][:]     v_mfma_f32_16x16x32_bf16, A = K rows, B = Q rows
+//   O^T[d][col]  += V^T[d][key] * P[key][col]  same instruction, A = V^T rows, B = P
+// Row r = 4g + i of score tile t is fed key 8g + 4t + i of the 32, so that lane
+// group g ends up holding the scores of keys 8g .. 8g+7 in order: exactly the
+// eight k-slots of its B operand for the second product.  P therefore never
+// leaves the registers; K fragments come straight from the cache ([key][d],
+// 16 bytes per lane) and so do V fragments, because the cache keeps values
+// transposed ([d][key]).  No LDS is used in the main loops.
+//
+// Order of summation: keys are visited in ascending order, 32 at a time, within
+// a wave; decode merges waves (pages) and then blocks (chunks of 4 pages) in
+// ascending order.  It depends on positions only, not on the batch.
+#include "mfma.cuh"
+
+#ifndef SB_HEAD_DIM
+#error "compile with -DSB_HEAD_DIM=<head size>"
+#endif
+
+namespace sb {
+char *error_slot() {
+  static thread_local char slot[kErrorLen] = {0};
+  return slot;
+}
+}  // namespace sb
+
+extern "C" const char *sb_attn_last_error(void) { return sb::error_slot(); }
+extern "C" int sb_attn_head_dim(void) { return SB_HEAD_DIM; }
+
+namespace {
+
+constexpr int HD = SB_HEAD_DIM;
+static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head size must be a multiple of 16 up to 256");
+constexpr int KS = (HD + 31) / 32;   // k-steps of the score product
+constexpr int DT = HD / 16;          // 16-row tiles of O^T
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kPagesPerChunk = 4;
+
+struct WaveState {
+  floatx4_t o[DT];   // O^T[d = 16 dt + 4 g + i][col]
+  float m;           // running maximum of the column (log2 domain), same in the four lane groups
+  float l;           // this lane's share of the running sum
+};
+
+__device__ __forceinline__ void init_state(WaveState &st) {
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) st.o[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+  st.m = -__builtin_inff();
+  st.l = 0.f;
+}
+
+// Zero the elements of a fragment of 8 consecutive keys from index n_keep on.
+__device__ __forceinline__ uint4 keep_first(uint4 v, int n_keep) {
+  uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int have = n_keep - 2 * i;   // elements of this word that stay
+    w[i] = have >= 2 ? w[i] : (have == 1 ? (w[i] & 0xffffu) : 0u);
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+// Zero the elements before index n_drop.
+__device__ __forceinline__ uint4 drop_first(uint4 v, int n_drop) {
+  uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int gone = n_drop - 2 * i;
+    w[i] = gone >= 2 ? 0u : (gone == 1 ? (w[i] & 0xffff0000u) : w[i]);
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// One page (64 keys at absolute positions page_pos .. page_pos+63) for the wave's 16 columns.
+// qf: the columns' query fragments; col_pos / col_lo: last and first visible key of this lane's
+// column (col_pos < 0: the column is empty).  key_hi / key_lo: the same over all columns of the
+// wave (uniform), used to skip work and to decide whether values need masking.
+__device__ __forceinline__ void attend_page(WaveState &st, const bf16x8_t (&qf)[KS],
+                                            const bf16_t *__restrict__ kp, const bf16_t *__restrict__ vp,
+                                            int page_pos, int col_pos, int col_lo, int key_lo, int key_hi,
+                                            float scale_log2, int lane) {
+  const int r = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int half = 0; half < 2; ++half) {
+    const int base = page_pos + 32 * half;
+    if (base > key_hi || base + 31 < key_lo) continue;   // uniform: nothing visible in these 32 keys
+    floatx4_t s[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      s[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+      // A row r = 4 gg + i is key 8 gg + 4 t + i of the 32
+      const int key = 32 * half + 8 * (r >> 2) + 4 * t + (r & 3);
+      const bf16_t *krow = kp + size_t(key) * HD;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d = ks * 32 + g * 8;
+        const uint4 a = ld16(krow + d, d < HD);
+        s[t] = mfma16(as_bf16x8(a), qf[ks], s[t]);
+      }
+    }
+    // this lane: column r, keys base + 8 g + e, e = 0..7 (s[0] holds e = 0..3, s[1] e = 4..7)
+    float sc[8];
+    float mx = -__builtin_inff();
+    const int k0 = base + 8 * g;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int j = k0 + e;
+      const bool vis = j <= col_pos && j >= col_lo;
+      const float v = (e < 4 ? s[0][e] : s[1][e - 4]) * scale_log2;
+      sc[e] = vis ? v : -__builtin_inff();
+      mx = fmaxf(mx, sc[e]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(st.m, mx);
+    // a column that has seen no key yet keeps m = -inf: give it a finite stand-in
+    const float m_use = m_new == -__builtin_inff() ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(st.m - m_use);   // st.m = -inf gives 0
+    float p[8];
+    float psum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      p[e] = __builtin_amdgcn_exp2f(sc[e] - m_use);             // -inf gives 0
+      psum += p[e];
+    }
+    st.l = st.l * alpha + psum;
+    st.m = m_new;
+    const uint4 pb = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]),
+                                pack_bf16(p[6], p[7]));
+    // values of keys outside [key_lo, key_hi] may be stale or never written: 0 * garbage must not
+    // reach the accumulator, so such keys are cut out of the V fragment as well
+    const bool cut_hi = base + 31 > key_hi, cut_lo = base < key_lo;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      uint4 a = ld16(vp + size_t(dt * 16 + r) * SB_PAGE + 32 * half + 8 * g, true);
+      if (cut_hi) a = keep_first(a, key_hi - k0 + 1);
+      if (cut_lo) a = drop_first(a, key_lo - k0);
+      floatx4_t acc = st.o[dt];
+      acc[0] *= alpha; acc[1] *= alpha; acc[2] *= alpha; acc[3] *= alpha;
+      st.o[dt] = mfma16(as_bf16x8(a), as_bf16x8(pb), acc);
+    }
+  }
+}
+
+__device__ __forceinline__ void load_q(bf16x8_t (&qf)[KS], const bf16_t *qrow, bool col_ok, int lane) {
+  const int g = lane >> 4;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d = ks * 32 + g * 8;
+    qf[ks] = as_bf16x8(ld16(qrow + d, col_ok && d < HD));
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Prefill: a wave takes a tile of up to 16 consecutive rows of one sequence and one query head.
+// tiles: int32 [n_tiles][4] = (first row, rows, sequence, unused).
+__global__ void __launch_bounds__(256)
+attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
+                    const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
+                    const int32_t *__restrict__ page_table, int max_pages, int n_pages_total,
+                    const int32_t *__restrict__ row_pos, const int32_t *__restrict__ tiles, int n_tiles,
+                    int heads_q, int heads_kv, float scale_log2, int window) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  // heavy tiles (late rows, long key ranges) first
+  const int tile = n_tiles - 1 - (blockIdx.x * 4 + wave);
+  if (tile < 0) return;
+  const int head = blockIdx.y;
+  const int kvh = head / (heads_q / heads_kv);
+  const int row0 = tiles[tile * 4 + 0], n_rows = tiles[tile * 4 + 1], seq = tiles[tile * 4 + 2];
+  const int r = lane & 15, g = lane >> 4;
+  const bool col_ok = r < n_rows;
+  const int row = row0 + (col_ok ? r : 0);
+  const int pos = row_pos[row];
+  const int col_pos = col_ok ? pos : -1;
+  const int col_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
+  // rows of a tile are consecutive positions: the first row has the lowest window start,
+  // the last valid row the highest position
+  const int pos_first = row_pos[row0], pos_last = row_pos[row0 + n_rows - 1];
+  const int key_lo = (window > 0 && pos_first >= window) ? pos_first - window + 1 : 0;
+  const int key_hi = pos_last;
+
+  bf16x8_t qf[KS];
+  load_q(qf, q + (size_t(row) * heads_q + head) * HD, col_ok, lane);
+  WaveState st;
+  init_state(st);
+  const int32_t *pt = page_table + size_t(seq) * max_pages;
+  for (int pg = key_lo / SB_PAGE; pg <= key_hi / SB_PAGE; ++pg) {
+    const int page = pg < max_pages ? pt[pg] : -1;
+    if (page < 0 || page >= n_pages_total) continue;
+    const size_t off = (size_t(page) * heads_kv + kvh) * SB_PAGE * HD;
+    attend_page(st, qf, k_cache + off, v_cache + off, pg * SB_PAGE, col_pos, col_lo, key_lo, key_hi,
+                scale_log2, lane);
+  }
+  float l = st.l;
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!col_ok) return;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  bf16_t *orow = out + (size_t(row) * heads_q + head) * HD;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    const uint2 v = make_uint2(pack_bf16(st.o[dt][0] * inv, st.o[dt][1] * inv),
+                               pack_bf16(st.o[dt][2] * inv, st.o[dt][3] * inv));
+    *reinterpret_cast<uint2 *>(orow + dt * 16 + 4 * g) = v;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Decode: one row per sequence.  Block (chunk, kv head x head tile, sequence); wave w of the
+// block takes page 4 * chunk + w; columns are the query heads of the kv head.
+// part_o: float [seqs][heads_q][n_chunks][HD], part_ml: float [seqs][heads_q][n_chunks][2].
+__global__ void __launch_bounds__(256)
+attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
+                   const bf16_t *__restrict__ q, const bf16_t *__restrict__ k_cache,
+                   const bf16_t *__restrict__ v_cache, const int32_t *__restrict__ page_table,
+                   int max_pages, int n_pages_total, const int32_t *__restrict__ row_pos, int heads_q,
+                   int heads_kv, int n_chunks, float scale_log2, int window) {
+  __shared__ float lds_o[4][HD * 16];   // [wave][d][col]
+  __shared__ float lds_m[4][16], lds_l[4][16];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int chunk = blockIdx.x, seq = blockIdx.z;
+  const int group = heads_q / heads_kv;
+  const int head_tiles = (group + 15) / 16;
+  const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y - kvh * head_tiles;
+  const int pos = row_pos[seq];
+  const int key_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
+  const int first_chunk = key_lo / (SB_PAGE * kPagesPerChunk), last_chunk = pos / (SB_PAGE * kPagesPerChunk);
+  if (chunk < first_chunk || chunk > last_chunk) return;   // uniform over the block
+
+  const int r = lane & 15, g = lane >> 4;
+  const int hq = ht * 16 + r;                 // query head within the group
+  const bool col_ok = hq < group;
+  const int head = kvh * group + (col_ok ? hq : 0);
+  bf16x8_t qf[KS];
+  load_q(qf, q + (size_t(seq) * heads_q + head) * HD, col_ok, lane);
+  WaveState st;
+  init_state(st);
+  const int pg = chunk * kPagesPerChunk + wave;
+  if (pg >= key_lo / SB_PAGE && pg <= pos / SB_PAGE && pg < max_pages) {
+    const int page = page_table[size_t(seq) * max_pages + pg];
+    if (page >= 0 && page < n_pages_total) {
+      const size_t off = (size_t(page) * heads_kv + kvh) * SB_PAGE * HD;
+      attend_page(st, qf, k_cache + off, v_cache + off, pg * SB_PAGE, col_ok ? pos : -1, key_lo, key_lo, pos,
+                  scale_log2, lane);
+    }
+  }
+  float l = st.l;
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) lds_o[wave][(dt * 16 + 4 * g + i) * 16 + r] = st.o[dt][i];
+  if (g == 0) {
+    lds_m[wave][r] = st.m;
+    lds_l[wave][r] = l;
+  }
+  __syncthreads();
+  // merge the four waves (pages in ascending order); thread e owns (d, col)
+  for (int e = threadIdx.x; e < HD * 16; e += 256) {
+    const int c = e & 15, d = e >> 4;
+    const int hh = ht * 16 + c;
+    if (hh >= group) continue;
+    float m = -__builtin_inff();
+#pragma unroll
+    for (int w = 0; w < 4; ++w) m = fmaxf(m, lds_m[w][c]);
+    const float m_use = m == -__builtin_inff() ? 0.f : m;
+    float o = 0.f, lsum = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = __builtin_amdgcn_exp2f(lds_m[w][c] - m_use);
+      o += lds_o[w][e] * f;
+      lsum += lds_l[w][c] * f;
+    }
+    const int oh = kvh * group + hh;
+    if (n_chunks == 1) {
+      out[(size_t(seq) * heads_q + oh) * HD + d] = f32_to_bf16(lsum > 0.f ? o / lsum : 0.f);
+    } else {
+      const size_t pi = (size_t(seq) * heads_q + oh) * n_chunks + chunk;
+      part_o[pi * HD + d] = o;
+      if (d == 0) {
+        part_ml[pi * 2 + 0] = m;
+        part_ml[pi * 2 + 1] = lsum;
+      }
+    }
+  }
+}
+
+// Merge the chunks of a (sequence, head) in ascending order.
+__global__ void attn_decode_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o,
+                                         const float *__restrict__ part_ml,
+                                         const int32_t *__restrict__ row_pos, int heads_q, int n_chunks,
+                                         int window) {
+  const int seq = blockIdx.y, head = blockIdx.x;
+  const int pos = row_pos[seq];
+  const int key_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
+  const int first = key_lo / (SB_PAGE * kPagesPerChunk), last = min(pos / (SB_PAGE * kPagesPerChunk), n_chunks - 1);
+  const size_t base = (size_t(seq) * heads_q + head) * n_chunks;
+  float m = -__builtin_inff();
+  for (int c = first; c <= last; ++c) m = fmaxf(m, part_ml[(base + c) * 2]);
+  const float m_use = m == -__builtin_inff() ? 0.f : m;
+  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
+    float o = 0.f, l = 0.f;
+    for (int c = first; c <= last; ++c) {
+      const float f = __builtin_amdgcn_exp2f(part_ml[(base + c) * 2] - m_use);
+      o += part_o[(base + c) * HD + d] * f;
+      l += part_ml[(base + c) * 2 + 1] * f;
+    }
+    out[(size_t(seq) * heads_q + head) * HD + d] = f32_to_bf16(l > 0.f ? o / l : 0.f);
+  }
+}
+
+int check_common(const void *out, const void *q, const void *k, const void *v, const void *pt,
+                 const void *row_pos, int max_pages, int n_pages_total, int heads_q, int heads_kv,
+                 int window, const char *who) {
+  SB_REQUIRE(out && q && k && v && pt && row_pos, "%s: null pointer", who);
+  SB_REQUIRE(max_pages > 0 && n_pages_total > 0 && heads_q > 0 && heads_kv > 0 && window >= 0,
+             "%s: bad sizes", who);
+  SB_REQUIRE(heads_q % heads_kv == 0, "%s: %d query heads are not a multiple of %d kv heads", who, heads_q,
+             heads_kv);
+  SB_SUPPORT(heads_q <= 65535, "%s: more than 65535 query heads", who);
+  SB_SUPPORT(((reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k) |
+               reinterpret_cast<uintptr_t>(v) | reinterpret_cast<uintptr_t>(out)) % 16) == 0,
+             "%s: operands must be 16-byte aligned", who);
+  return SB_OK;
+}
+
+}  // namespace
+
+// Chunks the decode kernel splits `max_pages` pages into (the third size of its partial buffers).
+extern "C" int sb_attn_decode_chunks(int max_pages) {
+  return (max_pages + kPagesPerChunk - 1) / kPagesPerChunk;
+}
+
+// q, out: bf16 [n_seqs, heads_q * HD], one row per sequence; k_cache bf16 [pages][heads_kv][64][HD],
+// v_cache bf16 [pages][heads_kv][HD][64].  part_o float [n_seqs * heads_q * chunks * HD] and part_ml
+// float [n_seqs * heads_q * chunks * 2] with chunks = sb_attn_decode_chunks(max_pages) (unused, may be
+// NULL, when chunks == 1).
+extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
+                                   const int32_t *page_table, int max_pages, int n_pages_total,
+                                   const int32_t *row_pos, float *part_o, float *part_ml, int n_seqs,
+                                   int heads_q, int heads_kv, float scale, int window, void *stream) {
+  int rc = check_common(out, q, k_cache, v_cache, page_table, row_pos, max_pages, n_pages_total, heads_q,
+                        heads_kv, window, "sb_attn_decode_bf16");
+  if (rc != SB_OK) return rc;
+  SB_REQUIRE(n_seqs >= 0, "sb_attn_decode_bf16: bad batch");
+  SB_SUPPORT(n_seqs <= 65535, "sb_attn_decode_bf16: more than 65535 sequences in a step");
+  if (n_seqs == 0) return SB_OK;
+  const int n_chunks = sb_attn_decode_chunks(max_pages);
+  SB_REQUIRE(n_chunks == 1 || (part_o && part_ml), "sb_attn_decode_bf16: no buffers for the partial results");
+  const int group = heads_q / heads_kv;
+  const int head_tiles = (group + 15) / 16;
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid(n_chunks, heads_kv * head_tiles, n_seqs);
+  SB_SUPPORT(heads_kv * head_tiles <= 65535, "sb_attn_decode_bf16: too many heads");
+  attn_decode_kernel<<<grid, 256, 0, s>>>((bf16_t *)out, part_o, part_ml, (const bf16_t *)q,
+                                          (const bf16_t *)k_cache, (const bf16_t *)v_cache, page_table,
+                                          max_pages, n_pages_total, row_pos, heads_q, heads_kv, n_chunks,
+                                          scale * kLog2e, window);
+  rc = sb::check_launch("sb_attn_decode_bf16");
+  if (rc != SB_OK || n_chunks == 1) return rc;
+  attn_decode_merge_kernel<<<dim3(heads_q, n_seqs), HD < 64 ? 64 : HD, 0, s>>>(
+      (bf16_t *)out, part_o, part_ml, row_pos, heads_q, n_chunks, window);
+  return sb::check_launch("sb_attn_decode_bf16 (merge)");
+}
+
+// q, out: bf16 [n_rows, heads_q * HD]; tiles int32 [n_tiles][4] = (first row, rows <= 16, sequence, 0),
+// every tile inside one sequence and its rows at consecutive positions.
+extern "C" int sb_attn_prefill_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
+                                    const int32_t *page_table, int max_pages, int n_pages_total,
+                                    const int32_t *row_pos, const int32_t *tiles, int n_tiles, int heads_q,
+                                    int heads_kv, float scale, int window, void *stream) {
+  int rc = check_common(out, q, k_cache, v_cache, page_table, row_pos, max_pages, n_pages_total, heads_q,
+                        heads_kv, window, "sb_attn_prefill_bf16");
+  if (rc != SB_OK) return rc;
+  SB_REQUIRE(tiles && n_tiles >= 0, "sb_attn_prefill_bf16: no tiles");
+  if (n_tiles == 0) return SB_OK;
+  hipStream_t s = (hipStream_t)stream;
+  dim3 grid((n_tiles + 3) / 4, heads_q);
+  attn_prefill_kernel<<<grid, 256, 0, s>>>((bf16_t *)out, (const bf16_t *)q, (const bf16_t *)k_cache,
+                                           (const bf16_t *)v_cache, page_table, max_pages, n_pages_total,
+                                           row_pos, tiles, n_tiles, heads_q, heads_kv, scale * kLog2e, window);
+  return sb::check_launch("sb_attn_prefill_bf16");
+}

@@ -7,6 +7,9 @@
 // visible when j <= p and (window == 0 or p - j < window); softmax with the
 // maximum subtracted; a row without visible keys is zero.
 //
+// The cache holds keys as [page][kv head][position][d] and values transposed,
+// [page][kv head][d][position].
+//
 // Keys are taken 64 at a time in chunks at absolute positions [64c, 64c+64),
 // lane l owning key 64c+l.  The running maximum, the running sum and the
 // output accumulate chunk after chunk in ascending c, and inside a chunk in
@@ -67,7 +70,7 @@ attention_plain_kernel(TA *__restrict__ out, const TA *__restrict__ q, int q_str
       const int d = lane + 64 * i;
       if (d < head_dim) {
         float acc = o[i] * alpha;
-        for (int jj = j0; jj <= j1; ++jj) acc = fmaf(ps[jj], ld_f(vp, size_t(jj) * head_dim + d), acc);
+        for (int jj = j0; jj <= j1; ++jj) acc = fmaf(ps[jj], ld_f(vp, size_t(d) * SB_PAGE + jj), acc);
         o[i] = acc;
       }
     }

@@ -43,8 +43,8 @@ CORE_SOURCES = [
 HEADERS = ["common.cuh", "sb_hip.h", "mfma.cuh"]
 ATTN_SOURCES = ["attention_mfma.hip"]
 
-# Head sizes compiled ahead of time by build_all(): what tests, smoke and bench use.
-PREBUILT_HEAD_DIMS = (16, 32, 48, 64, 80, 96, 128)
+# Head sizes compiled ahead of time by build_all(): every size the kernels take.
+PREBUILT_HEAD_DIMS = tuple(range(16, 257, 16))
 MAX_HEAD_DIM = 256
 
 
@@ -63,19 +63,24 @@ def hipcc() -> str:
     raise BuildError("hipcc not found (looked at $HIPCC, PATH and /opt/rocm/bin/hipcc)")
 
 
+_BUILD_DIR = None
+
+
 def build_dir() -> str:
-    d = os.path.join(HERE, "_build")
-    try:
-        os.makedirs(d, exist_ok=True)
-        probe = os.path.join(d, f".w{os.getpid()}")
-        with open(probe, "w"):
-            pass
-        os.remove(probe)
-        return d
-    except OSError:
-        d = os.path.join(tempfile.gettempdir(), f"sonicboom_amd_build_{os.getuid()}")
-        os.makedirs(d, exist_ok=True)
-        return d
+    """``_build/`` beside the sources, or a per-user folder when that cannot be written."""
+    global _BUILD_DIR
+    if _BUILD_DIR is None:
+        d = os.path.join(HERE, "_build")
+        try:
+            os.makedirs(d, exist_ok=True)
+            fd, probe = tempfile.mkstemp(dir=d)
+            os.close(fd)
+            os.remove(probe)
+        except OSError:
+            d = os.path.join(tempfile.gettempdir(), f"sonicboom_amd_build_{os.getuid()}")
+            os.makedirs(d, exist_ok=True)
+        _BUILD_DIR = d
+    return _BUILD_DIR
 
 
 def _existing(names):
@@ -179,8 +184,8 @@ def build_all(force: bool = True) -> None:
     """Compile the core library and the attention libraries of the usual head sizes."""
     ensure_core(force=force)
     if _existing(ATTN_SOURCES):
-        for hd in PREBUILT_HEAD_DIMS:
-            ensure_attention(hd, force=force)
+        with ThreadPoolExecutor(max_workers=_jobs()) as ex:
+            list(ex.map(lambda hd: ensure_attention(hd, force=force), PREBUILT_HEAD_DIMS))
 
 
 if __name__ == "__main__":

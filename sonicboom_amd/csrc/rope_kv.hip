@@ -30,12 +30,14 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
 
   // Where this row's key and value go.
   size_t slot_base = 0;
+  int page_of_row = 0;
   bool store = heads_kv > 0;
   if (store) {
     const int seq = row_seq[row];
     const int lp = pos / SB_PAGE;
     const int page = (lp >= 0 && lp < max_pages) ? page_table[size_t(seq) * max_pages + lp] : -1;
     if (page < 0 || page >= n_pages_total) store = false;  // refused on the host; never write astray
+    page_of_row = page < 0 ? 0 : page;
     slot_base = (size_t(page < 0 ? 0 : page) * heads_kv * SB_PAGE + size_t(pos % SB_PAGE)) * head_dim;
   }
   const size_t head_step = size_t(SB_PAGE) * head_dim;  // from one kv head to the next within a page
@@ -74,10 +76,12 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
     const int kh = it / plain, d = first_plain + (it - kh * plain);
     st_f(k_cache, slot_base + kh * head_step + d, ld_f(r, size_t(q_width) + kh * head_dim + d));
   }
-  // Values.
+  // Values: the cache keeps them transposed, [d][position in page], so that the matrix-core
+  // kernels read eight consecutive keys of one d with one 16-byte load.
+  const size_t v_base = size_t(page_of_row) * heads_kv * head_step + size_t(pos % SB_PAGE);
   for (int it = threadIdx.x; it < kv_width; it += blockDim.x) {
     const int kh = it / head_dim, d = it - kh * head_dim;
-    st_f(v_cache, slot_base + kh * head_step + d, ld_f(r, size_t(q_width) + kv_width + it));
+    st_f(v_cache, v_base + kh * head_step + size_t(d) * SB_PAGE, ld_f(r, size_t(q_width) + kv_width + it));
   }
 }
 

@@ -10,8 +10,9 @@
  * never computed wrongly.
  *
  * Element types are named by sb_dtype.  Tensors are row-major and dense unless
- * a stride is given.  The KV cache is paged: a layer's keys (values) are
- * [pages][kv_heads][SB_PAGE][head_dim]; `page_table` is int32 [batch][max_pages]
+ * a stride is given.  The KV cache is paged: a layer's keys are
+ * [pages][kv_heads][SB_PAGE][head_dim], its values transposed,
+ * [pages][kv_heads][head_dim][SB_PAGE]; `page_table` is int32 [batch][max_pages]
  * and maps the logical page (position / SB_PAGE) of a sequence to a physical
  * page, -1 for none.
  */

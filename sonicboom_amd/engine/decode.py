@@ -1,0 +1,180 @@
+"""Repeated single-token steps of a set of sequences, with the step replayed as a HIP graph.
+
+A decode step of B sequences launches a few hundred small kernels; launched one
+by one from Python they cost more than the step's memory traffic.  The loop
+therefore keeps the step's bookkeeping (token ids, positions, page tables) in
+fixed device buffers, runs the step once or twice kernel by kernel, then
+captures exactly the same launches into a HIP graph per (batch size, page
+table width) and replays it, refreshing the buffers with one small copy per
+step.  Graph and kernel-by-kernel steps run the same kernels on the same
+shapes, so they give the same bits; the graph is only a way of launching.
+Nothing in the graph clears memory with a memset node.
+
+The reference captures its decode step the same way
+(/root/reference/core/src/model/gemma4_plan.cpp:1650-1687, :1704-1797: set the
+position, replay the captured step, read the token).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from .. import ops
+from ..cache.paged import CacheError
+from .step import StepError
+
+WIDTH_STEP = 16      # page-table widths are rounded up to this many pages (1024 tokens)
+CAPTURE_AFTER = 2    # kernel-by-kernel steps of a shape before its graph is captured
+
+
+class _StaticContext:
+    """A decode step's bookkeeping in device buffers whose addresses never change."""
+
+    def __init__(self, engine, batch: int, width: int):
+        cache = engine.cache
+        self.batch, self.width = batch, width
+        self.n_groups = len(cache.groups)
+        self.n_rows = self.n_seqs = self.n_wanted = batch
+        self.is_decode = True
+        self.max_new = 1
+        sizes = [batch, batch, batch, batch + 1, batch, batch, batch, 4 * batch] + [batch * width] * self.n_groups
+        total = sum(sizes)
+        dev = engine.device
+        # two pinned staging buffers used in turn: a step never overwrites the one whose copy
+        # may still be in flight
+        self._hosts = [torch.zeros(total, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self._turn = 0
+        self.dev = torch.zeros(total, dtype=torch.int32, device=dev)
+        self.next_ids = torch.zeros(batch, dtype=torch.int32, device=dev)
+        offs = np.concatenate([[0], np.cumsum(sizes)])
+        self._off = offs
+        v = [self.dev[offs[i]:offs[i + 1]] for i in range(len(sizes))]
+        (self.ids, self.row_pos, self.row_seq, self.cu_rows, self.len_before, self.slots, self.want_rows,
+         flat_tiles) = v[:8]
+        self.tiles = flat_tiles.view(-1, 4)
+        self._tables = [t.view(batch, width) for t in v[8:]]
+        # the parts that never change for a decode step of this batch size
+        ar = np.arange(batch, dtype=np.int32)
+        for h in self._hosts:
+            n = h.numpy()
+            n[offs[2]:offs[3]] = ar
+            n[offs[3]:offs[4]] = np.arange(batch + 1, dtype=np.int32)
+            n[offs[6]:offs[7]] = ar
+            n[offs[7]:offs[8]] = np.stack([ar, np.ones_like(ar), ar, np.zeros_like(ar)], axis=1).reshape(-1)
+
+    def page_table(self, group: int) -> torch.Tensor:
+        return self._tables[group]
+
+    def refresh(self, cache, slots: Sequence[int], tokens: Sequence[int]) -> None:
+        """This step's ids, positions and page tables, in one copy to the device."""
+        host = self._hosts[self._turn]
+        self._turn ^= 1
+        n, o = host.numpy(), self._off
+        lengths = np.asarray([cache.length(s) for s in slots], dtype=np.int32)
+        n[o[0]:o[1]] = np.asarray(tokens, dtype=np.int32)
+        n[o[1]:o[2]] = lengths
+        n[o[4]:o[5]] = lengths
+        n[o[5]:o[6]] = np.asarray(slots, dtype=np.int32)
+        for g in range(self.n_groups):
+            n[o[8 + g]:o[9 + g]] = cache.page_table(g, slots, min_width=self.width).reshape(-1)
+        self.max_len_after = int(lengths.max()) + 1
+        self.dev.copy_(host, non_blocking=True)
+
+
+class DecodeLoop:
+    """Single-token steps of a set of live sequences: ``step`` chooses greedily on the device,
+    ``step_logits`` hands the logits to a sampler."""
+
+    def __init__(self, engine, use_graph: bool = True):
+        self.engine = engine
+        self.use_graph = use_graph
+        self._ctx: Dict[Tuple[int, int], _StaticContext] = {}
+        self._graphs: Dict[Tuple[int, int, bool], Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
+        self._uses: Dict[Tuple[int, int, bool], int] = {}
+        self.slots: List[int] = []
+        self.pending: List[int] = []
+
+    def start(self, slots: Sequence[int], tokens: Sequence[int]) -> None:
+        """The sequences to continue and the token each feeds next."""
+        if len(slots) != len(tokens) or not slots:
+            raise StepError("a decode loop needs one next token per sequence")
+        self.slots = list(slots)
+        self.pending = [int(t) for t in tokens]
+
+    def close(self) -> None:
+        self._graphs.clear()
+        self._ctx.clear()
+
+    def _key(self) -> Tuple[int, int]:
+        cache = self.engine.cache
+        need = max((cache.length(s) + 1 + 63) // 64 for s in self.slots)
+        return len(self.slots), ((need + WIDTH_STEP - 1) // WIDTH_STEP) * WIDTH_STEP
+
+    def _run(self, tokens: Sequence[int], choose: bool):
+        """One step of the live sequences feeding ``tokens``: the logits [B, vocab] and the
+        buffer that holds the greedy choice when ``choose``."""
+        eng = self.engine
+        cache = eng.cache
+        vocab = eng.model.vocab
+        for t in tokens:
+            if not 0 <= t < vocab:
+                raise StepError(f"token id {t} is outside the vocabulary of {vocab}")
+        ones = [1] * len(self.slots)
+        try:
+            cache.reserve(self.slots, ones)
+        except CacheError as e:
+            raise StepError(str(e)) from None
+        key = self._key()
+        ctx = self._ctx.get(key)
+        if ctx is None:
+            ctx = self._ctx[key] = _StaticContext(eng, *key)
+        ctx.refresh(cache, self.slots, tokens)
+        gkey = (*key, choose)
+        entry = self._graphs.get(gkey)
+        if entry is not None:
+            entry[0].replay()
+            logits = entry[1]
+        else:
+            logits = eng.forward(ctx)
+            if choose:
+                ops.argmax(logits, out=ctx.next_ids)
+            n = self._uses[gkey] = self._uses.get(gkey, 0) + 1
+            if self.use_graph and n >= CAPTURE_AFTER:
+                self._capture(gkey, ctx, choose)
+        cache.advance(self.slots, ones)
+        return logits, ctx.next_ids
+
+    def _capture(self, gkey, ctx, choose: bool) -> None:
+        """Record the launches of a step of this shape.  Capture runs nothing; replays read the
+        ids, positions and page tables that ``refresh`` puts into the fixed buffers."""
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            logits = self.engine.forward(ctx)
+            if choose:
+                ops.argmax(logits, out=ctx.next_ids)
+        self._graphs[gkey] = (graph, logits)
+
+    def step(self) -> List[int]:
+        """Feed the pending tokens and choose greedily; the new token of every sequence, which
+        is also what the next step feeds."""
+        _, ids = self._run(self.pending, choose=True)
+        self.pending = ids.tolist()
+        return self.pending
+
+    def step_logits(self, tokens: Optional[Sequence[int]] = None) -> torch.Tensor:
+        """Feed ``tokens`` (default: the pending ones); float32 logits [B, vocab] of the new
+        positions, valid until the next step."""
+        if tokens is not None:
+            self.pending = [int(t) for t in tokens]
+        logits, _ = self._run(self.pending, choose=False)
+        return logits
+
+    def keep(self, flags: Sequence[bool], tokens: Optional[Sequence[int]] = None) -> None:
+        """Go on with the sequences whose flag is true; ``tokens`` (default: the pending ones)
+        are filtered alike and become what the next step feeds."""
+        src = self.pending if tokens is None else [int(t) for t in tokens]
+        self.slots = [s for s, k in zip(self.slots, flags) if k]
+        self.pending = [t for t, k in zip(src, flags) if k]

@@ -70,7 +70,9 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = 
     """Continue every prompt; returns the produced tokens per prompt.
 
     ``engine`` has ``alloc_slot()``, ``free_slot(slot)``, ``step(entries) ->
-    logits`` and ``cache.n_pages`` / ``cache.max_slots``.  ``stop_tokens``
+    logits`` and ``cache.n_pages`` / ``cache.max_slots``; when it also has
+    ``decode_loop()`` the single-token steps go through that loop (fixed buffers,
+    HIP graph replay, greedy choice on the device).  ``stop_tokens``
     defaults to the model's own (its configuration's eos ids).  ``callback(i,
     token)`` is called for every produced token of request i in order; a true
     return value ends that request, and the token it was called with is still
@@ -78,6 +80,7 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = 
     and defaults to the device sampler for ``params``.
     """
     params = params.validated()
+    own_sampler = sampler is None
     sampler = sampler or Sampler(params)
     if stop_tokens is None:
         stop_tokens = getattr(getattr(engine, "model", None), "spec", None)
@@ -89,14 +92,17 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = 
         return outputs
     batches = plan_batches([len(p) for p in prompts], params.max_tokens, engine.cache.n_pages, max_batch,
                            engine.cache.max_slots)
+    loop = engine.decode_loop() if hasattr(engine, "decode_loop") else None
+    on_device = loop is not None and own_sampler and not params.temperature > 0.0 and not params.has_penalties
     for batch in batches:
         live = [_Live(i, engine.alloc_slot(), list(prompts[i]), len(prompts[i])) for i in batch]
         try:
             # The prompts in one step; logits of every last row.
             logits = engine.step([StepEntry(s.slot, prompts[s.index], (s.prompt_len - 1,)) for s in live])
+            tokens = sampler.pick(logits, [len(s.history) for s in live], [s.history for s in live])
+            started = False
             while True:
-                tokens = sampler.pick(logits, [len(s.history) for s in live], [s.history for s in live])
-                nxt = []
+                flags = []
                 for s, t in zip(live, tokens):
                     t = int(t)
                     s.out.append(t)
@@ -108,12 +114,24 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = 
                         outputs[s.index] = s.out
                         engine.free_slot(s.slot)
                         s.slot = -1
-                    else:
-                        nxt.append(s)
-                live = nxt
+                    flags.append(not ended)
+                fed = [int(t) for t, k in zip(tokens, flags) if k]
+                live = [s for s, k in zip(live, flags) if k]
                 if not live:
                     break
-                logits = engine.step([StepEntry(s.slot, (s.history[-1],), (0,)) for s in live])
+                # every live sequence goes on by the token it has just produced
+                if loop is None:
+                    logits = engine.step([StepEntry(s.slot, (t,), (0,)) for s, t in zip(live, fed)])
+                    tokens = sampler.pick(logits, [len(s.history) for s in live], [s.history for s in live])
+                    continue
+                if not started or not all(flags):
+                    loop.start([s.slot for s in live], fed)
+                    started = True
+                if on_device:
+                    tokens = loop.step()             # greedy choice on the device, fed back by the loop
+                else:
+                    logits = loop.step_logits(fed)
+                    tokens = sampler.pick(logits, [len(s.history) for s in live], [s.history for s in live])
         finally:
             for s in live:
                 if s.slot >= 0:

@@ -20,6 +20,9 @@ from ..cache.paged import CacheError, PagedCache
 from .model import DecoderModel
 
 
+ROW_TILE = 16      # rows of one sequence that the attention kernels take together
+
+
 class StepError(ValueError):
     """A step that cannot run: unknown slot, token outside the vocabulary, no room in the cache."""
 
@@ -38,7 +41,9 @@ class StepContext:
     positions, ``row_seq`` [rows] index of the row's sequence in the batch,
     ``cu_rows`` [seqs+1] first row of every sequence, ``len_before`` [seqs]
     cached length before the step, ``slots`` [seqs] (rows of the state
-    tensors), ``want_rows`` [wanted]; ``page_table(group)`` [seqs, pages].
+    tensors), ``want_rows`` [wanted], ``tiles`` [n, 4] (first row, rows <= 16,
+    sequence, 0: runs of consecutive rows of one sequence);
+    ``page_table(group)`` [seqs, pages].
     Host: ``n_rows``, ``n_seqs``, ``n_new`` list, ``lengths_before`` list,
     ``is_decode`` (every sequence brings one token), ``max_new``,
     ``max_len_after``.
@@ -62,8 +67,12 @@ class StepContext:
         want = [int(cu[i]) + int(w) for i, e in enumerate(entries) for w in e.want]
         self.n_wanted = len(want)
         tables = [cache.page_table(g, self.slot_list) for g in range(len(cache.groups))]
+        # runs of up to 16 consecutive rows of one sequence: (first row, rows, sequence, 0)
+        tiles = np.asarray([(int(cu[i]) + r0, min(ROW_TILE, n - r0), i, 0)
+                            for i, n in enumerate(self.n_new) for r0 in range(0, n, ROW_TILE)], dtype=np.int32)
         parts = [ids, row_pos, row_seq, cu, np.asarray(self.lengths_before, dtype=np.int32),
-                 np.asarray(self.slot_list, dtype=np.int32), np.asarray(want, dtype=np.int32)]
+                 np.asarray(self.slot_list, dtype=np.int32), np.asarray(want, dtype=np.int32),
+                 tiles.reshape(-1)]
         parts += [t.reshape(-1) for t in tables]
         sizes = [p.size for p in parts]
         # One pinned staging buffer, one copy to the device, views into it.
@@ -76,8 +85,9 @@ class StepContext:
             views.append(dev[off:off + n])
             off += n
         (self.ids, self.row_pos, self.row_seq, self.cu_rows, self.len_before, self.slots,
-         self.want_rows) = views[:7]
-        self._tables = [v.view(t.shape) for v, t in zip(views[7:], tables)]
+         self.want_rows, flat_tiles) = views[:8]
+        self.tiles = flat_tiles.view(-1, 4)
+        self._tables = [v.view(t.shape) for v, t in zip(views[8:], tables)]
         self.host_row_pos = row_pos
 
     def page_table(self, group: int) -> torch.Tensor:
@@ -92,6 +102,15 @@ class Engine:
         self.device = model.rt.device
         self.cache = model.new_cache(max_tokens, max_slots)
         self.bindings = model.bindings(self.cache)
+        self.use_graphs = True
+        self._loop = None
+
+    def decode_loop(self):
+        """The engine's loop for single-token steps (one per engine: it keeps the captured graphs)."""
+        if self._loop is None:
+            from .decode import DecodeLoop
+            self._loop = DecodeLoop(self, use_graph=self.use_graphs)
+        return self._loop
 
     # ---- slots -----------------------------------------------------------------
     def alloc_slot(self) -> int:
@@ -129,12 +148,18 @@ class Engine:
             self.cache.reserve(slots, n_new)
         except CacheError as e:
             raise StepError(str(e)) from None
-        model = self.model
         ctx = StepContext(self.cache, entries, self.device)
+        logits = self.forward(ctx)
+        self.cache.advance(slots, n_new)
+        return logits
+
+    def forward(self, ctx) -> torch.Tensor:
+        """The device work of a step whose bookkeeping ``ctx`` holds: embedding, the blocks in
+        their run order, and for the wanted rows the final norm and the head."""
+        model = self.model
         x = model.embedding.forward(ctx.ids)
         for i, e in enumerate(model.order):
             model.blocks[e.block].forward(x, ctx, self.bindings[i])
-        self.cache.advance(slots, n_new)
         if ctx.n_wanted == 0:
             return torch.empty((0, model.vocab), dtype=torch.float32, device=self.device)
         h = model.final_norm.forward(x, model.rt.act_dtype, rows=ctx.want_rows)

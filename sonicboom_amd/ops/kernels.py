@@ -143,11 +143,12 @@ def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
 
 
 def _check_cache(k_cache, v_cache, heads_kv, head_dim):
-    if k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (heads_kv, PAGE, head_dim) or k_cache.shape != v_cache.shape \
+    if k_cache.dim() != 4 or v_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (heads_kv, PAGE, head_dim) \
+            or tuple(v_cache.shape[1:]) != (heads_kv, head_dim, PAGE) or k_cache.shape[0] != v_cache.shape[0] \
             or k_cache.dtype != v_cache.dtype:
         raise KernelLibraryError(
-            f"cache must be [pages, {heads_kv}, {PAGE}, {head_dim}] for keys and values alike, "
-            f"found {tuple(k_cache.shape)} and {tuple(v_cache.shape)}")
+            f"cache must be keys [pages, {heads_kv}, {PAGE}, {head_dim}] and values "
+            f"[pages, {heads_kv}, {head_dim}, {PAGE}], found {tuple(k_cache.shape)} and {tuple(v_cache.shape)}")
 
 
 def _check_rows(row_pos, row_seq, page_table, n_rows):
@@ -294,9 +295,73 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], re
     return out
 
 
+MFMA_MAX_HEAD_DIM = 256
+
+
+def attention_mfma_ok(q_dtype, cache_dtype, head_dim: int) -> bool:
+    """Whether the matrix-core attention kernels take these types and this head size."""
+    return (q_dtype == torch.bfloat16 and cache_dtype == torch.bfloat16 and head_dim % 16 == 0
+            and 16 <= head_dim <= MFMA_MAX_HEAD_DIM)
+
+
+def attention_decode_mfma(q, k_cache, v_cache, page_table, seq_pos, heads_q, heads_kv, head_dim, scale, window):
+    """One bf16 query row per sequence (row i belongs to row i of ``page_table``) at position
+    ``seq_pos[i]``, over the cache; keys are split over blocks and merged in ascending order."""
+    _dev(q, k_cache, v_cache, page_table, seq_pos)
+    n = q.shape[0]
+    if q.dim() != 2 or q.shape[1] != heads_q * head_dim or q.dtype != torch.bfloat16:
+        raise KernelLibraryError(f"queries must be bfloat16 [sequences, {heads_q * head_dim}]")
+    _check_cache(k_cache, v_cache, heads_kv, head_dim)
+    _i32(seq_pos, n, "sequence positions")
+    if page_table.dtype != torch.int32 or page_table.dim() != 2 or page_table.shape[0] < n:
+        raise KernelLibraryError("page table must be int32 [sequences, pages]")
+    lib = library.attention_library(head_dim)
+    max_pages = page_table.shape[1]
+    chunks = lib.sb_attn_decode_chunks(max_pages)
+    out = torch.empty_like(q)
+    part_o = part_ml = None
+    if chunks > 1:
+        part_o = torch.empty((n * heads_q * chunks * head_dim,), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((n * heads_q * chunks * 2,), dtype=torch.float32, device=q.device)
+    check(lib.sb_attn_decode_bf16(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(page_table), max_pages,
+                                  k_cache.shape[0], _p(seq_pos), _p(part_o), _p(part_ml), n, heads_q, heads_kv,
+                                  float(scale), int(window), _stream()), lib, "sb_attn_last_error")
+    return out
+
+
+def attention_prefill_mfma(q, k_cache, v_cache, page_table, row_pos, tiles, heads_q, heads_kv, head_dim, scale,
+                           window):
+    """bf16 query rows over the cache; ``tiles`` int32 [n, 4] = (first row, rows <= 16, sequence, 0)
+    cuts the rows into runs of consecutive positions of one sequence."""
+    _dev(q, k_cache, v_cache, page_table, row_pos, tiles)
+    n = q.shape[0]
+    if q.dim() != 2 or q.shape[1] != heads_q * head_dim or q.dtype != torch.bfloat16:
+        raise KernelLibraryError(f"queries must be bfloat16 [rows, {heads_q * head_dim}]")
+    _check_cache(k_cache, v_cache, heads_kv, head_dim)
+    _i32(row_pos, n, "row positions")
+    if tiles.dtype != torch.int32 or tiles.dim() != 2 or tiles.shape[1] != 4:
+        raise KernelLibraryError("tiles must be int32 [n, 4]")
+    if page_table.dtype != torch.int32 or page_table.dim() != 2:
+        raise KernelLibraryError("page table must be int32 [sequences, pages]")
+    lib = library.attention_library(head_dim)
+    out = torch.empty_like(q)
+    check(lib.sb_attn_prefill_bf16(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(page_table), page_table.shape[1],
+                                   k_cache.shape[0], _p(row_pos), _p(tiles), tiles.shape[0], heads_q, heads_kv,
+                                   float(scale), int(window), _stream()), lib, "sb_attn_last_error")
+    return out
+
+
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor, ctx,
               heads_q: int, heads_kv: int, head_dim: int, scale: float, window: int,
               fast: bool = True) -> torch.Tensor:
-    """Attention of a step's rows over the cache; ``ctx`` is the step's context."""
+    """Attention of a step's rows over the cache; ``ctx`` is the step's context.  bfloat16 with a
+    head size in steps of 16 runs on the matrix cores (a decode kernel when every sequence brings
+    one row, else the prefill kernel); everything else takes the plain kernel."""
+    if fast and attention_mfma_ok(q.dtype, k_cache.dtype, head_dim):
+        if ctx.is_decode:
+            return attention_decode_mfma(q, k_cache, v_cache, page_table, ctx.row_pos, heads_q, heads_kv,
+                                         head_dim, scale, window)
+        return attention_prefill_mfma(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.tiles, heads_q, heads_kv,
+                                      head_dim, scale, window)
     return attention_plain(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_seq, heads_q, heads_kv,
                            head_dim, scale, window)

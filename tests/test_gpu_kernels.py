@@ -162,8 +162,11 @@ def test_silu_mul_add_cast(dtype):
 
 
 def make_cache(n_pages, heads_kv, head_dim, dtype, fill=float("nan")):
+    """Keys [pages, heads, 64, d] and values [pages, heads, d, 64], filled with NaN: whatever a
+    kernel reads beyond what was stored shows in its result."""
     k = torch.full((n_pages, heads_kv, 64, head_dim), fill, dtype=dtype, device=DEV)
-    return k, k.clone()
+    v = torch.full((n_pages, heads_kv, head_dim, 64), fill, dtype=dtype, device=DEV)
+    return k, v
 
 
 @pytest.mark.parametrize("hq, hkv, hd, rot", [(4, 2, 16, 0), (3, 1, 32, 0), (5, 5, 48, 0), (2, 1, 64, 32), (8, 2, 128, 0)])
@@ -196,7 +199,7 @@ def test_rope_kv_store(hq, hkv, hd, rot, dtype):
     for r in range(n):
         page = table[seq[r], pos[r] // 64]
         got_k = kc[page, :, pos[r] % 64, :].reshape(-1)
-        got_v = vc[page, :, pos[r] % 64, :].reshape(-1)
+        got_v = vc[page, :, :, pos[r] % 64].reshape(-1)
         close(got_k, want_k[r], what=f"k row {r}", **tol)
         close(got_v, qkv[r, qw + kvw:].to(dtype).float(), atol=0, rtol=0, what=f"v row {r}")
     # nothing else was written
@@ -235,7 +238,7 @@ def fill_cache_from(keys, values, table, dtype):
         for p in range(k.shape[0]):
             page = table[s, p // 64]
             kc[page, :, p % 64, :] = k[p].to(dtype)
-            vc[page, :, p % 64, :] = v[p].to(dtype)
+            vc[page, :, :, p % 64] = v[p].to(dtype)
     return kc, vc
 
 
@@ -266,6 +269,75 @@ def test_attention_plain_kernel(hq, hkv, hd, dtype, window):
                                causal=True, window=window)
         tol = dict(atol=3e-6, rtol=2e-5) if dtype == F32 else dict(atol=2e-2, rtol=1e-2)
         close(got[r:r + 1], want, what=f"row {r} (seq {s}, pos {p})", **tol)
+
+
+def attention_case(hq, hkv, hd, lens, rows_per_seq, window, seed=0):
+    """Random bf16 keys, values and queries for sequences of ``lens`` tokens on scattered pages;
+    ``rows_per_seq[s]`` lists the positions of sequence s that ask.  Returns device operands and the
+    plain result per row."""
+    n_seq = len(lens)
+    width = max((n + 63) // 64 for n in lens)
+    perm = torch.randperm(n_seq * width + 3, generator=torch.Generator().manual_seed(seed))
+    table = torch.full((n_seq, width), -1, dtype=torch.int32)
+    it = iter(perm.tolist())
+    for s_, n in enumerate(lens):
+        for pg in range((n + 63) // 64):
+            table[s_, pg] = next(it)
+    keys = [randn(n, hkv, hd, seed=seed + s_).to(BF16).float() for s_, n in enumerate(lens)]
+    vals = [randn(n, hkv, hd, seed=seed + 50 + s_).to(BF16).float() for s_, n in enumerate(lens)]
+    hkv_, hd_ = keys[0].shape[1:]
+    kc, vc = make_cache(n_seq * width + 3, hkv_, hd_, BF16)
+    for s_, (k, v) in enumerate(zip(keys, vals)):
+        for p in range(k.shape[0]):
+            page = table[s_, p // 64]
+            kc[page, :, p % 64, :] = k[p].to(BF16)
+            vc[page, :, :, p % 64] = v[p].to(BF16)
+    rows = [(s_, p) for s_, ps in enumerate(rows_per_seq) for p in ps]
+    q = randn(len(rows), hq * hd, seed=seed + 7).to(BF16)
+    scale = 1.0 / math.sqrt(hd)
+    want = []
+    for r, (s_, p) in enumerate(rows):
+        n = lens[s_]
+        want.append(plain.attention(q[r:r + 1].float().numpy(), keys[s_].reshape(n, -1).numpy(),
+                                    vals[s_].reshape(n, -1).numpy(), [p], np.arange(n), hq, hkv, hd, scale,
+                                    causal=True, window=window))
+    return q, kc, vc, table, rows, scale, np.concatenate(want, axis=0)
+
+
+MFMA_SHAPES = [(4, 2, 16), (3, 1, 32), (5, 5, 48), (6, 2, 80), (28, 4, 128), (2, 1, 256), (40, 2, 64)]
+
+
+@pytest.mark.parametrize("hq, hkv, hd", MFMA_SHAPES)
+@pytest.mark.parametrize("window", [0, 70])
+def test_attention_decode_matrix_cores(hq, hkv, hd, window):
+    """One row per sequence, lengths on both sides of page and chunk (4 pages) edges."""
+    from sonicboom_amd import ops
+    lens = [1, 2, 64, 65, 255, 256, 257, 700]
+    q, kc, vc, table, rows, scale, want = attention_case(hq, hkv, hd, lens, [[n - 1] for n in lens], window)
+    pos = torch.tensor([p for _, p in rows], dtype=torch.int32)
+    got = ops.attention_decode_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), hq, hkv, hd, scale, window)
+    close(got, want, atol=1.5e-2, rtol=1e-2, what="decode")
+
+
+@pytest.mark.parametrize("hq, hkv, hd", MFMA_SHAPES)
+@pytest.mark.parametrize("window", [0, 70])
+def test_attention_prefill_matrix_cores(hq, hkv, hd, window):
+    """Whole prompts of unequal lengths, and a continuation on top of cached keys."""
+    from sonicboom_amd import ops
+    lens = [1, 17, 64, 150, 200]
+    starts = [0, 0, 0, 0, 120]           # the last sequence has 120 keys cached and brings 80 rows
+    rows_per_seq = [list(range(s0, n)) for s0, n in zip(starts, lens)]
+    q, kc, vc, table, rows, scale, want = attention_case(hq, hkv, hd, lens, rows_per_seq, window, seed=3)
+    pos = torch.tensor([p for _, p in rows], dtype=torch.int32)
+    tiles, row0 = [], 0
+    for s_, ps in enumerate(rows_per_seq):
+        for r0 in range(0, len(ps), 16):
+            tiles.append((row0 + r0, min(16, len(ps) - r0), s_, 0))
+        row0 += len(ps)
+    tiles = torch.tensor(tiles, dtype=torch.int32)
+    got = ops.attention_prefill_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), tiles.to(DEV), hq, hkv, hd,
+                                     scale, window)
+    close(got, want, atol=1.5e-2, rtol=1e-2, what="prefill")
 
 
 def test_attention_reference_vectors():
