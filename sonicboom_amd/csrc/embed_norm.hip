@@ -23,7 +23,12 @@ __global__ void embed_kernel(float *__restrict__ out, const TT *__restrict__ tab
 }
 
 constexpr int kNormThreads = 256;
+constexpr int kNormKeep = 8;   // float4 groups of a row that a thread keeps in registers
 
+// One block per row.  A thread takes float4 groups tid, tid + 256, ...; all of a thread's loads
+// are issued before the first is used, and the first kNormKeep groups stay in registers for the
+// second pass.  The squares are summed in double: per thread in ascending order, then by a
+// fixed butterfly over the wave, then wave by wave.
 template <typename TO>
 __global__ void __launch_bounds__(kNormThreads)
 rmsnorm_kernel(TO *__restrict__ y, const float *__restrict__ x, const void *__restrict__ w,
@@ -32,32 +37,54 @@ rmsnorm_kernel(TO *__restrict__ y, const float *__restrict__ x, const void *__re
   const int src = rows ? rows[r] : r;
   const float *xr = x + size_t(src) * width;
   TO *yr = y + size_t(r) * width;
+  const int tid = threadIdx.x;
+  const bool vec = (width % 4 == 0) && (reinterpret_cast<uintptr_t>(xr) % 16 == 0);
+  const int n_groups = vec ? width / 4 : 0;
 
-  // Each thread sums its strided elements in ascending order; the partial sums
-  // are combined by a fixed butterfly, then wave by wave in ascending order.
+  float4 keep[kNormKeep];
   double part = 0.0;
-  for (int i = threadIdx.x; i < width; i += kNormThreads) {
+#pragma unroll
+  for (int i = 0; i < kNormKeep; ++i) {
+    const int g = tid + i * kNormThreads;
+    keep[i] = g < n_groups ? reinterpret_cast<const float4 *>(xr)[g] : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+#pragma unroll
+  for (int i = 0; i < kNormKeep; ++i)
+    part += double(keep[i].x * keep[i].x) + double(keep[i].y * keep[i].y) + double(keep[i].z * keep[i].z) +
+            double(keep[i].w * keep[i].w);
+  // what does not fit the registers, or a row that cannot be read in groups of four
+  const int tail0 = vec ? min(n_groups, kNormKeep * kNormThreads) * 4 : 0;
+  for (int i = tail0 + tid; i < width; i += kNormThreads) {
     const float v = xr[i];
     part += double(v * v);
   }
   part = wave_sum(part);
   __shared__ double wave_part[kNormThreads / 64];
-  __shared__ float inv_s;
-  if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = part;
+  if ((tid & 63) == 0) wave_part[tid >> 6] = part;
   __syncthreads();
-  if (threadIdx.x == 0) {
-    double total = 0.0;
-    for (int k = 0; k < kNormThreads / 64; ++k) total += wave_part[k];
-    const float mean = float(total / double(width));
-    inv_s = 1.0f / sqrtf(mean + eps);
+  double total = 0.0;
+#pragma unroll
+  for (int k = 0; k < kNormThreads / 64; ++k) total += wave_part[k];
+  const float mean = float(total / double(width));
+  const float inv = 1.0f / sqrtf(mean + eps);
+
+#pragma unroll
+  for (int i = 0; i < kNormKeep; ++i) {
+    const int g = tid + i * kNormThreads;
+    if (g < n_groups) {
+      const float v[4] = {keep[i].x, keep[i].y, keep[i].z, keep[i].w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float o = v[e] * inv;
+        if (w) o = o * ld_dyn(w, w_dtype, g * 4 + e);
+        st_f(yr, g * 4 + e, o);
+      }
+    }
   }
-  __syncthreads();
-  const float inv = inv_s;
-  if (w == nullptr) {
-    for (int i = threadIdx.x; i < width; i += kNormThreads) st_f(yr, i, xr[i] * inv);
-  } else {
-    for (int i = threadIdx.x; i < width; i += kNormThreads)
-      st_f(yr, i, (xr[i] * inv) * ld_dyn(w, w_dtype, i));
+  for (int i = tail0 + tid; i < width; i += kNormThreads) {
+    float o = xr[i] * inv;
+    if (w) o = o * ld_dyn(w, w_dtype, i);
+    st_f(yr, i, o);
   }
 }
 

@@ -35,13 +35,17 @@ struct Args {
   int n_rows, n_out, n_in;
   int gated;       // W is [2*n_out, n_in]: rows n (gate) and n_out + n (up)
   int tiles_m, tiles_n;
+  int w_tiles;     // packed W: 16-row tiles of one half (ceil(n_out / 16))
+  int w_steps;     // packed W: 32-wide k-steps (ceil(n_in / 32))
 };
 
 __device__ __forceinline__ int swz(int row, int chunk) { return row * kChunksPerRow + (chunk ^ (row & 7)); }
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
-template <int GATED>
+// PACKED: W comes in the packed tile layout (1 KB blocks of 16 rows x 32 k in fragment order,
+// zero padded), which makes its global loads contiguous and free of bounds checks.
+template <int GATED, bool PACKED>
 __global__ void __launch_bounds__(kThreads)
 gemm_mfma_kernel(Args a) {
   __shared__ uint4 lds_a[2][BM * kChunksPerRow];
@@ -75,8 +79,28 @@ gemm_mfma_kernel(Args a) {
     sa[i] = swz(row, c);
     ca[i] = c * 8;
   }
+  int step_b[kLoadsB];    // packed: which of the two k-steps of a BK stage this load takes
 #pragma unroll
   for (int i = 0; i < kLoadsB; ++i) {
+    if (PACKED) {
+      // load id -> 1 KB block (id / 64) = (row tile of the LDS tile, k-step), lane id % 64
+      const int id = tid + kThreads * i, blk = id >> 6, l = id & 63;
+      const int rt = blk >> 1, j = blk & 1;      // LDS rows rt * 16 .., k-step j of the stage
+      int tile;
+      if (GATED) {
+        const int half = rt >> 2, within = rt & 3;
+        tile = (within >> 1) * a.w_tiles + min(n0 / 16 + half * 2 + (within & 1), a.w_tiles - 1);
+      } else {
+        tile = min(n0 / 16 + rt, a.w_tiles - 1);
+      }
+      okb[i] = true;
+      gb[i] = a.w + size_t(tile) * a.w_steps * 512 + size_t(l) * 8;
+      sb_[i] = swz(rt * 16 + (l & 15), j * 4 + (l >> 4));
+      cb[i] = 0;
+      step_b[i] = j;
+      continue;
+    }
+    step_b[i] = 0;
     const int id = tid + kThreads * i, row = id / kChunksPerRow, c = id % kChunksPerRow;
     int n;       // output feature, and the row of W that feeds LDS row `row`
     int wrow;
@@ -109,7 +133,14 @@ gemm_mfma_kernel(Args a) {
 #pragma unroll
     for (int i = 0; i < kLoadsA; ++i) ra[i] = ld16(ga[i] + k0, oka[i] && (k0 + ca[i]) < a.n_in);
 #pragma unroll
-    for (int i = 0; i < kLoadsB; ++i) rb[i] = ld16(gb[i] + k0, okb[i] && (k0 + cb[i]) < a.n_in);
+    for (int i = 0; i < kLoadsB; ++i) {
+      if (PACKED) {
+        const int ks = k0 / 32 + step_b[i];
+        rb[i] = ld16(gb[i] + size_t(ks) * 512, ks < a.w_steps);
+      } else {
+        rb[i] = ld16(gb[i] + k0, okb[i] && (k0 + cb[i]) < a.n_in);
+      }
+    }
   };
   auto store_lds = [&](int buf) {
 #pragma unroll
@@ -180,10 +211,11 @@ gemm_mfma_kernel(Args a) {
 }  // namespace
 
 // Y = X W^T (+bias) (+resid), or gated: Y = silu(X Wg^T) * (X Wu^T), W = [Wg; Wu].
-// X [n_rows, n_in] and W bf16, n_in a multiple of 8, operands 16-byte aligned.
+// X [n_rows, n_in] and W bf16, n_in a multiple of 8, operands 16-byte aligned; packed != 0: W is
+// in the packed tile layout.
 extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,
                                  int bias_dtype, const float *resid, int n_rows, int n_out, int n_in,
-                                 int gated, void *stream) {
+                                 int gated, int packed, void *stream) {
   SB_REQUIRE(y && x && w, "sb_gemm_mfma_bf16: null pointer");
   SB_REQUIRE(n_rows >= 0 && n_out > 0 && n_in > 0, "sb_gemm_mfma_bf16: bad sizes rows=%d out=%d in=%d",
              n_rows, n_out, n_in);
@@ -204,7 +236,11 @@ extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void
   const long long blocks = (long long)a.tiles_m * a.tiles_n;
   SB_SUPPORT(blocks <= 0x7fffffffLL, "sb_gemm_mfma_bf16: too many tiles");
   hipStream_t s = (hipStream_t)stream;
-  if (gated) gemm_mfma_kernel<1><<<unsigned(blocks), kThreads, 0, s>>>(a);
-  else gemm_mfma_kernel<0><<<unsigned(blocks), kThreads, 0, s>>>(a);
+  a.w_tiles = (n_out + 15) / 16;
+  a.w_steps = (n_in + 31) / 32;
+  if (gated && packed) gemm_mfma_kernel<1, true><<<unsigned(blocks), kThreads, 0, s>>>(a);
+  else if (gated) gemm_mfma_kernel<1, false><<<unsigned(blocks), kThreads, 0, s>>>(a);
+  else if (packed) gemm_mfma_kernel<0, true><<<unsigned(blocks), kThreads, 0, s>>>(a);
+  else gemm_mfma_kernel<0, false><<<unsigned(blocks), kThreads, 0, s>>>(a);
   return sb::check_launch("sb_gemm_mfma_bf16");
 }

@@ -2,8 +2,8 @@
 // t <= 64, with the epilogues the model needs (bias, residual, SiLU gate).
 //
 // The step is bound by reading W once from HBM.  A block owns 16*R output
-// features; its four waves take the k-steps of the block's K slice in turn
-// (wave w: steps w, w+4, ...), each loading W fragments straight from global
+// features; its four waves take a quarter each of the k-steps of the block's K
+// slice, each loading W fragments straight from global
 // memory into MFMA operands (16 rows x 64 bytes per load, every byte of W
 // read once) and the matching X fragments from cache.  The waves' partial
 // tiles are summed through shared memory in wave order, so the result does
@@ -42,7 +42,10 @@ __device__ __forceinline__ void store_out(const Epilogue &e, int t, int n, float
 }
 
 // G = 1: plain.  G = 2: rows n and n_out + n of W are gate and up of output n.
-template <int R, int TT, int G>
+// PACKED: W is stored tile by tile in MFMA fragment order (see sb_hip.h, "packed weights"): the
+// fragment of row tile nb and k-step ks is the 1 KB block (nb * n_steps + ks), lane l's eight
+// elements at l * 8; rows and k are padded with zeros to whole tiles.
+template <int R, int TT, int G, bool PACKED>
 __global__ void __launch_bounds__(kThreads)
 gemm_skinny_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ w, Epilogue ep,
                    float *__restrict__ partial, int n_in, int steps_per_slice) {
@@ -63,14 +66,21 @@ gemm_skinny_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ w, E
 
   const bf16_t *w_row[G * R];
   bool w_ok[G * R];
+  const int tiles_out = (ep.n_out + 15) / 16;
 #pragma unroll
   for (int g = 0; g < G; ++g)
 #pragma unroll
     for (int i = 0; i < R; ++i) {
       const int n = n0 + i * 16 + r;
-      w_ok[g * R + i] = n < ep.n_out;
-      const int row = min(g * ep.n_out + n, n_w_rows - 1);
-      w_row[g * R + i] = w + size_t(row) * n_in;
+      if (PACKED) {
+        const int tile = blockIdx.x * R + i;
+        w_ok[g * R + i] = tile < tiles_out;
+        w_row[g * R + i] = w + (size_t(g * tiles_out + min(tile, tiles_out - 1)) * n_steps) * 512 + lane * 8;
+      } else {
+        w_ok[g * R + i] = n < ep.n_out;
+        const int row = min(g * ep.n_out + n, n_w_rows - 1);
+        w_row[g * R + i] = w + size_t(row) * n_in;
+      }
     }
   const bf16_t *x_row[TT];
   bool x_ok[TT];
@@ -81,18 +91,25 @@ gemm_skinny_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ w, E
     x_row[j] = x + size_t(min(t, ep.n_rows - 1)) * n_in;
   }
 
-  // U steps' fragments are requested before the first MFMA, to keep loads in flight.
+  // Each wave takes a contiguous quarter of the slice's k-steps, so that it streams whole
+  // cache lines of every row; U steps' fragments are requested before the first MFMA, to
+  // keep loads in flight.
   constexpr int U = (G * R + TT <= 4) ? 4 : 2;
-  for (int s = s_begin + wave; s < s_end; s += kWaves * U) {
+  const int per_wave = (s_end - s_begin + kWaves - 1) / kWaves;
+  const int w_begin = s_begin + wave * per_wave;
+  const int w_end = min(w_begin + per_wave, s_end);
+  for (int s = w_begin; s < w_end; s += U) {
     uint4 a[U][G * R], b[U][TT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int ss = s + u * kWaves;
+      const int ss = s + u;
       const int k = ss * kStepK + q * 8;
       // n_in is a multiple of 8: a 16-byte group lies inside a row or outside as a whole
-      const bool k_ok = ss < s_end && k < n_in;
+      const bool k_ok = ss < w_end && k < n_in;
 #pragma unroll
-      for (int i = 0; i < G * R; ++i) a[u][i] = ld16(w_row[i] + k, k_ok && w_ok[i]);
+      for (int i = 0; i < G * R; ++i)
+        a[u][i] = PACKED ? ld16(w_row[i] + size_t(ss) * 512, ss < w_end && w_ok[i])
+                         : ld16(w_row[i] + k, k_ok && w_ok[i]);
 #pragma unroll
       for (int j = 0; j < TT; ++j) b[u][j] = ld16(x_row[j] + k, k_ok && x_ok[j]);
     }
@@ -169,12 +186,12 @@ reduce_slices_kernel(const float *__restrict__ partial, Epilogue ep, int n_slice
   store_out(ep, t, n, ep.gated ? silu_f(g) * u : g);
 }
 
-template <int R, int TT, int G>
+template <int R, int TT, int G, bool PACKED>
 void launch(const bf16_t *x, const bf16_t *w, const Epilogue &ep, float *partial, int n_in,
             int n_slices, int steps_per_slice, hipStream_t s) {
   dim3 grid((ep.n_out + 16 * R - 1) / (16 * R), n_slices);
   const size_t lds = size_t(kWaves) * G * R * TT * 64 * 4 * sizeof(float);
-  auto kern = gemm_skinny_kernel<R, TT, G>;
+  auto kern = gemm_skinny_kernel<R, TT, G, PACKED>;
   static bool raised = false;   // once per instantiation: allow more than the default dynamic LDS
   if (lds > 48 * 1024 && !raised) {
     (void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
@@ -183,14 +200,15 @@ void launch(const bf16_t *x, const bf16_t *w, const Epilogue &ep, float *partial
   kern<<<grid, kThreads, lds, s>>>(x, w, ep, partial, n_in, steps_per_slice);
 }
 
-template <int G>
+template <int G, bool PACKED>
 void launch_rt(int R, int TT, const bf16_t *x, const bf16_t *w, const Epilogue &ep, float *partial,
                int n_in, int n_slices, int steps_per_slice, hipStream_t s) {
 #define SB_CASE(r, tt) \
-  if (R == r && TT == tt) return launch<r, tt, G>(x, w, ep, partial, n_in, n_slices, steps_per_slice, s)
+  if (R == r && TT == tt) \
+  return launch<r, tt, G, PACKED>(x, w, ep, partial, n_in, n_slices, steps_per_slice, s)
   SB_CASE(1, 1); SB_CASE(1, 2); SB_CASE(1, 4);
   SB_CASE(2, 1); SB_CASE(2, 2); SB_CASE(2, 4);
-  SB_CASE(4, 1); SB_CASE(4, 2); SB_CASE(4, 4);
+  if (G == 1) { SB_CASE(4, 1); SB_CASE(4, 2); SB_CASE(4, 4); }
 #undef SB_CASE
 }
 
@@ -206,12 +224,14 @@ namespace {
 struct Plan {
   int R, TT, n_slices, steps_per_slice;
 };
+int g_force_r = 0, g_force_slices = 0;   // measurement hooks, see sb_gemm_skinny_force
 Plan plan_for(int n_rows, int n_out, int n_in, int gated) {
   Plan p;
   p.TT = n_rows <= 16 ? 1 : (n_rows <= 32 ? 2 : 4);
   const int tiles = (n_out + 15) / 16;
   p.R = tiles >= 2048 ? 4 : (tiles >= 1024 ? 2 : 1);
   if (gated && p.R == 4) p.R = 2;   // gate and up double the fragments a wave holds
+  if (g_force_r) p.R = g_force_r;
   const int blocks = (tiles + p.R - 1) / p.R;
   const int n_steps = (n_in + kStepK - 1) / kStepK;
   int slices = 1;
@@ -221,11 +241,19 @@ Plan plan_for(int n_rows, int n_out, int n_in, int gated) {
     if (slices > most) slices = most;
     if (slices < 1) slices = 1;
   }
+  if (g_force_slices) slices = g_force_slices;
   p.steps_per_slice = (n_steps + slices - 1) / slices;
   p.n_slices = (n_steps + p.steps_per_slice - 1) / p.steps_per_slice;
   return p;
 }
 }  // namespace
+
+// For measurements: fix the rows-tiles per block (1, 2, 4; 0 = choose) and the number of K
+// slices over the grid (0 = choose) of every later call.
+extern "C" void sb_gemm_skinny_force(int r, int slices) {
+  g_force_r = r;
+  g_force_slices = slices;
+}
 
 extern "C" size_t sb_gemm_skinny_scratch(int n_rows, int n_out, int n_in, int gated) {
   if (n_rows <= 0 || n_out <= 0 || n_in <= 0) return 0;
@@ -235,9 +263,11 @@ extern "C" size_t sb_gemm_skinny_scratch(int n_rows, int n_out, int n_in, int ga
 
 // Y = X W^T (+bias) (+resid), or with gated != 0: Y = silu(X Wg^T) * (X Wu^T) where W = [Wg; Wu]
 // is [2*n_out, n_in].  X [n_rows, n_in] and W are bf16; n_rows <= 64; n_in a multiple of 8.
+// packed != 0: W is in the packed tile layout (sb_pack_weight_bf16).
 extern "C" int sb_gemm_skinny_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,
                                    int bias_dtype, const float *resid, int n_rows, int n_out, int n_in,
-                                   int gated, float *scratch, size_t scratch_floats, void *stream) {
+                                   int gated, int packed, float *scratch, size_t scratch_floats,
+                                   void *stream) {
   SB_REQUIRE(y && x && w, "sb_gemm_skinny_bf16: null pointer");
   SB_REQUIRE(n_rows >= 0 && n_out > 0 && n_in > 0, "sb_gemm_skinny_bf16: bad sizes rows=%d out=%d in=%d",
              n_rows, n_out, n_in);
@@ -256,12 +286,11 @@ extern "C" int sb_gemm_skinny_bf16(void *y, int y_dtype, const void *x, const vo
   hipStream_t s = (hipStream_t)stream;
   Epilogue ep{y, y_dtype, bias, bias_dtype, resid, n_rows, n_out, gated ? 1 : 0};
   float *partial = p.n_slices > 1 ? scratch : nullptr;
-  if (gated)
-    launch_rt<2>(p.R, p.TT, (const bf16_t *)x, (const bf16_t *)w, ep, partial, n_in, p.n_slices,
-                 p.steps_per_slice, s);
-  else
-    launch_rt<1>(p.R, p.TT, (const bf16_t *)x, (const bf16_t *)w, ep, partial, n_in, p.n_slices,
-                 p.steps_per_slice, s);
+  const bf16_t *xb = (const bf16_t *)x, *wb = (const bf16_t *)w;
+  if (gated && packed) launch_rt<2, true>(p.R, p.TT, xb, wb, ep, partial, n_in, p.n_slices, p.steps_per_slice, s);
+  else if (gated) launch_rt<2, false>(p.R, p.TT, xb, wb, ep, partial, n_in, p.n_slices, p.steps_per_slice, s);
+  else if (packed) launch_rt<1, true>(p.R, p.TT, xb, wb, ep, partial, n_in, p.n_slices, p.steps_per_slice, s);
+  else launch_rt<1, false>(p.R, p.TT, xb, wb, ep, partial, n_in, p.n_slices, p.steps_per_slice, s);
   int rc = sb::check_launch("sb_gemm_skinny_bf16");
   if (rc != SB_OK) return rc;
   if (p.n_slices > 1) {

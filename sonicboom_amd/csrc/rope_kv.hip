@@ -12,6 +12,8 @@
 
 namespace {
 
+constexpr int kMaxPairs = 256;   // rotated pairs of a head at most (head sizes up to 512)
+
 template <typename TI, typename TQ, typename TC>
 __global__ void __launch_bounds__(256)
 rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_stride,
@@ -42,14 +44,22 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
   }
   const size_t head_step = size_t(SB_PAGE) * head_dim;  // from one kv head to the next within a page
 
-  // Rotated pairs of the query heads and of the key heads.
+  // Rotated pairs of the query heads and of the key heads.  The angle of pair i is the same
+  // for every head of the row: its cosine and sine are computed once and shared.
+  __shared__ float cs[kMaxPairs], sn[kMaxPairs];
   if (inv_freq != nullptr) {
-    const int n_pairs = (heads_q + heads_kv) * half;
-    for (int it = threadIdx.x; it < n_pairs; it += blockDim.x) {
-      const int head = it / half, i = it - head * half;
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
       float theta = float(pos) * inv_freq[i];
       if (freq_factors) theta = theta / freq_factors[i];
-      const float c = cosf(theta), s = sinf(theta);
+      cs[i] = cosf(theta);
+      sn[i] = sinf(theta);
+    }
+    __syncthreads();
+    const int n_pairs = (heads_q + heads_kv) * half;
+#pragma unroll 4
+    for (int it = threadIdx.x; it < n_pairs; it += blockDim.x) {
+      const int head = it / half, i = it - head * half;
+      const float c = cs[i], s = sn[i];
       const size_t e0 = size_t(head) * head_dim + i, e1 = e0 + half;
       const float x0 = ld_f(r, e0), x1 = ld_f(r, e1);
       const float y0 = x0 * c - x1 * s;
@@ -103,10 +113,12 @@ extern "C" int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int q
              (heads_q + 2 * heads_kv) * head_dim);
   SB_REQUIRE(sb::valid_dtype(q_dtype) && sb::valid_dtype(qkv_dtype) && sb::valid_dtype(cache_dtype),
              "sb_rope_kv_store: unknown dtype");
-  if (inv_freq)
+  if (inv_freq) {
     SB_REQUIRE(rot_dims > 0 && rot_dims % 2 == 0 && rot_dims <= head_dim,
                "sb_rope_kv_store: rotary width %d must be even and at most head_dim %d", rot_dims,
                head_dim);
+    SB_SUPPORT(rot_dims / 2 <= kMaxPairs, "sb_rope_kv_store: more than %d rotated pairs per head", kMaxPairs);
+  }
   if (heads_kv > 0)
     SB_REQUIRE(k_cache && v_cache && page_table && row_seq && max_pages > 0 && n_pages_total > 0,
                "sb_rope_kv_store: a layer that stores keys needs a cache and a page table");

@@ -15,30 +15,50 @@ constexpr int kSelThreads = 1024;
 constexpr int kSelWaves = kSelThreads / 64;
 constexpr int kMaxCand = 256;
 
-__global__ void __launch_bounds__(kSelThreads)
-argmax_kernel(int32_t *__restrict__ ids, const float *__restrict__ logits, int vocab) {
-  const float *x = logits + size_t(blockIdx.x) * vocab;
+// Larger value wins; equal values go to the lower index; an index of INT_MAX marks "nothing".
+__device__ __forceinline__ void take_better(float &bv, int &bi, float ov, int oi) {
+  if (oi != 0x7fffffff && (bi == 0x7fffffff || ov > bv || (ov == bv && oi < bi))) {
+    bv = ov;
+    bi = oi;
+  }
+}
+
+constexpr int kArgThreads = 256;
+
+// Stage 1: block (part, row) scans elements [part * span, (part + 1) * span) of its row, four per
+// thread and round, all four loads in flight together.  Stage 2 (n_parts partials per row) runs
+// with span covering the partial arrays.  Within a thread indices ascend, so "first maximum"
+// needs only strict comparison there; across threads take_better breaks ties.
+__global__ void __launch_bounds__(kArgThreads)
+argmax_kernel(int32_t *__restrict__ ids, float *__restrict__ part_val, int32_t *__restrict__ part_idx,
+              const float *__restrict__ vals, const int32_t *__restrict__ idxs, int row_len, int span) {
+  const int row = blockIdx.y, part = blockIdx.x;
+  const float *x = vals + size_t(row) * row_len;
+  const int32_t *xi = idxs ? idxs + size_t(row) * row_len : nullptr;
+  const int begin = part * span, end = min(begin + span, row_len);
   float best_v = -__builtin_inff();
   int best_i = 0x7fffffff;
-  for (int i = threadIdx.x; i < vocab; i += kSelThreads) {
-    const float v = x[i];
-    if (best_i == 0x7fffffff || v > best_v) {
-      best_v = v;
-      best_i = i;
+  for (int i0 = begin + threadIdx.x; i0 < end; i0 += 4 * kArgThreads) {
+    float v[4];
+    int id[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = i0 + u * kArgThreads;
+      const bool ok = i < end;
+      v[u] = ok ? x[i] : -__builtin_inff();
+      id[u] = ok ? (xi ? xi[i] : i) : 0x7fffffff;
     }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) take_better(best_v, best_i, v[u], id[u]);
   }
-  // Larger value wins; equal values go to the lower index.
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     const float ov = __shfl_xor(best_v, off, 64);
     const int oi = __shfl_xor(best_i, off, 64);
-    if (oi != 0x7fffffff && (best_i == 0x7fffffff || ov > best_v || (ov == best_v && oi < best_i))) {
-      best_v = ov;
-      best_i = oi;
-    }
+    take_better(best_v, best_i, ov, oi);
   }
-  __shared__ float wv[kSelWaves];
-  __shared__ int wi[kSelWaves];
+  __shared__ float wv[kArgThreads / 64];
+  __shared__ int wi[kArgThreads / 64];
   if ((threadIdx.x & 63) == 0) {
     wv[threadIdx.x >> 6] = best_v;
     wi[threadIdx.x >> 6] = best_i;
@@ -47,13 +67,13 @@ argmax_kernel(int32_t *__restrict__ ids, const float *__restrict__ logits, int v
   if (threadIdx.x == 0) {
     float bv = wv[0];
     int bi = wi[0];
-    for (int k = 1; k < kSelWaves; ++k) {
-      if (wi[k] != 0x7fffffff && (bi == 0x7fffffff || wv[k] > bv || (wv[k] == bv && wi[k] < bi))) {
-        bv = wv[k];
-        bi = wi[k];
-      }
+    for (int k = 1; k < kArgThreads / 64; ++k) take_better(bv, bi, wv[k], wi[k]);
+    if (ids) {
+      ids[row] = bi == 0x7fffffff ? 0 : bi;
+    } else {
+      part_val[size_t(row) * gridDim.x + part] = bv;
+      part_idx[size_t(row) * gridDim.x + part] = bi;
     }
-    ids[blockIdx.x] = bi == 0x7fffffff ? 0 : bi;
   }
 }
 
@@ -186,12 +206,34 @@ top_candidates_kernel(int32_t *__restrict__ cand_id, float *__restrict__ cand_z,
 
 }  // namespace
 
-extern "C" int sb_argmax(int32_t *ids, const float *logits, int n_rows, int vocab, void *stream) {
+// Parts a row is cut into for the first stage (the second size of the partial buffers).
+extern "C" int sb_argmax_parts(int vocab) {
+  const int parts = (vocab + 4095) / 4096;
+  return parts < 1 ? 1 : (parts > 256 ? 256 : parts);
+}
+
+// part_val float [n_rows * parts], part_idx int32 [n_rows * parts] with parts = sb_argmax_parts(vocab);
+// unused (may be NULL) when parts == 1.
+extern "C" int sb_argmax(int32_t *ids, const float *logits, int n_rows, int vocab, float *part_val,
+                         int32_t *part_idx, void *stream) {
   SB_REQUIRE(ids && logits, "sb_argmax: null pointer");
   SB_REQUIRE(n_rows >= 0 && vocab > 0, "sb_argmax: bad sizes rows=%d vocab=%d", n_rows, vocab);
+  SB_SUPPORT(n_rows <= 65535, "sb_argmax: more than 65535 rows");
   if (n_rows == 0) return SB_OK;
-  argmax_kernel<<<n_rows, kSelThreads, 0, (hipStream_t)stream>>>(ids, logits, vocab);
-  return sb::check_launch("sb_argmax");
+  hipStream_t s = (hipStream_t)stream;
+  const int parts = sb_argmax_parts(vocab);
+  if (parts == 1) {
+    argmax_kernel<<<dim3(1, n_rows), kArgThreads, 0, s>>>(ids, nullptr, nullptr, logits, nullptr, vocab, vocab);
+    return sb::check_launch("sb_argmax");
+  }
+  SB_REQUIRE(part_val && part_idx, "sb_argmax: no buffers for the partial results");
+  const int span = (vocab + parts - 1) / parts;
+  argmax_kernel<<<dim3(parts, n_rows), kArgThreads, 0, s>>>(nullptr, part_val, part_idx, logits, nullptr, vocab,
+                                                            span);
+  int rc = sb::check_launch("sb_argmax");
+  if (rc != SB_OK) return rc;
+  argmax_kernel<<<dim3(1, n_rows), kArgThreads, 0, s>>>(ids, nullptr, nullptr, part_val, part_idx, parts, parts);
+  return sb::check_launch("sb_argmax (second stage)");
 }
 
 extern "C" int sb_penalize(float *logits, int vocab, const int32_t *item_row, const int32_t *item_token,

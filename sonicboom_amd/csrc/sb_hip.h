@@ -99,8 +99,12 @@ int sb_attention(void *out, const void *q, int act_dtype, int q_stride, const vo
                  int n_pages_total, const int32_t *row_pos, const int32_t *row_seq, int n_rows,
                  int heads_q, int heads_kv, int head_dim, float scale, int window, void *stream);
 
-/* ids[r] = index of the first maximum of logits[r,:]. */
-int sb_argmax(int32_t *ids, const float *logits, int n_rows, int vocab, void *stream);
+/* ids[r] = index of the first maximum of logits[r,:].  Two stages over
+ * sb_argmax_parts(vocab) parts of a row; part_val / part_idx hold n_rows * parts
+ * partial results (NULL allowed when parts == 1). */
+int sb_argmax_parts(int vocab);
+int sb_argmax(int32_t *ids, const float *logits, int n_rows, int vocab, float *part_val,
+              int32_t *part_idx, void *stream);
 
 /* Sampling penalties on the logits in place, for `n_items` (row, token, count)
  * triples: v = v>0 ? v/rp : v*rp (when rp != 1), then v -= freq*count + presence.

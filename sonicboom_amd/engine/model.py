@@ -49,6 +49,13 @@ class DecoderModel:
                 if t.name not in shared:
                     tensors.pop(t.name, None)
         self.order = list(spec.order)
+        for e in self.order:
+            mixer = self.blocks[e.block].mixer
+            if e.cache is not None and not e.writes_cache and hasattr(mixer, "query_only"):
+                mixer.query_only()
+        for b in self.blocks:
+            if hasattr(b.mixer, "finish_build"):
+                b.mixer.finish_build()
         # What every cache entry stores, and which order entries want per-sequence state.
         self.cache_specs: Dict[int, tuple] = {}
         self.state_specs: Dict[int, tuple] = {}

@@ -219,7 +219,12 @@ def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Te
     else:
         _i32(out, n, "argmax output")
     lib = library.core()
-    check(lib.sb_argmax(_p(out), _p(logits), n, vocab, _stream()))
+    parts = lib.sb_argmax_parts(vocab)
+    pv = pi = None
+    if parts > 1:
+        pv = torch.empty((n * parts,), dtype=torch.float32, device=logits.device)
+        pi = torch.empty((n * parts,), dtype=torch.int32, device=logits.device)
+    check(lib.sb_argmax(_p(out), _p(logits), n, vocab, _p(pv), _p(pi), _stream()))
     return out
 
 
@@ -258,21 +263,43 @@ def top_candidates(logits: torch.Tensor, temperature: float, k: int = MAX_CANDID
 SKINNY_MAX_ROWS = 64
 
 
+def pack_weight(w: torch.Tensor, gated: bool = False) -> torch.Tensor:
+    """A bf16 projection weight [out, in] in the matrix-core tile layout: rows padded to 16, k to
+    32, and every 16 x 32 tile stored as one 1 KB block in fragment order — lane l = 16 g + r of a
+    wave owns elements [row r][k = 8 g .. 8 g + 7] at offset 8 l — tiles of one row block being
+    consecutive in k.  A wave then reads a whole fragment with one contiguous 1 KB load and walks
+    K through consecutive memory.  With ``gated`` the two halves [gate; up] are packed one after
+    the other.  Returns a flat bf16 tensor."""
+    if w.dim() != 2 or w.dtype != torch.bfloat16:
+        raise KernelLibraryError("pack_weight takes a bfloat16 matrix [out, in]")
+    halves = w.chunk(2, dim=0) if gated else (w,)
+    out = []
+    for h in halves:
+        n, k = h.shape
+        n16, k32 = (n + 15) // 16 * 16, (k + 31) // 32 * 32
+        if (n16, k32) != (n, k):
+            h = torch.nn.functional.pad(h, (0, k32 - k, 0, n16 - n))
+        out.append(h.reshape(n16 // 16, 16, k32 // 32, 4, 8).permute(0, 2, 3, 1, 4).reshape(-1))
+    return torch.cat(out).contiguous() if len(out) > 1 else out[0].contiguous()
+
+
 def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], resid: Optional[torch.Tensor],
-              out_dtype: torch.dtype, out: Optional[torch.Tensor] = None, gated: bool = False
-              ) -> Optional[torch.Tensor]:
+              out_dtype: torch.dtype, out: Optional[torch.Tensor] = None, gated: bool = False,
+              packed_shape=None) -> Optional[torch.Tensor]:
     """bfloat16 product on the matrix cores: y = x w^T (+bias) (+resid), or with ``gated``
     y = silu(x wg^T) * (x wu^T) for w = [wg; wu].  Up to 64 rows go to the weight-streaming
-    kernel, more to the tiled one.  Returns None when the sizes fit neither (an inner size
-    that is not a multiple of 8): the caller then takes the plain kernel."""
+    kernel, more to the tiled one.  ``packed_shape`` = (rows of w, inner size) says that ``w`` is
+    in the layout of :func:`pack_weight`.  Returns None when the sizes fit neither kernel (an
+    inner size that is not a multiple of 8): the caller then takes the plain kernel."""
     _dev(x, w, bias, resid, out)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         return None
-    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
-        raise KernelLibraryError(f"gemm shapes do not match: x {tuple(x.shape)}, w {tuple(w.shape)}")
+    w_rows, w_k = packed_shape if packed_shape is not None else (w.shape[0], w.shape[-1])
+    if x.dim() != 2 or x.shape[1] != w_k or (packed_shape is None and w.dim() != 2):
+        raise KernelLibraryError(f"gemm shapes do not match: x {tuple(x.shape)}, w {(w_rows, w_k)}")
     t, k = x.shape
-    n = w.shape[0] // 2 if gated else w.shape[0]
-    if k % 8 or x.data_ptr() % 16 or w.data_ptr() % 16 or (gated and w.shape[0] % 2):
+    n = w_rows // 2 if gated else w_rows
+    if k % 8 or x.data_ptr() % 16 or w.data_ptr() % 16 or (gated and w_rows % 2):
         return None
     if bias is not None and bias.numel() != n:
         raise KernelLibraryError(f"bias has {bias.numel()} elements, the product has {n} columns")
@@ -284,14 +311,15 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], re
         raise KernelLibraryError("gemm output buffer has the wrong shape or type")
     lib = library.core()
     bdt = _dt(bias) if bias is not None else 0
+    packed = 1 if packed_shape is not None else 0
     if t <= SKINNY_MAX_ROWS:
         need = lib.sb_gemm_skinny_scratch(t, n, k, 1 if gated else 0)
         scratch = torch.empty((need,), dtype=torch.float32, device=x.device) if need else None
         check(lib.sb_gemm_skinny_bf16(_p(out), _dt(out), _p(x), _p(w), _p(bias), bdt, _p(resid), t, n, k,
-                                      1 if gated else 0, _p(scratch), need, _stream()))
+                                      1 if gated else 0, packed, _p(scratch), need, _stream()))
     else:
         check(lib.sb_gemm_mfma_bf16(_p(out), _dt(out), _p(x), _p(w), _p(bias), bdt, _p(resid), t, n, k,
-                                    1 if gated else 0, _stream()))
+                                    1 if gated else 0, packed, _stream()))
     return out
 
 

@@ -27,14 +27,15 @@ _CORE_SIGNATURES = {
     "sb_cast": [_P, _I, _P, _I, _Z, _P],
     "sb_rope_kv_store": [_P, _I, _P, _I, _I, _P, _P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
     "sb_attention": [_P, _P, _I, _I, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _P],
-    "sb_argmax": [_P, _P, _I, _I, _P],
+    "sb_argmax": [_P, _P, _I, _I, _P, _P, _P],
+    "sb_argmax_parts": [_I],
     "sb_penalize": [_P, _I, _P, _P, _P, _I, _F, _F, _F, _I, _P],
     "sb_top_candidates": [_P, _P, _P, _I, _I, _I, _F, _P],
 }
 # Entry points of later kernels; declared when the library has them.
 _OPTIONAL_SIGNATURES = {
-    "sb_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P, _Z, _P],
-    "sb_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P],
+    "sb_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _P, _Z, _P],
+    "sb_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _P],
 }
 _ATTN_SIGNATURES = {
     # out, q, k_cache, v_cache, page_table, max_pages, n_pages, row_pos, part_o, part_ml, n_seqs,

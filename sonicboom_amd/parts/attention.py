@@ -77,9 +77,21 @@ class Attention(Mixer):
             bs = [tensors["q_bias"], tensors["k_bias"], tensors["v_bias"]]
             b_qkv = torch.cat([b.float() for b in bs], dim=0)
         self.qkv = Linear(w_qkv, b_qkv, rt.fast_kernels)
-        self.q_only = Linear(w_qkv[: self.q_width], None if b_qkv is None else b_qkv[: self.q_width],
-                             rt.fast_kernels)
+        # an order entry that reads another entry's cache projects queries only: the model asks for
+        # that projection (query_only) before finish_build() drops the separate query weight
+        self._q_parts = (tensors["q_weight"], None if b_qkv is None else b_qkv[: self.q_width])
+        self._q_only = None
         self.out = Linear(tensors["o_weight"], tensors.get("o_bias"), rt.fast_kernels)
+
+    def query_only(self) -> None:
+        """Build the queries-only projection (for run-order entries that read another entry's cache)."""
+        if self._q_only is None:
+            if self._q_parts is None:
+                raise RuntimeError("the queries-only projection must be asked for while the model is built")
+            self._q_only = Linear(self._q_parts[0], self._q_parts[1], self.rt.fast_kernels)
+
+    def finish_build(self) -> None:
+        self._q_parts = None
 
     def cache_spec(self) -> KVSpec:
         return KVSpec(self.heads_kv, self.head_dim, self.window)
@@ -87,7 +99,9 @@ class Attention(Mixer):
     def forward(self, h, x, ctx, binding) -> None:
         rt = self.rt
         writes = binding.writes_cache
-        proj = self.qkv if writes else self.q_only
+        if not writes:
+            self.query_only()
+        proj = self.qkv if writes else self._q_only
         # q, k, v stay float32 until they have been rotated: one rounding on the way to the cache.
         qkv = proj(h, torch.float32)
         tables = self.position.rotary_tables()

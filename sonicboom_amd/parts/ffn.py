@@ -41,9 +41,9 @@ class GatedDenseFFN(Part):
         g, u = tensors["gate_weight"], tensors["up_weight"]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
-        self.gate_up = Linear(torch.cat([g, u], dim=0), None, rt.fast_kernels)
+        self.gate_up = Linear(torch.cat([g, u], dim=0), None, rt.fast_kernels, gated=True)
         self.down = Linear(tensors["down_weight"], None, rt.fast_kernels)
 
     def forward(self, h, x, ctx) -> None:
-        mid = self.gate_up.gated(h, self.rt.act_dtype)
+        mid = self.gate_up.gated_product(h, self.rt.act_dtype)
         self.down(mid, torch.float32, resid=x, out=x)

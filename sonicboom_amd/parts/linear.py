@@ -5,8 +5,15 @@ call this helper, which picks the kernel from the types and sizes at hand:
 
 * float32 weights (the 32-bit path, or a tensor the file stores in 32-bit):
   the plain kernel, true float32 throughout;
-* bfloat16 weights and activations: the MFMA kernels (a skinny one for a few
-  rows, a tiled one for many) when the sizes fit them, else the plain kernel.
+* bfloat16 weights and activations: the matrix-core kernels (a weight-streaming
+  one for up to 64 rows, a tiled one for more).  For them the weight is
+  re-laid once, when the projection is built, into the tile order the matrix
+  cores read (:func:`sonicboom_amd.ops.pack_weight`) and the row-major copy is
+  dropped.  An inner size that is not a multiple of 8 keeps the row-major
+  weight and the plain kernel.
+
+``gated=True`` marks a stacked weight [W_gate; W_up] whose product is
+silu(x W_gate^T) * (x W_up^T).
 """
 from __future__ import annotations
 
@@ -18,33 +25,52 @@ from .. import ops
 
 
 class Linear:
-    def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor], fast: bool = True):
+    def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor], fast: bool = True,
+                 gated: bool = False):
         if weight.dim() != 2:
             raise ValueError("a projection weight must be [out, in]")
-        if bias is not None and bias.numel() != weight.shape[0]:
-            raise ValueError(f"bias has {bias.numel()} elements, the projection has {weight.shape[0]} outputs")
-        self.weight = weight.contiguous()
+        self.gated = gated
+        self.rows, self.n_in = weight.shape
+        self.n_out = self.rows // 2 if gated else self.rows
+        if gated and self.rows % 2:
+            raise ValueError("a gated projection stacks two matrices of equal height")
+        if bias is not None and bias.numel() != self.n_out:
+            raise ValueError(f"bias has {bias.numel()} elements, the projection has {self.n_out} outputs")
         self.bias = None if bias is None else bias.contiguous()
-        self.fast = fast
-        self.n_out, self.n_in = weight.shape
+        self.packed = None
+        self.weight = weight.contiguous()
+        if fast and weight.is_cuda and weight.dtype == torch.bfloat16 and self.n_in % 8 == 0:
+            self.packed = ops.pack_weight(self.weight, gated)
+            self.weight = None
+
+    def _row_major(self) -> torch.Tensor:
+        if self.weight is None:
+            raise RuntimeError("this projection only keeps its packed weight")
+        return self.weight
 
     def __call__(self, x: torch.Tensor, out_dtype: torch.dtype, resid: Optional[torch.Tensor] = None,
                  out: Optional[torch.Tensor] = None) -> torch.Tensor:
-        w = self.weight
+        if self.gated:
+            return self.gated_product(x, out_dtype)
+        if self.packed is not None:
+            if x.dtype != torch.bfloat16:
+                x = ops.cast(x, torch.bfloat16)
+            return ops.gemm_bf16(x, self.packed, self.bias, resid, out_dtype, out,
+                                 packed_shape=(self.rows, self.n_in))
+        w = self._row_major()
         if w.dtype == torch.float32 and x.dtype != torch.float32:
             x = ops.cast(x, torch.float32)
-        if self.fast and w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
-            y = ops.gemm_bf16(x, w, self.bias, resid, out_dtype, out)
-            if y is not None:
-                return y
         return ops.gemm_plain(x, w, self.bias, resid, out_dtype, out)
 
-    def gated(self, x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-        """silu(x Wg^T) * (x Wu^T) for a stacked weight [Wg; Wu]: one fused kernel on the
-        matrix cores when the sizes allow, else the product in float32 and the activation kernel."""
-        w = self.weight
-        if self.fast and w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
-            y = ops.gemm_bf16(x, w, None, None, out_dtype, gated=True)
-            if y is not None:
-                return y
-        return ops.silu_mul(self(x, torch.float32), out_dtype)
+    def gated_product(self, x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+        """silu(x Wg^T) * (x Wu^T): one fused kernel on the matrix cores, or the product in
+        float32 followed by the activation kernel."""
+        if self.packed is not None:
+            if x.dtype != torch.bfloat16:
+                x = ops.cast(x, torch.bfloat16)
+            return ops.gemm_bf16(x, self.packed, None, None, out_dtype, gated=True,
+                                 packed_shape=(self.rows, self.n_in))
+        w = self._row_major()
+        if w.dtype == torch.float32 and x.dtype != torch.float32:
+            x = ops.cast(x, torch.float32)
+        return ops.silu_mul(ops.gemm_plain(x, w, None, None, torch.float32), out_dtype)
