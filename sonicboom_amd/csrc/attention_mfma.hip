@@ -83,73 +83,110 @@ __device__ __forceinline__ uint4 drop_first(uint4 v, int n_drop) {
   return make_uint4(w[0], w[1], w[2], w[3]);
 }
 
-// One page (64 keys at absolute positions page_pos .. page_pos+63) for the wave's 16 columns.
-// qf: the columns' query fragments; col_pos / col_lo: last and first visible key of this lane's
-// column (col_pos < 0: the column is empty).  key_hi / key_lo: the same over all columns of the
-// wave (uniform), used to skip work and to decide whether values need masking.
+// The fragments of one half page (32 keys): keys for both score tiles, values for all d tiles.
+struct HalfPage {
+  uint4 k[2][KS];
+  uint4 v[DT];
+};
+
+__device__ __forceinline__ void load_half(HalfPage &hp, const bf16_t *__restrict__ kp,
+                                          const bf16_t *__restrict__ vp, int half, int lane) {
+  const int r = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    // A row r = 4 gg + i of score tile t is key 8 gg + 4 t + i of the 32
+    const int key = 32 * half + 8 * (r >> 2) + 4 * t + (r & 3);
+    const bf16_t *krow = kp + size_t(key) * HD;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 32 + g * 8;
+      hp.k[t][ks] = ld16(krow + d, d < HD);
+    }
+  }
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) hp.v[dt] = ld16(vp + size_t(dt * 16 + r) * SB_PAGE + 32 * half + 8 * g, true);
+}
+
+// 32 keys at absolute positions base .. base+31, their fragments in hp, for the wave's 16 columns.
+// col_pos / col_lo: last and first visible key of this lane's column (col_pos < 0: the column is
+// empty).  key_hi / key_lo: the same over all columns of the wave (uniform).
+__device__ __forceinline__ void attend_half(WaveState &st, const bf16x8_t (&qf)[KS], const HalfPage &hp,
+                                            int base, int col_pos, int col_lo, int key_lo, int key_hi,
+                                            float scale_log2, int lane) {
+  const int g = lane >> 4;
+  floatx4_t s[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    s[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) s[t] = mfma16(as_bf16x8(hp.k[t][ks]), qf[ks], s[t]);
+  }
+  // this lane: column lane % 16, keys base + 8 g + e, e = 0..7 (s[0] holds e = 0..3, s[1] e = 4..7)
+  float sc[8];
+  float mx = -__builtin_inff();
+  const int k0 = base + 8 * g;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const int j = k0 + e;
+    const bool vis = j <= col_pos && j >= col_lo;
+    const float v = (e < 4 ? s[0][e] : s[1][e - 4]) * scale_log2;
+    sc[e] = vis ? v : -__builtin_inff();
+    mx = fmaxf(mx, sc[e]);
+  }
+  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+  const float m_new = fmaxf(st.m, mx);
+  // a column that has seen no key yet keeps m = -inf: give it a finite stand-in
+  const float m_use = m_new == -__builtin_inff() ? 0.f : m_new;
+  const float alpha = __builtin_amdgcn_exp2f(st.m - m_use);   // st.m = -inf gives 0
+  float p[8];
+  float psum = 0.f;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    p[e] = __builtin_amdgcn_exp2f(sc[e] - m_use);             // -inf gives 0
+    psum += p[e];
+  }
+  st.l = st.l * alpha + psum;
+  st.m = m_new;
+  const uint4 pb = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]),
+                              pack_bf16(p[6], p[7]));
+  // values of keys outside [key_lo, key_hi] may be stale or never written: 0 * garbage must not
+  // reach the accumulator, so such keys are cut out of the V fragment as well
+  const bool cut_hi = base + 31 > key_hi, cut_lo = base < key_lo;
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    uint4 a = hp.v[dt];
+    if (cut_hi) a = keep_first(a, key_hi - k0 + 1);
+    if (cut_lo) a = drop_first(a, key_lo - k0);
+    floatx4_t acc = st.o[dt];
+    acc[0] *= alpha; acc[1] *= alpha; acc[2] *= alpha; acc[3] *= alpha;
+    st.o[dt] = mfma16(as_bf16x8(a), as_bf16x8(pb), acc);
+  }
+}
+
+// One page (64 keys at absolute positions page_pos .. page_pos+63): both halves' fragments are
+// requested before the first product, so a page costs one round trip to memory.
 __device__ __forceinline__ void attend_page(WaveState &st, const bf16x8_t (&qf)[KS],
                                             const bf16_t *__restrict__ kp, const bf16_t *__restrict__ vp,
                                             int page_pos, int col_pos, int col_lo, int key_lo, int key_hi,
                                             float scale_log2, int lane) {
-  const int r = lane & 15, g = lane >> 4;
-#pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    const int base = page_pos + 32 * half;
-    if (base > key_hi || base + 31 < key_lo) continue;   // uniform: nothing visible in these 32 keys
-    floatx4_t s[2];
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      s[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-      // A row r = 4 gg + i is key 8 gg + 4 t + i of the 32
-      const int key = 32 * half + 8 * (r >> 2) + 4 * t + (r & 3);
-      const bf16_t *krow = kp + size_t(key) * HD;
-#pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int d = ks * 32 + g * 8;
-        const uint4 a = ld16(krow + d, d < HD);
-        s[t] = mfma16(as_bf16x8(a), qf[ks], s[t]);
-      }
+  const bool use0 = !(page_pos > key_hi || page_pos + 31 < key_lo);
+  const bool use1 = !(page_pos + 32 > key_hi || page_pos + 63 < key_lo);
+  if (HD <= 128) {
+    HalfPage h0, h1;
+    if (use0) load_half(h0, kp, vp, 0, lane);
+    if (use1) load_half(h1, kp, vp, 1, lane);
+    if (use0) attend_half(st, qf, h0, page_pos, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
+    if (use1) attend_half(st, qf, h1, page_pos + 32, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
+  } else {
+    HalfPage h;
+    if (use0) {
+      load_half(h, kp, vp, 0, lane);
+      attend_half(st, qf, h, page_pos, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
     }
-    // this lane: column r, keys base + 8 g + e, e = 0..7 (s[0] holds e = 0..3, s[1] e = 4..7)
-    float sc[8];
-    float mx = -__builtin_inff();
-    const int k0 = base + 8 * g;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const int j = k0 + e;
-      const bool vis = j <= col_pos && j >= col_lo;
-      const float v = (e < 4 ? s[0][e] : s[1][e - 4]) * scale_log2;
-      sc[e] = vis ? v : -__builtin_inff();
-      mx = fmaxf(mx, sc[e]);
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(st.m, mx);
-    // a column that has seen no key yet keeps m = -inf: give it a finite stand-in
-    const float m_use = m_new == -__builtin_inff() ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(st.m - m_use);   // st.m = -inf gives 0
-    float p[8];
-    float psum = 0.f;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      p[e] = __builtin_amdgcn_exp2f(sc[e] - m_use);             // -inf gives 0
-      psum += p[e];
-    }
-    st.l = st.l * alpha + psum;
-    st.m = m_new;
-    const uint4 pb = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]),
-                                pack_bf16(p[6], p[7]));
-    // values of keys outside [key_lo, key_hi] may be stale or never written: 0 * garbage must not
-    // reach the accumulator, so such keys are cut out of the V fragment as well
-    const bool cut_hi = base + 31 > key_hi, cut_lo = base < key_lo;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-      uint4 a = ld16(vp + size_t(dt * 16 + r) * SB_PAGE + 32 * half + 8 * g, true);
-      if (cut_hi) a = keep_first(a, key_hi - k0 + 1);
-      if (cut_lo) a = drop_first(a, key_lo - k0);
-      floatx4_t acc = st.o[dt];
-      acc[0] *= alpha; acc[1] *= alpha; acc[2] *= alpha; acc[3] *= alpha;
-      st.o[dt] = mfma16(as_bf16x8(a), as_bf16x8(pb), acc);
+    if (use1) {
+      load_half(h, kp, vp, 1, lane);
+      attend_half(st, qf, h, page_pos + 32, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
     }
   }
 }

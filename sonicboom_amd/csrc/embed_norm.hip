@@ -22,13 +22,44 @@ __global__ void embed_kernel(float *__restrict__ out, const TT *__restrict__ tab
   for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = ld_f(src, i);
 }
 
-constexpr int kNormThreads = 256;
-constexpr int kNormKeep = 8;   // float4 groups of a row that a thread keeps in registers
+constexpr int kNormThreads = 1024;
+constexpr int kNormWaves = kNormThreads / 64;
+constexpr int kNormKeep = 2;   // float4 groups of a row that a thread keeps in registers
+constexpr int kMaxSlices = 8;  // K slices of a product that the fused kernel adds
 
-// One block per row.  A thread takes float4 groups tid, tid + 256, ...; all of a thread's loads
-// are issued before the first is used, and the first kNormKeep groups stay in registers for the
-// second pass.  The squares are summed in double: per thread in ascending order, then by a
-// fixed butterfly over the wave, then wave by wave.
+// Sum of the squares of a block's kept values: per thread in ascending order, a fixed butterfly
+// over the wave, then wave by wave in ascending order; all in double
+// (/root/reference/core/src/nn/cpu_reduce.h:55-57 sums float products in double).
+__device__ __forceinline__ double block_sum(double part) {
+  __shared__ double wave_part[kNormWaves];
+  part = wave_sum(part);
+  if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = part;
+  __syncthreads();
+  double total = 0.0;
+#pragma unroll
+  for (int k = 0; k < kNormWaves; ++k) total += wave_part[k];
+  return total;
+}
+
+__device__ __forceinline__ double squares(const float4 &v) {
+  return double(v.x * v.x) + double(v.y * v.y) + double(v.z * v.z) + double(v.w * v.w);
+}
+
+template <typename TO>
+__device__ __forceinline__ void write_normed(TO *yr, const float4 &v, int g, float inv, const void *w, int w_dtype) {
+  const float x[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    float o = x[e] * inv;
+    if (w) o = o * ld_dyn(w, w_dtype, g * 4 + e);
+    st_f(yr, g * 4 + e, o);
+  }
+}
+
+// One block per row.  A thread takes float4 groups tid and tid + 1024; its loads are issued
+// unconditionally (from a clamped address) so that all are in flight together, and the groups
+// stay in registers for the second pass.  Rows wider than 8192, or not readable in groups of
+// four, go through the scalar tail loops.
 template <typename TO>
 __global__ void __launch_bounds__(kNormThreads)
 rmsnorm_kernel(TO *__restrict__ y, const float *__restrict__ x, const void *__restrict__ w,
@@ -43,43 +74,26 @@ rmsnorm_kernel(TO *__restrict__ y, const float *__restrict__ x, const void *__re
 
   float4 keep[kNormKeep];
   double part = 0.0;
+  if (n_groups > 0) {
 #pragma unroll
-  for (int i = 0; i < kNormKeep; ++i) {
-    const int g = tid + i * kNormThreads;
-    keep[i] = g < n_groups ? reinterpret_cast<const float4 *>(xr)[g] : make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int i = 0; i < kNormKeep; ++i)
+      keep[i] = reinterpret_cast<const float4 *>(xr)[min(tid + i * kNormThreads, n_groups - 1)];
+#pragma unroll
+    for (int i = 0; i < kNormKeep; ++i)
+      if (tid + i * kNormThreads < n_groups) part += squares(keep[i]);
   }
-#pragma unroll
-  for (int i = 0; i < kNormKeep; ++i)
-    part += double(keep[i].x * keep[i].x) + double(keep[i].y * keep[i].y) + double(keep[i].z * keep[i].z) +
-            double(keep[i].w * keep[i].w);
-  // what does not fit the registers, or a row that cannot be read in groups of four
-  const int tail0 = vec ? min(n_groups, kNormKeep * kNormThreads) * 4 : 0;
+  const int tail0 = min(n_groups, kNormKeep * kNormThreads) * 4;
   for (int i = tail0 + tid; i < width; i += kNormThreads) {
     const float v = xr[i];
     part += double(v * v);
   }
-  part = wave_sum(part);
-  __shared__ double wave_part[kNormThreads / 64];
-  if ((tid & 63) == 0) wave_part[tid >> 6] = part;
-  __syncthreads();
-  double total = 0.0;
-#pragma unroll
-  for (int k = 0; k < kNormThreads / 64; ++k) total += wave_part[k];
+  const double total = block_sum(part);
   const float mean = float(total / double(width));
   const float inv = 1.0f / sqrtf(mean + eps);
-
 #pragma unroll
   for (int i = 0; i < kNormKeep; ++i) {
     const int g = tid + i * kNormThreads;
-    if (g < n_groups) {
-      const float v[4] = {keep[i].x, keep[i].y, keep[i].z, keep[i].w};
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        float o = v[e] * inv;
-        if (w) o = o * ld_dyn(w, w_dtype, g * 4 + e);
-        st_f(yr, g * 4 + e, o);
-      }
-    }
+    if (g < n_groups) write_normed(yr, keep[i], g, inv, w, w_dtype);
   }
   for (int i = tail0 + tid; i < width; i += kNormThreads) {
     float o = xr[i] * inv;
@@ -88,7 +102,90 @@ rmsnorm_kernel(TO *__restrict__ y, const float *__restrict__ x, const void *__re
   }
 }
 
+// x[t,:] += sum_s partial[s][t][:] (+ bias), then optionally y[t,:] = rmsnorm(x[t,:]) * w.
+// The slices are added in ascending order, then the bias, then the residual: the order of the
+// unfused kernels (product, bias, residual).  width % 4 == 0 and width <= 8192 (host-checked).
+template <typename TO>
+__global__ void __launch_bounds__(kNormThreads)
+reduce_resid_norm_kernel(TO *__restrict__ y, float *__restrict__ x, const float *__restrict__ partial,
+                         int n_slices, size_t slice_stride, const void *__restrict__ bias, int bias_dtype,
+                         const void *__restrict__ w, int w_dtype, int width, float eps, int do_norm) {
+  const int r = blockIdx.x;
+  float *xr = x + size_t(r) * width;
+  const float *pr = partial + size_t(r) * width;
+  const int tid = threadIdx.x;
+  const int n_groups = width / 4;
+
+  float4 keep[kNormKeep];
+  double part = 0.0;
+#pragma unroll
+  for (int i = 0; i < kNormKeep; ++i) {
+    const int g = tid + i * kNormThreads;
+    const int gc = min(g, n_groups - 1);
+    float4 p[kMaxSlices];
+#pragma unroll
+    for (int s = 0; s < kMaxSlices; ++s)
+      p[s] = reinterpret_cast<const float4 *>(pr + min(s, n_slices - 1) * slice_stride)[gc];
+    const float4 old = reinterpret_cast<const float4 *>(xr)[gc];
+    float4 acc = p[0];
+#pragma unroll
+    for (int s = 1; s < kMaxSlices; ++s)
+      if (s < n_slices) { acc.x += p[s].x; acc.y += p[s].y; acc.z += p[s].z; acc.w += p[s].w; }
+    if (bias) {
+      acc.x += ld_dyn(bias, bias_dtype, gc * 4 + 0); acc.y += ld_dyn(bias, bias_dtype, gc * 4 + 1);
+      acc.z += ld_dyn(bias, bias_dtype, gc * 4 + 2); acc.w += ld_dyn(bias, bias_dtype, gc * 4 + 3);
+    }
+    acc.x += old.x; acc.y += old.y; acc.z += old.z; acc.w += old.w;
+    if (g < n_groups) {
+      reinterpret_cast<float4 *>(xr)[g] = acc;
+      part += squares(acc);
+    }
+    keep[i] = acc;
+  }
+  if (!do_norm) return;
+  const double total = block_sum(part);
+  const float mean = float(total / double(width));
+  const float inv = 1.0f / sqrtf(mean + eps);
+  TO *yr = y + size_t(r) * width;
+#pragma unroll
+  for (int i = 0; i < kNormKeep; ++i) {
+    const int g = tid + i * kNormThreads;
+    if (g < n_groups) write_normed(yr, keep[i], g, inv, w, w_dtype);
+  }
+}
+
 }  // namespace
+
+// The widest row sb_reduce_resid_norm takes.
+extern "C" int sb_reduce_resid_norm_max_width(void) { return 4 * kNormKeep * kNormThreads; }
+
+// x[t,:] += sum over slices of partial[s][t][:] (+ bias); with do_norm also
+// y[t,:] = (x[t,:] * inv) * w in y_dtype.  partial is float [n_slices][n_rows][width].
+extern "C" int sb_reduce_resid_norm(void *y, int y_dtype, float *x, const float *partial, int n_slices,
+                                    const void *bias, int bias_dtype, const void *w, int w_dtype,
+                                    int n_rows, int width, float eps, int do_norm, void *stream) {
+  SB_REQUIRE(x && partial && (!do_norm || y), "sb_reduce_resid_norm: null pointer");
+  SB_REQUIRE(n_rows >= 0 && width > 0 && n_slices >= 1, "sb_reduce_resid_norm: bad sizes");
+  SB_SUPPORT(n_slices <= kMaxSlices, "sb_reduce_resid_norm: %d slices, at most %d", n_slices, kMaxSlices);
+  SB_REQUIRE((!do_norm || sb::valid_dtype(y_dtype)) && (!bias || sb::valid_dtype(bias_dtype)) &&
+                 (!w || sb::valid_dtype(w_dtype)),
+             "sb_reduce_resid_norm: unknown dtype");
+  SB_SUPPORT(width % 4 == 0 && width <= sb_reduce_resid_norm_max_width(),
+             "sb_reduce_resid_norm: width %d must be a multiple of 4 and at most %d", width,
+             sb_reduce_resid_norm_max_width());
+  SB_SUPPORT((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(partial)) % 16 == 0,
+             "sb_reduce_resid_norm: operands must be 16-byte aligned");
+  if (n_rows == 0) return SB_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const size_t stride = size_t(n_rows) * width;
+  if (!do_norm || y_dtype == SB_F32)
+    reduce_resid_norm_kernel<float><<<n_rows, kNormThreads, 0, s>>>(
+        (float *)y, x, partial, n_slices, stride, bias, bias_dtype, w, w_dtype, width, eps, do_norm);
+  else
+    reduce_resid_norm_kernel<bf16_t><<<n_rows, kNormThreads, 0, s>>>(
+        (bf16_t *)y, x, partial, n_slices, stride, bias, bias_dtype, w, w_dtype, width, eps, do_norm);
+  return sb::check_launch("sb_reduce_resid_norm");
+}
 
 extern "C" int sb_embed(float *out, const void *table, int table_dtype, const int32_t *ids,
                         int n_rows, int width, int vocab, void *stream) {

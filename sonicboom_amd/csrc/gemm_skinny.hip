@@ -229,7 +229,9 @@ Plan plan_for(int n_rows, int n_out, int n_in, int gated) {
   Plan p;
   p.TT = n_rows <= 16 ? 1 : (n_rows <= 32 ? 2 : 4);
   const int tiles = (n_out + 15) / 16;
-  p.R = tiles >= 2048 ? 4 : (tiles >= 1024 ? 2 : 1);
+  // measured on MI355X: one row tile per block streams best up to 16 rows; more rows reuse each
+  // X fragment for several row tiles
+  p.R = p.TT == 1 ? 1 : (tiles >= 2048 ? 4 : (tiles >= 1024 ? 2 : 1));
   if (gated && p.R == 4) p.R = 2;   // gate and up double the fragments a wave holds
   if (g_force_r) p.R = g_force_r;
   const int blocks = (tiles + p.R - 1) / p.R;
@@ -239,6 +241,7 @@ Plan plan_for(int n_rows, int n_out, int n_in, int gated) {
     slices = (1024 + blocks - 1) / blocks;
     const int most = n_steps / (kWaves * 4);   // every wave keeps at least four steps
     if (slices > most) slices = most;
+    if (slices > 8) slices = 8;     // what the kernels that add the slices take
     if (slices < 1) slices = 1;
   }
   if (g_force_slices) slices = g_force_slices;
@@ -299,4 +302,31 @@ extern "C" int sb_gemm_skinny_bf16(void *y, int y_dtype, const void *x, const vo
     rc = sb::check_launch("sb_gemm_skinny_bf16 (slice sum)");
   }
   return rc;
+}
+
+// K slices sb_gemm_skinny_partial_bf16 will produce for these sizes.
+extern "C" int sb_gemm_skinny_slices(int n_rows, int n_out, int n_in) {
+  if (n_rows <= 0 || n_out <= 0 || n_in <= 0) return 1;
+  return plan_for(n_rows, n_out, n_in, 0).n_slices;
+}
+
+// The raw product in K slices, for a consumer that adds them (and bias, residual, ...) itself:
+// partial float [slices][n_rows][n_out], slices = sb_gemm_skinny_slices(...), slice s holding
+// sum over its k range of X[t,k] W[n,k].
+extern "C" int sb_gemm_skinny_partial_bf16(float *partial, const void *x, const void *w, int n_rows,
+                                           int n_out, int n_in, int packed, void *stream) {
+  SB_REQUIRE(partial && x && w, "sb_gemm_skinny_partial_bf16: null pointer");
+  SB_REQUIRE(n_rows >= 0 && n_out > 0 && n_in > 0, "sb_gemm_skinny_partial_bf16: bad sizes");
+  SB_SUPPORT(n_rows <= 64, "sb_gemm_skinny_partial_bf16: %d rows, at most 64", n_rows);
+  SB_SUPPORT(n_in % 8 == 0, "sb_gemm_skinny_partial_bf16: inner size %d is not a multiple of 8", n_in);
+  SB_SUPPORT((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) % 16 == 0,
+             "sb_gemm_skinny_partial_bf16: operands must be 16-byte aligned");
+  if (n_rows == 0) return SB_OK;
+  const Plan p = plan_for(n_rows, n_out, n_in, 0);
+  Epilogue ep{nullptr, SB_F32, nullptr, 0, nullptr, n_rows, n_out, 0};
+  const bf16_t *xb = (const bf16_t *)x, *wb = (const bf16_t *)w;
+  hipStream_t s = (hipStream_t)stream;
+  if (packed) launch_rt<1, true>(p.R, p.TT, xb, wb, ep, partial, n_in, p.n_slices, p.steps_per_slice, s);
+  else launch_rt<1, false>(p.R, p.TT, xb, wb, ep, partial, n_in, p.n_slices, p.steps_per_slice, s);
+  return sb::check_launch("sb_gemm_skinny_partial_bf16");
 }

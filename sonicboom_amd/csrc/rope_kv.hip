@@ -13,10 +13,31 @@
 namespace {
 
 constexpr int kMaxPairs = 256;   // rotated pairs of a head at most (head sizes up to 512)
+constexpr int kMaxSlices = 8;    // K slices of the projection that are added on load
 
+// Element e of a qkv row: the sum of the product's K slices in ascending order, then the bias.
+template <typename TI>
+__device__ __forceinline__ float qkv_at(const TI *r, size_t e, int n_slices, size_t slice_stride,
+                                        const float *bias) {
+  float p[kMaxSlices];
+#pragma unroll
+  for (int s = 0; s < kMaxSlices; ++s) p[s] = s < n_slices ? ld_f(r + s * slice_stride, e) : 0.f;
+  float v = p[0];
+#pragma unroll
+  for (int s = 1; s < kMaxSlices; ++s)
+    if (s < n_slices) v += p[s];
+  if (bias) v = v + bias[e];
+  return v;
+}
+
+constexpr int kHeadsPerBlock = 4;
+
+// Block (row, head group): heads [4 y, 4 y + 4) of the row's heads_q query heads, heads_kv key
+// heads and heads_kv value heads, in that order.
 template <typename TI, typename TQ, typename TC>
 __global__ void __launch_bounds__(256)
-rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_stride,
+rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_stride, int n_slices,
+               size_t slice_stride, const float *__restrict__ bias,
                const float *__restrict__ inv_freq, const float *__restrict__ freq_factors,
                int rot_dims, const int32_t *__restrict__ row_pos,
                const int32_t *__restrict__ row_seq, TC *__restrict__ k_cache,
@@ -27,11 +48,11 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
   const TI *r = qkv + size_t(row) * row_stride;
   const int half = rot_dims / 2;
   const int q_width = heads_q * head_dim;
-  const int kv_width = heads_kv * head_dim;
   TQ *qo = q_out + size_t(row) * q_width;
+  const int n_heads = heads_q + 2 * heads_kv;
+  const int h_begin = blockIdx.y * kHeadsPerBlock, h_end = min(h_begin + kHeadsPerBlock, n_heads);
 
   // Where this row's key and value go.
-  size_t slot_base = 0;
   int page_of_row = 0;
   bool store = heads_kv > 0;
   if (store) {
@@ -40,65 +61,73 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
     const int page = (lp >= 0 && lp < max_pages) ? page_table[size_t(seq) * max_pages + lp] : -1;
     if (page < 0 || page >= n_pages_total) store = false;  // refused on the host; never write astray
     page_of_row = page < 0 ? 0 : page;
-    slot_base = (size_t(page < 0 ? 0 : page) * heads_kv * SB_PAGE + size_t(pos % SB_PAGE)) * head_dim;
   }
   const size_t head_step = size_t(SB_PAGE) * head_dim;  // from one kv head to the next within a page
+  const size_t page_base = size_t(page_of_row) * heads_kv * head_step;
+  const size_t k_base = page_base + size_t(pos % SB_PAGE) * head_dim;   // keys   [position][d]
+  const size_t v_base = page_base + size_t(pos % SB_PAGE);              // values [d][position]
 
-  // Rotated pairs of the query heads and of the key heads.  The angle of pair i is the same
-  // for every head of the row: its cosine and sine are computed once and shared.
+  // The angle of pair i is the same for every head of the row: cosine and sine once per block.
   __shared__ float cs[kMaxPairs], sn[kMaxPairs];
-  if (inv_freq != nullptr) {
+  const bool rotate = inv_freq != nullptr;
+  if (rotate && h_begin < heads_q + heads_kv) {
     for (int i = threadIdx.x; i < half; i += blockDim.x) {
       float theta = float(pos) * inv_freq[i];
       if (freq_factors) theta = theta / freq_factors[i];
       cs[i] = cosf(theta);
       sn[i] = sinf(theta);
     }
-    __syncthreads();
-    const int n_pairs = (heads_q + heads_kv) * half;
-#pragma unroll 4
-    for (int it = threadIdx.x; it < n_pairs; it += blockDim.x) {
-      const int head = it / half, i = it - head * half;
-      const float c = cs[i], s = sn[i];
-      const size_t e0 = size_t(head) * head_dim + i, e1 = e0 + half;
-      const float x0 = ld_f(r, e0), x1 = ld_f(r, e1);
-      const float y0 = x0 * c - x1 * s;
-      const float y1 = x0 * s + x1 * c;
-      if (head < heads_q) {
-        st_f(qo, e0, y0);
-        st_f(qo, e1, y1);
-      } else if (store) {
-        const int kh = head - heads_q;
-        st_f(k_cache, slot_base + kh * head_step + i, y0);
-        st_f(k_cache, slot_base + kh * head_step + i + half, y1);
-      }
-    }
   }
-  // Elements that do not rotate (all of them without a table).
-  const int first_plain = inv_freq ? rot_dims : 0;
+  __syncthreads();
+  const int first_plain = rotate ? rot_dims : 0;
   const int plain = head_dim - first_plain;
-  for (int it = threadIdx.x; it < heads_q * plain; it += blockDim.x) {
-    const int h = it / plain, d = first_plain + (it - h * plain);
-    st_f(qo, size_t(h) * head_dim + d, ld_f(r, size_t(h) * head_dim + d));
-  }
-  if (!store) return;
-  for (int it = threadIdx.x; it < heads_kv * plain; it += blockDim.x) {
-    const int kh = it / plain, d = first_plain + (it - kh * plain);
-    st_f(k_cache, slot_base + kh * head_step + d, ld_f(r, size_t(q_width) + kh * head_dim + d));
-  }
-  // Values: the cache keeps them transposed, [d][position in page], so that the matrix-core
-  // kernels read eight consecutive keys of one d with one 16-byte load.
-  const size_t v_base = size_t(page_of_row) * heads_kv * head_step + size_t(pos % SB_PAGE);
-  for (int it = threadIdx.x; it < kv_width; it += blockDim.x) {
-    const int kh = it / head_dim, d = it - kh * head_dim;
-    st_f(v_cache, v_base + kh * head_step + size_t(d) * SB_PAGE, ld_f(r, size_t(q_width) + kv_width + it));
+  // work items of a head: `half` rotated pairs, then `plain` elements that are copied
+  const int per_head = (rotate ? half : 0) + plain;
+  const int n_items = (h_end - h_begin) * per_head;
+#pragma unroll 2
+  for (int it = threadIdx.x; it < n_items; it += blockDim.x) {
+    const int head = h_begin + it / per_head, w = it % per_head;
+    const size_t hoff = size_t(head) * head_dim;      // heads lie back to back in the qkv row
+    if (head >= heads_q + heads_kv) {
+      // a value head: every element is copied, transposed into the page
+      if (!store) continue;
+      const int kh = head - heads_q - heads_kv;
+#pragma unroll 1
+      for (int d = w; d < head_dim; d += per_head)
+        st_f(v_cache, v_base + kh * head_step + size_t(d) * SB_PAGE,
+             qkv_at(r, hoff + d, n_slices, slice_stride, bias));
+      continue;
+    }
+    const bool is_q = head < heads_q;
+    if (!is_q && !store) continue;
+    const int kh = head - heads_q;
+    if (rotate && w < half) {
+      const int i = w;
+      const float c = cs[i], sv = sn[i];
+      const float x0 = qkv_at(r, hoff + i, n_slices, slice_stride, bias);
+      const float x1 = qkv_at(r, hoff + i + half, n_slices, slice_stride, bias);
+      const float y0 = x0 * c - x1 * sv;
+      const float y1 = x0 * sv + x1 * c;
+      if (is_q) {
+        st_f(qo, hoff + i, y0);
+        st_f(qo, hoff + i + half, y1);
+      } else {
+        st_f(k_cache, k_base + kh * head_step + i, y0);
+        st_f(k_cache, k_base + kh * head_step + i + half, y1);
+      }
+    } else {
+      const int d = first_plain + (w - (rotate ? half : 0));
+      const float v = qkv_at(r, hoff + d, n_slices, slice_stride, bias);
+      if (is_q) st_f(qo, hoff + d, v);
+      else st_f(k_cache, k_base + kh * head_step + d, v);
+    }
   }
 }
 
 }  // namespace
 
 extern "C" int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int qkv_dtype,
-                                int row_stride, const float *inv_freq, const float *freq_factors,
+                                int row_stride, int n_slices, const float *bias, const float *inv_freq, const float *freq_factors,
                                 int rot_dims, const int32_t *row_pos, const int32_t *row_seq,
                                 void *k_cache, void *v_cache, int cache_dtype,
                                 const int32_t *page_table, int max_pages, int n_pages_total,
@@ -113,6 +142,9 @@ extern "C" int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int q
              (heads_q + 2 * heads_kv) * head_dim);
   SB_REQUIRE(sb::valid_dtype(q_dtype) && sb::valid_dtype(qkv_dtype) && sb::valid_dtype(cache_dtype),
              "sb_rope_kv_store: unknown dtype");
+  SB_REQUIRE(n_slices >= 1, "sb_rope_kv_store: at least one slice");
+  SB_SUPPORT(n_slices <= kMaxSlices, "sb_rope_kv_store: %d slices, at most %d", n_slices, kMaxSlices);
+  const size_t slice_stride = size_t(n_rows) * row_stride;
   if (inv_freq) {
     SB_REQUIRE(rot_dims > 0 && rot_dims % 2 == 0 && rot_dims <= head_dim,
                "sb_rope_kv_store: rotary width %d must be even and at most head_dim %d", rot_dims,
@@ -124,9 +156,12 @@ extern "C" int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int q
                "sb_rope_kv_store: a layer that stores keys needs a cache and a page table");
   if (n_rows == 0) return SB_OK;
   hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(n_rows, (heads_q + 2 * heads_kv + kHeadsPerBlock - 1) / kHeadsPerBlock);
+  SB_SUPPORT(grid.y <= 65535, "sb_rope_kv_store: too many heads");
 #define SB_GO(TI, TQ, TC)                                                                        \
-  rope_kv_kernel<TI, TQ, TC><<<n_rows, 256, 0, s>>>(                                              \
-      (TQ *)q_out, (const TI *)qkv, row_stride, inv_freq, freq_factors, rot_dims, row_pos, row_seq, \
+  rope_kv_kernel<TI, TQ, TC><<<grid, 256, 0, s>>>(                                              \
+      (TQ *)q_out, (const TI *)qkv, row_stride, n_slices, slice_stride, bias, inv_freq, freq_factors,   \
+      rot_dims, row_pos, row_seq,                                                                    \
       (TC *)k_cache, (TC *)v_cache, page_table, max_pages, n_pages_total, heads_q, heads_kv, head_dim)
   const int key = qkv_dtype * 4 + q_dtype * 2 + cache_dtype;
   switch (key) {

@@ -51,6 +51,12 @@ int sb_embed(float *out, const void *table, int table_dtype, const int32_t *ids,
 int sb_rmsnorm(void *y, int out_dtype, const float *x, const void *w, int w_dtype,
                const int32_t *rows, int n_rows, int width, float eps, void *stream);
 
+/* x[t,:] += sum_s partial[s][t][:] (+ bias), slices in ascending order; with do_norm
+ * also y[t,:] = rmsnorm(x[t,:]) * w.  partial is f32 [n_slices][n_rows][width]. */
+int sb_reduce_resid_norm(void *y, int y_dtype, float *x, const float *partial, int n_slices,
+                         const void *bias, int bias_dtype, const void *w, int w_dtype, int n_rows,
+                         int width, float eps, int do_norm, void *stream);
+
 /* Y[t,n] = sum_k X[t,k] W[n,k] (+ bias[n]) (+ resid[t,n]).   Plain tiled kernel,
  * float accumulation in ascending k for every element whatever the batch.
  * resid is f32 [t,n] and may be the same buffer as Y (when Y is f32). */
@@ -70,8 +76,10 @@ int sb_cast(void *dst, int dst_dtype, const void *src, int src_dtype, size_t n, 
 
 /* Rotate the query heads and key heads of a step's qkv rows, write the queries
  * to q_out and store keys and values into the paged cache.
- *   qkv        [n_rows, row_stride] of qkv_dtype, read only; a row is
- *              [heads_q*hd queries | heads_kv*hd keys | heads_kv*hd values]
+ *   qkv        [n_slices][n_rows, row_stride] of qkv_dtype, read only; a row is
+ *              [heads_q*hd queries | heads_kv*hd keys | heads_kv*hd values];
+ *              the slices (partial sums of the projection over K) are added
+ *              in ascending order, then `bias` (f32 [row], may be NULL)
  *   q_out      [n_rows, heads_q*hd] of q_dtype
  *   inv_freq   f32 [rot_dims/2]: angle of pair i at position p is
  *              float(p)*inv_freq[i], divided by freq_factors[i] when given.
@@ -82,7 +90,7 @@ int sb_cast(void *dst, int dst_dtype, const void *src, int src_dtype, size_t n, 
  *              stores nothing.
  */
 int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int qkv_dtype, int row_stride,
-                     const float *inv_freq, const float *freq_factors, int rot_dims,
+                     int n_slices, const float *bias, const float *inv_freq, const float *freq_factors, int rot_dims,
                      const int32_t *row_pos, const int32_t *row_seq, void *k_cache, void *v_cache,
                      int cache_dtype, const int32_t *page_table, int max_pages, int n_pages_total,
                      int n_rows, int heads_q, int heads_kv, int head_dim, void *stream);

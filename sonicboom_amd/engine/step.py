@@ -158,8 +158,11 @@ class Engine:
         their run order, and for the wanted rows the final norm and the head."""
         model = self.model
         x = model.embedding.forward(ctx.ids)
+        h = None
         for i, e in enumerate(model.order):
-            model.blocks[e.block].forward(x, ctx, self.bindings[i])
+            nxt = model.order[i + 1].block if i + 1 < len(model.order) else None
+            next_norm = getattr(model.blocks[nxt], "mixer_norm", None) if nxt is not None else None
+            h = model.blocks[e.block].forward(x, ctx, self.bindings[i], h=h, next_norm=next_norm)
         if ctx.n_wanted == 0:
             return torch.empty((0, model.vocab), dtype=torch.float32, device=self.device)
         h = model.final_norm.forward(x, model.rt.act_dtype, rows=ctx.want_rows)

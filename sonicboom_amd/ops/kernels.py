@@ -161,15 +161,24 @@ def _check_rows(row_pos, row_seq, page_table, n_rows):
 def rope_kv_store(qkv: torch.Tensor, q_dtype: torch.dtype, inv_freq: Optional[torch.Tensor],
                   freq_factors: Optional[torch.Tensor], rot_dims: int, row_pos: torch.Tensor,
                   row_seq: torch.Tensor, k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                  page_table: Optional[torch.Tensor], heads_q: int, heads_kv: int, head_dim: int) -> torch.Tensor:
+                  page_table: Optional[torch.Tensor], heads_q: int, heads_kv: int, head_dim: int,
+                  bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Rotate queries and keys of ``qkv`` [n, (hq+2hkv)*hd], return the queries
     [n, hq*hd] in ``q_dtype`` and store keys and values in the paged cache.
-    ``heads_kv`` = 0 (and no cache) for a layer that stores nothing."""
-    _dev(qkv, inv_freq, freq_factors, row_pos, row_seq, k_cache, v_cache, page_table)
-    n = qkv.shape[0]
+    ``heads_kv`` = 0 (and no cache) for a layer that stores nothing.  ``qkv`` may be
+    [slices, n, width]: partial sums of the projection, added here in ascending order;
+    ``bias`` (float32 [width]) is added after them."""
+    _dev(qkv, inv_freq, freq_factors, row_pos, row_seq, k_cache, v_cache, page_table, bias)
+    n_slices = 1
+    if qkv.dim() == 3:
+        n_slices = qkv.shape[0]
+        qkv = qkv.view(-1, qkv.shape[2])
+    n = qkv.shape[0] // n_slices
     need = (heads_q + 2 * heads_kv) * head_dim
     if qkv.dim() != 2 or qkv.shape[1] < need:
         raise KernelLibraryError(f"qkv rows have {qkv.shape[1]} elements, {need} are needed")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() < need):
+        raise KernelLibraryError("the qkv bias must be float32 and cover a whole row")
     if inv_freq is not None:
         if inv_freq.dtype != torch.float32 or inv_freq.numel() != rot_dims // 2:
             raise KernelLibraryError("inv_freq must be float32 [rot_dims/2]")
@@ -184,7 +193,7 @@ def rope_kv_store(qkv: torch.Tensor, q_dtype: torch.dtype, inv_freq: Optional[to
     q = torch.empty((n, heads_q * head_dim), dtype=q_dtype, device=qkv.device)
     lib = library.core()
     check(lib.sb_rope_kv_store(
-        _p(q), _dt(q), _p(qkv), _dt(qkv), qkv.shape[1], _p(inv_freq), _p(freq_factors), rot_dims,
+        _p(q), _dt(q), _p(qkv), _dt(qkv), qkv.shape[1], n_slices, _p(bias), _p(inv_freq), _p(freq_factors), rot_dims,
         _p(row_pos), _p(row_seq), _p(k_cache), _p(v_cache), _dt(k_cache) if k_cache is not None else 0,
         _p(page_table), max_pages, n_pages, n, heads_q, heads_kv, head_dim, _stream()))
     return q
@@ -261,6 +270,57 @@ def top_candidates(logits: torch.Tensor, temperature: float, k: int = MAX_CANDID
 # dispatch between the plain kernels and the MFMA kernels
 # --------------------------------------------------------------------------
 SKINNY_MAX_ROWS = 64
+
+
+def gemm_bf16_partial(x: torch.Tensor, w: torch.Tensor, packed_shape=None) -> Optional[torch.Tensor]:
+    """The raw product x w^T of up to 64 bfloat16 rows in K slices, float32 [slices, rows, out], for
+    a consumer that adds the slices itself (:func:`reduce_resid_norm`, :func:`rope_kv_store`).
+    None when the weight-streaming kernel does not take the sizes."""
+    _dev(x, w)
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or x.dim() != 2:
+        return None
+    n, k = packed_shape if packed_shape is not None else (w.shape[0], w.shape[-1])
+    t = x.shape[0]
+    if x.shape[1] != k:
+        raise KernelLibraryError(f"gemm shapes do not match: x {tuple(x.shape)}, w {(n, k)}")
+    if t > SKINNY_MAX_ROWS or t == 0 or k % 8 or x.data_ptr() % 16 or w.data_ptr() % 16:
+        return None
+    lib = library.core()
+    slices = lib.sb_gemm_skinny_slices(t, n, k)
+    partial = torch.empty((slices, t, n), dtype=torch.float32, device=x.device)
+    check(lib.sb_gemm_skinny_partial_bf16(_p(partial), _p(x), _p(w), t, n, k, 1 if packed_shape is not None else 0,
+                                          _stream()))
+    return partial
+
+
+def reduce_resid_norm(partial: torch.Tensor, bias: Optional[torch.Tensor], x: torch.Tensor,
+                      norm_weight: Optional[torch.Tensor], eps: float, out_dtype: Optional[torch.dtype]
+                      ) -> Optional[torch.Tensor]:
+    """x += sum of the slices of ``partial`` [slices, rows, width] (+ bias); when ``out_dtype`` is
+    given also returns rmsnorm(x) * norm_weight in that type.  One pass over the row."""
+    _dev(partial, bias, x, norm_weight)
+    if partial.dim() != 3 or partial.dtype != torch.float32 or x.dtype != torch.float32 \
+            or tuple(x.shape) != tuple(partial.shape[1:]):
+        raise KernelLibraryError("reduce_resid_norm needs float32 slices [s, rows, width] and a residual [rows, width]")
+    s_, t, width = partial.shape
+    if bias is not None and bias.numel() != width:
+        raise KernelLibraryError("bias does not match the row width")
+    if norm_weight is not None and norm_weight.numel() != width:
+        raise KernelLibraryError("norm weight does not match the row width")
+    lib = library.core()
+    if width % 4 or width > lib.sb_reduce_resid_norm_max_width():
+        raise KernelLibraryError(f"reduce_resid_norm takes widths in steps of 4 up to "
+                                 f"{lib.sb_reduce_resid_norm_max_width()}, not {width}")
+    y = torch.empty((t, width), dtype=out_dtype, device=x.device) if out_dtype is not None else None
+    check(lib.sb_reduce_resid_norm(_p(y), _dt(y) if y is not None else 0, _p(x), _p(partial), s_, _p(bias),
+                                   _dt(bias) if bias is not None else 0, _p(norm_weight),
+                                   _dt(norm_weight) if norm_weight is not None else 0, t, width, float(eps),
+                                   1 if out_dtype is not None else 0, _stream()))
+    return y
+
+
+def reduce_resid_norm_ok(width: int) -> bool:
+    return width % 4 == 0 and width <= library.core().sb_reduce_resid_norm_max_width()
 
 
 def pack_weight(w: torch.Tensor, gated: bool = False) -> torch.Tensor:

@@ -25,7 +25,9 @@ _CORE_SIGNATURES = {
     "sb_silu_mul": [_P, _I, _P, _I, _I, _I, _P],
     "sb_add_into": [_P, _P, _I, _Z, _P],
     "sb_cast": [_P, _I, _P, _I, _Z, _P],
-    "sb_rope_kv_store": [_P, _I, _P, _I, _I, _P, _P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
+    "sb_rope_kv_store": [_P, _I, _P, _I, _I, _I, _P, _P, _P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
+    "sb_reduce_resid_norm": [_P, _I, _P, _P, _I, _P, _I, _P, _I, _I, _I, _F, _I, _P],
+    "sb_reduce_resid_norm_max_width": [],
     "sb_attention": [_P, _P, _I, _I, _P, _P, _I, _P, _I, _I, _P, _P, _I, _I, _I, _I, _F, _I, _P],
     "sb_argmax": [_P, _P, _I, _I, _P, _P, _P],
     "sb_argmax_parts": [_I],
@@ -34,6 +36,8 @@ _CORE_SIGNATURES = {
 }
 # Entry points of later kernels; declared when the library has them.
 _OPTIONAL_SIGNATURES = {
+    "sb_gemm_skinny_partial_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
+    "sb_gemm_skinny_slices": [_I, _I, _I],
     "sb_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _P, _Z, _P],
     "sb_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _P],
 }

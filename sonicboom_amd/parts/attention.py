@@ -96,15 +96,24 @@ class Attention(Mixer):
     def cache_spec(self) -> KVSpec:
         return KVSpec(self.heads_kv, self.head_dim, self.window)
 
-    def forward(self, h, x, ctx, binding) -> None:
+    fuses_norm = True
+
+    def forward(self, h, x, ctx, binding, then_norm=None):
+        """x += attention(h).  Returns then_norm(x) when the output projection could apply the
+        norm in its last pass, else None."""
         rt = self.rt
         writes = binding.writes_cache
         if not writes:
             self.query_only()
         proj = self.qkv if writes else self._q_only
         # q, k, v stay float32 until they have been rotated: one rounding on the way to the cache.
-        qkv = proj(h, torch.float32)
         tables = self.position.rotary_tables()
+        bias = None
+        qkv = proj.partial(h) if tables is not None else None
+        if qkv is not None:
+            bias = proj.bias          # the rotate-and-store kernel adds the K slices and the bias
+        else:
+            qkv = proj(h, torch.float32)
         if tables is None:
             self.position.apply(qkv, ctx, self.heads_q, self.heads_kv if writes else 0, self.head_dim)
             tables = (None, None, 0)
@@ -113,7 +122,8 @@ class Attention(Mixer):
         q = ops.rope_kv_store(
             qkv, rt.act_dtype, inv_freq, freq_factors, rot_dims, ctx.row_pos, ctx.row_seq,
             binding.k_cache if writes else None, binding.v_cache if writes else None,
-            page_table if writes else None, self.heads_q, self.heads_kv if writes else 0, self.head_dim)
+            page_table if writes else None, self.heads_q, self.heads_kv if writes else 0, self.head_dim,
+            bias=bias)
         a = ops.attention(q, binding.k_cache, binding.v_cache, page_table, ctx, self.heads_q, self.heads_kv,
                           self.head_dim, self.scale, self.window, fast=rt.fast_kernels)
-        self.out(a, torch.float32, resid=x, out=x)
+        return self.out.add_into(a, x, then_norm, rt.act_dtype)

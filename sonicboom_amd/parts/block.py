@@ -27,7 +27,23 @@ class PreNormBlock(Part):
         self.ffn_norm = parts["ffn_norm"]
         self.ffn = parts["ffn"]
 
-    def forward(self, x, ctx, binding) -> None:
+    def forward(self, x, ctx, binding, h=None, next_norm=None):
+        """Run the block on the residual stream ``x`` in place.  ``h`` is mixer_norm(x) when the
+        previous block has already computed it; ``next_norm`` is the norm the next block starts
+        with.  Returns next_norm(x) when the feed-forward's last pass produced it, else None.
+        Mixers and feed-forwards that can apply a norm in their last pass say so with
+        ``fuses_norm``; the others are simply followed by the norm."""
         act = self.rt.act_dtype
-        self.mixer.forward(self.mixer_norm.forward(x, act), x, ctx, binding)
-        self.ffn.forward(self.ffn_norm.forward(x, act), x, ctx)
+        if h is None:
+            h = self.mixer_norm.forward(x, act)
+        f = None
+        if getattr(self.mixer, "fuses_norm", False):
+            f = self.mixer.forward(h, x, ctx, binding, then_norm=self.ffn_norm)
+        else:
+            self.mixer.forward(h, x, ctx, binding)
+        if f is None:
+            f = self.ffn_norm.forward(x, act)
+        if getattr(self.ffn, "fuses_norm", False):
+            return self.ffn.forward(f, x, ctx, then_norm=next_norm)
+        self.ffn.forward(f, x, ctx)
+        return None

@@ -44,6 +44,10 @@ class GatedDenseFFN(Part):
         self.gate_up = Linear(torch.cat([g, u], dim=0), None, rt.fast_kernels, gated=True)
         self.down = Linear(tensors["down_weight"], None, rt.fast_kernels)
 
-    def forward(self, h, x, ctx) -> None:
+    fuses_norm = True
+
+    def forward(self, h, x, ctx, then_norm=None):
+        """x += ffn(h).  Returns then_norm(x) when the down projection could apply the norm in
+        its last pass, else None."""
         mid = self.gate_up.gated_product(h, self.rt.act_dtype)
-        self.down(mid, torch.float32, resid=x, out=x)
+        return self.down.add_into(mid, x, then_norm, self.rt.act_dtype)

@@ -62,6 +62,24 @@ class Linear:
             x = ops.cast(x, torch.float32)
         return ops.gemm_plain(x, w, self.bias, resid, out_dtype, out)
 
+    def partial(self, x: torch.Tensor) -> Optional[torch.Tensor]:
+        """The raw product in K slices, float32 [slices, rows, out] (bias and residual left to the
+        consumer), when the weight-streaming kernel takes this call; else None."""
+        if self.packed is None or self.gated or x.dtype != torch.bfloat16:
+            return None
+        return ops.gemm_bf16_partial(x, self.packed, packed_shape=(self.rows, self.n_in))
+
+    def add_into(self, x: torch.Tensor, resid: torch.Tensor, then_norm=None, out_dtype=None):
+        """resid += x W^T (+ b).  With ``then_norm`` (an RMS norm part) tries to return
+        then_norm(resid) in ``out_dtype`` from the same pass; None when the caller has to norm."""
+        part = self.partial(x)
+        if part is not None and ops.reduce_resid_norm_ok(self.n_out):
+            fuse = then_norm is not None and getattr(then_norm, "fusable", False)
+            return ops.reduce_resid_norm(part, self.bias, resid, then_norm.weight if fuse else None,
+                                         then_norm.eps if fuse else 0.0, out_dtype if fuse else None)
+        self(x, torch.float32, resid=resid, out=resid)
+        return None
+
     def gated_product(self, x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
         """silu(x Wg^T) * (x Wu^T): one fused kernel on the matrix cores, or the product in
         float32 followed by the activation kernel."""

@@ -15,6 +15,7 @@ def rmsnorm_spec(weight_name: str, width: int, eps: float) -> PartSpec:
 class RMSNorm(Part):
     """y = (x * 1/sqrt(mean(x^2) + eps)) * w; the weight multiplies as it is."""
     category = "norm"
+    fusable = True      # a projection's last pass may apply this norm (it exposes weight and eps)
 
     def __init__(self, spec, tensors, parts, rt):
         super().__init__(spec, tensors, parts, rt)
