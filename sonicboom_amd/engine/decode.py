@@ -80,6 +80,11 @@ class _StaticContext:
         for g in range(self.n_groups):
             n[o[8 + g]:o[9 + g]] = cache.page_table(g, slots, min_width=self.width).reshape(-1)
         self.max_len_after = int(lengths.max()) + 1
+        # the host's view of the step, as StepContext has it
+        self.slot_list = list(slots)
+        self.lengths_before = lengths.tolist()
+        self.n_new = [1] * len(slots)
+        self.host_row_pos = lengths
         self.dev.copy_(host, non_blocking=True)
 
 
@@ -89,7 +94,10 @@ class DecodeLoop:
 
     def __init__(self, engine, use_graph: bool = True):
         self.engine = engine
-        self.use_graph = use_graph
+        # a part that steers its work from the host (Python control flow over the step's
+        # sequences) cannot be replayed from a recording; parts say so with graph_safe
+        parts = [p for b in engine.model.blocks for p in (getattr(b, "mixer", None), getattr(b, "ffn", None))]
+        self.use_graph = use_graph and all(getattr(p, "graph_safe", False) for p in parts if p is not None)
         self._ctx: Dict[Tuple[int, int], _StaticContext] = {}
         self._graphs: Dict[Tuple[int, int, bool], Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
         self._uses: Dict[Tuple[int, int, bool], int] = {}

@@ -97,6 +97,7 @@ class Attention(Mixer):
         return KVSpec(self.heads_kv, self.head_dim, self.window)
 
     fuses_norm = True
+    graph_safe = True     # its launches depend on device buffers only
 
     def forward(self, h, x, ctx, binding, then_norm=None):
         """x += attention(h).  Returns then_norm(x) when the output projection could apply the

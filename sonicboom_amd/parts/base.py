@@ -17,6 +17,10 @@ copy in the activation type, ``ctx`` the step's
 * **mixer**     ``cache_spec() -> KVSpec | None``, ``state_spec() -> StateSpec | None``,
                 ``forward(h, x, ctx, binding)`` adds the mixer's output into ``x``.
 * **ffn**       ``forward(h, x, ctx)`` adds the feed-forward's output into ``x``.
+                Mixers and feed-forwards may set ``fuses_norm`` (their ``forward`` then
+                takes ``then_norm=`` and may return the normed stream) and ``graph_safe``
+                (their launches depend on device buffers only, so a decode step may be
+                recorded once and replayed).
 * **block**     ``mixer`` attribute and ``forward(x, ctx, binding)``.
 * **embedding** ``forward(ids) -> x``
 * **head**      ``forward(h) -> float32 logits [rows, vocab]``

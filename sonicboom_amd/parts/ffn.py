@@ -45,6 +45,7 @@ class GatedDenseFFN(Part):
         self.down = Linear(tensors["down_weight"], None, rt.fast_kernels)
 
     fuses_norm = True
+    graph_safe = True     # its launches depend on device buffers only
 
     def forward(self, h, x, ctx, then_norm=None):
         """x += ffn(h).  Returns then_norm(x) when the down projection could apply the norm in

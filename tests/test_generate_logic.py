@@ -1,0 +1,139 @@
+"""The generation loop's decisions, on the CPU with an engine whose "model" is a table:
+batches one after another, unequal prompts, stop tokens, sequences that end earlier, slots
+given back and used again, positions of the draws."""
+import numpy as np
+import pytest
+
+from sonicboom_amd.cache import PAGE, CacheError, GroupSpec, PagedCache
+from sonicboom_amd.engine.generate import generate, plan_batches
+from sonicboom_amd.sampling import SamplingParams
+
+VOCAB = 50
+
+
+class TableEngine:
+    """next token = (7 * last token + position) % VOCAB, delivered as one-hot logits.  Keeps the
+    cache's books exactly as the real engine does and records every step."""
+
+    def __init__(self, max_tokens, max_slots=None):
+        self.cache = PagedCache([GroupSpec(1, 16, 0, (0,))], max_tokens, allocate=False, max_slots=max_slots)
+        self.steps = []
+        self.max_live = 0
+        self.slot_uses = {}
+
+    def alloc_slot(self):
+        s = self.cache.alloc_slot()
+        self.slot_uses[s] = self.slot_uses.get(s, 0) + 1
+        self.max_live = max(self.max_live, len(self.cache.live_slots))
+        return s
+
+    def free_slot(self, s):
+        self.cache.free_slot(s)
+
+    def step(self, entries):
+        slots = [e.slot for e in entries]
+        n_new = [len(e.tokens) for e in entries]
+        self.cache.reserve(slots, n_new)
+        rows = []
+        for e in entries:
+            base = self.cache.length(e.slot)
+            for w in e.want:
+                row = np.full(VOCAB, -1.0, dtype=np.float32)
+                row[(7 * e.tokens[w] + base + w) % VOCAB] = 1.0
+                rows.append(row)
+        self.cache.advance(slots, n_new)
+        self.steps.append([(e.slot, len(e.tokens)) for e in entries])
+        return np.stack(rows)
+
+
+class HostSampler:
+    def __init__(self):
+        self.positions = []
+
+    def pick(self, logits, positions, histories):
+        self.positions.append(list(positions))
+        assert all(len(h) == p for h, p in zip(histories, positions))
+        return [int(np.argmax(r)) for r in logits]
+
+
+def expected(prompt, n, stop=()):
+    seq, out = list(prompt), []
+    for _ in range(n):
+        t = (7 * seq[-1] + len(seq) - 1) % VOCAB
+        out.append(t)
+        seq.append(t)
+        if t in stop:
+            break
+    return out
+
+
+def test_unequal_prompts_in_one_batch():
+    eng, smp = TableEngine(64 * 8), HostSampler()
+    prompts = [[1, 2, 3, 4, 5], [9] * 9, [4] * 13]
+    outs = generate(eng, prompts, SamplingParams(max_tokens=8), stop_tokens=(), sampler=smp)
+    assert outs == [expected(p, 8) for p in prompts]
+    assert eng.steps[0] == [(0, 5), (1, 9), (2, 13)]                 # the prompts in one step
+    assert all(n == 1 for st in eng.steps[1:] for _, n in st)         # then one token each
+    assert len(eng.steps) == 8                                        # the last token is not fed back
+    assert smp.positions[0] == [5, 9, 13] and smp.positions[1] == [6, 10, 14]
+    assert not eng.cache.live_slots and eng.cache.held_pages() == 0
+
+
+def test_stop_token_is_emitted_and_ends_only_its_sequence():
+    prompts = [[1, 2, 3], [5, 6], [8]]
+    free = [expected(p, 10) for p in prompts]
+    stop = (free[1][3],)
+    want = [expected(p, 10, stop) for p in prompts]
+    assert len(want[1]) == 4 and want[1][-1] == stop[0]
+    eng = TableEngine(64 * 8)
+    outs = generate(eng, prompts, SamplingParams(max_tokens=10), stop_tokens=stop, sampler=HostSampler())
+    assert outs == want
+    sizes = [len(st) for st in eng.steps]
+    assert sizes[0] == 3 and min(sizes) < 3                           # the batch shrinks when one ends
+    assert not eng.cache.live_slots
+
+
+def test_batches_one_after_another_reuse_slots_and_pages():
+    eng = TableEngine(64 * 3, max_slots=2)                            # room for two short requests at a time
+    prompts = [[i + 1] * (3 + i) for i in range(7)]
+    outs = generate(eng, prompts, SamplingParams(max_tokens=5), stop_tokens=(), max_batch=4, sampler=HostSampler())
+    assert outs == [expected(p, 5) for p in prompts]
+    assert eng.max_live == 2 and sum(eng.slot_uses.values()) == 7 and max(eng.slot_uses.values()) >= 3
+    assert eng.cache.held_pages() == 0 and not eng.cache.live_slots
+
+
+def test_callback_and_max_tokens():
+    eng = TableEngine(64 * 4)
+    seen = []
+
+    def cb(i, t):
+        seen.append((i, t))
+        return i == 0 and len([1 for j, _ in seen if j == 0]) == 2    # end request 0 after its second token
+
+    outs = generate(eng, [[1, 2], [3]], SamplingParams(max_tokens=4), stop_tokens=(), callback=cb, sampler=HostSampler())
+    assert outs == [expected([1, 2], 2), expected([3], 4)]
+    assert [t for i, t in seen if i == 1] == outs[1]
+    assert generate(eng, [[1]], SamplingParams(max_tokens=0), sampler=HostSampler()) == [[]]
+    assert generate(eng, [], SamplingParams(), sampler=HostSampler()) == []
+
+
+def test_slots_come_back_when_a_step_fails():
+    eng = TableEngine(64 * 4)
+
+    def boom(entries):
+        raise RuntimeError("device lost")
+    eng.step = boom
+    with pytest.raises(RuntimeError):
+        generate(eng, [[1, 2, 3]], SamplingParams(max_tokens=3), sampler=HostSampler())
+    assert not eng.cache.live_slots and eng.cache.held_pages() == 0
+
+
+def test_plan_batches():
+    assert plan_batches([5, 9, 13], 8, n_pages=8, max_batch=64) == [[0, 1, 2]]
+    assert plan_batches([5, 9, 13], 8, n_pages=8, max_batch=2) == [[0, 1], [2]]
+    assert plan_batches([60, 60, 60], 8, n_pages=4, max_batch=64) == [[0, 1], [2]]      # 2 pages each
+    assert plan_batches([1] * 5, 1, n_pages=100, max_batch=64, max_slots=2) == [[0, 1], [2, 3], [4]]
+    with pytest.raises(ValueError, match="request 1"):
+        plan_batches([5, 300], 8, n_pages=4, max_batch=64)
+    with pytest.raises(ValueError, match="empty prompt"):
+        plan_batches([0], 8, n_pages=4, max_batch=64)

@@ -1,0 +1,207 @@
+"""Generation through the Python entry point and the command line, on the GPU: greedy tokens
+against the plain implementation, seeded sampling, stop tokens, batches, long decoding and
+the first tokens of a sequence."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from conftest import ROOT, TINY, random_prompt
+from helpers import assert_logits_close, plain_logits, plain_model
+from plain import qwen2_plain, sampling_plain
+
+pytestmark = pytest.mark.gpu
+
+_MODELS = {}
+
+
+def model_for(folder, dtype):
+    from sonicboom_amd.api import Model
+    if (folder, dtype) not in _MODELS:
+        _MODELS[(folder, dtype)] = Model.load(folder, dtype=dtype)
+    return _MODELS[(folder, dtype)]
+
+
+def prompts_for(name, lengths, seed=0):
+    rng = np.random.default_rng(seed)
+    return [random_prompt(rng, TINY[name]["vocab_size"], n) for n in lengths]
+
+
+def test_greedy_float32_equals_the_plain_implementation(model_folders):
+    """Tiny A: 3 prompts of 5/9/13 tokens, 8 greedy steps, as one batch."""
+    folder = model_folders["A"]
+    cfg, w = plain_model(folder)
+    prompts = prompts_for("A", [5, 9, 13])
+    session = model_for(folder, "float32").session(max_tokens=64 * 4)
+    got = session.generate(prompts, max_tokens=8, stop_tokens=())
+    assert got == [qwen2_plain.greedy(cfg, w, p, 8) for p in prompts]
+    # each prompt alone gives the same tokens: the batch changes nothing
+    assert [session.generate([p], max_tokens=8, stop_tokens=())[0] for p in prompts] == got
+    assert not session.engine.cache.live_slots
+
+
+def test_greedy_bfloat16_follows_the_plain_logits(model_folders):
+    """In bfloat16 a near tie may flip: every chosen token must be within a small margin of the
+    plain implementation's best logit for the history the engine itself produced."""
+    for name in ("A", "B", "C"):
+        folder = model_folders[name]
+        prompts = prompts_for(name, [3, 17, 40], seed=2)
+        session = model_for(folder, "bfloat16").session(max_tokens=64 * 6)
+        outs = session.generate(prompts, max_tokens=10, stop_tokens=())
+        for p, out in zip(prompts, outs):
+            logits = plain_logits(folder, p + out)
+            for i, t in enumerate(out):
+                row = logits[len(p) - 1 + i]
+                assert row[t] >= row.max() - 0.05 * max(1.0, np.abs(row).max()), (name, i)
+
+
+def test_temperature_sampling_tiny_b(model_folders):
+    """Tiny B: prompts of 1/7/20/33 tokens, 12 steps at temperature 0.8 with a fixed seed."""
+    folder = model_folders["B"]
+    prompts = prompts_for("B", [1, 7, 20, 33], seed=4)
+    session = model_for(folder, "float32").session(max_tokens=64 * 8)
+    kw = dict(temperature=0.8, seed=1234, max_tokens=12, stop_tokens=())
+    a = session.generate(prompts, **kw)
+    assert a == session.generate(prompts, **kw)                                   # same seed, same tokens
+    assert a != session.generate(prompts, **{**kw, "seed": 1235})                 # another seed differs
+    assert [session.generate([p], **kw)[0] for p in prompts] == a                 # alone or in a batch
+    assert all(len(o) == 12 for o in a)
+    # the plain sampler over the plain logits draws the same tokens (teacher-forced on the
+    # engine's history, so one flipped near-tie would not cascade)
+    for p, out in zip(prompts, a):
+        logits = plain_logits(folder, p + out)
+        for i, t in enumerate(out):
+            want = sampling_plain.sample_token(logits[len(p) - 1 + i], len(p) + i, temperature=0.8, seed=1234)
+            assert t == want, (len(p), i)
+
+
+def test_sampling_filters_and_penalties_run_on_the_device(model_folders):
+    folder = model_folders["A"]
+    prompts = prompts_for("A", [6, 11], seed=5)
+    session = model_for(folder, "float32").session(max_tokens=64 * 4)
+    kw = dict(temperature=1.1, seed=9, top_k=12, top_p=0.9, min_p=0.02, repeat_penalty=1.3, repeat_last_n=8,
+              presence_penalty=0.1, frequency_penalty=0.05, max_tokens=10, stop_tokens=())
+    outs = session.generate(prompts, **kw)
+    for p, out in zip(prompts, outs):
+        logits = plain_logits(folder, p + out)
+        hist = list(p)
+        for i, t in enumerate(out):
+            want = sampling_plain.sample_token(
+                logits[len(p) - 1 + i], len(p) + i, temperature=1.1, seed=9, top_k=12, top_p=0.9, min_p=0.02,
+                repeat_penalty=1.3, repeat_last_n=8, presence_penalty=0.1, frequency_penalty=0.05, history=hist)
+            assert t == want, (len(p), i)
+            hist.append(t)
+    # greedy with penalties takes the other arithmetic path
+    g = session.generate(prompts, repeat_penalty=1.5, presence_penalty=0.3, max_tokens=6, stop_tokens=())
+    for p, out in zip(prompts, g):
+        logits = plain_logits(folder, p + out)
+        hist = list(p)
+        for i, t in enumerate(out):
+            assert t == sampling_plain.sample_token(logits[len(p) - 1 + i], 0, repeat_penalty=1.5,
+                                                    presence_penalty=0.3, history=hist)
+            hist.append(t)
+
+
+def test_stop_tokens_and_batches_on_a_small_cache(model_folders):
+    folder = model_folders["B"]                      # its config.json names eos 7
+    cfg, w = plain_model(folder)
+    prompts = prompts_for("B", [4, 9, 2, 30, 12, 5, 21], seed=6)
+    free = [qwen2_plain.greedy(cfg, w, p, 9) for p in prompts]
+    session = model_for(folder, "float32").session(max_tokens=64 * 3, max_slots=3)
+    assert model_for(folder, "float32").eos == (7,)
+    # a stop token that some sequence produces early
+    stop = free[3][2]
+    want = [qwen2_plain.greedy(cfg, w, p, 9, stop=(stop,)) for p in prompts]
+    assert any(len(o) < 9 for o in want)
+    got = session.generate(prompts, max_tokens=9, stop_tokens=(stop,), max_batch=3)
+    assert got == want
+    assert not session.engine.cache.live_slots and session.engine.cache.held_pages() == 0
+
+
+def test_graph_replay_gives_the_same_tokens(model_folders):
+    folder = model_folders["C"]
+    prompts = prompts_for("C", [5, 61, 20], seed=7)
+    model = model_for(folder, "bfloat16")
+    with_graph = model.session(max_tokens=64 * 12)
+    without = model.session(max_tokens=64 * 12)
+    without.engine.use_graphs = False
+    a = with_graph.generate(prompts, max_tokens=150, stop_tokens=())     # crosses pages, replays many times
+    b = without.generate(prompts, max_tokens=150, stop_tokens=())
+    assert a == b and all(len(o) == 150 for o in a)
+    assert with_graph.engine.decode_loop()._graphs, "the decode loop never captured a graph"
+    s = with_graph.generate(prompts, temperature=0.7, seed=3, max_tokens=40, stop_tokens=())
+    assert s == without.generate(prompts, temperature=0.7, seed=3, max_tokens=40, stop_tokens=())
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_token_by_token_from_the_first_token(model_folders, dtype):
+    """A sequence fed one token at a time from its very first token, over several pages,
+    together with a second sequence that starts from a prompt: logits at every position."""
+    from sonicboom_amd.engine import StepEntry
+    folder = model_folders["B"]
+    a, b = prompts_for("B", [260, 200], seed=8)
+    eng = model_for(folder, dtype).session(max_tokens=64 * 10).engine
+    sa, sb = eng.alloc_slot(), eng.alloc_slot()
+    got_a, got_b = [], []
+    out = eng.step([StepEntry(sa, a[:1], [0]), StepEntry(sb, b[:70], range(70))]).cpu().numpy()
+    got_a.append(out[:1])
+    got_b.append(out[1:])
+    for i in range(1, 260):
+        entries = [StepEntry(sa, [a[i]], [0])]
+        if 70 + i - 1 < 200:
+            entries.append(StepEntry(sb, [b[70 + i - 1]], [0]))
+        out = eng.step(entries).cpu().numpy()
+        got_a.append(out[:1])
+        if len(entries) == 2:
+            got_b.append(out[1:])
+    eng.free_slot(sa)
+    eng.free_slot(sb)
+    assert_logits_close(np.concatenate(got_a), plain_logits(folder, a), dtype, "token by token from position 0")
+    assert_logits_close(np.concatenate(got_b), plain_logits(folder, b), dtype, "prompt of 70, then token by token")
+
+
+def test_step_errors(model_folders):
+    from sonicboom_amd.engine import StepEntry, StepError
+    eng = model_for(model_folders["A"], "float32").session(max_tokens=64 * 2).engine
+    s = eng.alloc_slot()
+    with pytest.raises(StepError, match="outside the vocabulary"):
+        eng.step([StepEntry(s, [256], [0])])
+    with pytest.raises(StepError, match="at least one token"):
+        eng.step([StepEntry(s, [], [])])
+    with pytest.raises(StepError, match="wanted row"):
+        eng.step([StepEntry(s, [1, 2], [2])])
+    with pytest.raises(StepError, match="not in use"):
+        eng.step([StepEntry(99, [1], [0])])
+    with pytest.raises(StepError, match="out of cache pages"):
+        eng.step([StepEntry(s, [1] * 200, [0])])
+    assert eng.step([StepEntry(s, [1, 2, 3], [])]).shape == (0, 256)     # nothing wanted
+    assert eng.length(s) == 3
+    eng.free_slot(s)
+
+
+def test_command_line(model_folders, tmp_path):
+    folder = model_folders["A"]
+    cfg, w = plain_model(folder)
+    prompts = prompts_for("A", [4, 10], seed=9)
+    tokens = tmp_path / "prompts.txt"
+    tokens.write_text("\n".join(" ".join(map(str, p)) for p in prompts) + "\n")
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "sb-gen"), "-m", folder, "--tokens", str(tokens), "-n", "6",
+           "--dtype", "fp32", "--stop", ""]
+    out = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    got = [[int(t) for t in line.split()] for line in out.stdout.strip().splitlines()]
+    assert got == [qwen2_plain.greedy(cfg, w, p, 6) for p in prompts]
+    # random weights from a configuration file, sampled
+    cfg_file = tmp_path / "config.json"
+    cfg_file.write_text(json.dumps(TINY["B"]))
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "sb-gen"), "--random", str(cfg_file), "--seed", "3",
+           "--tokens", str(tokens), "-n", "5", "--temperature", "0.8", "--sample-seed", "11", "--top-k", "20"]
+    one = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    two = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert one.returncode == 0 and one.stdout == two.stdout and len(one.stdout.split()) <= 10
+    bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "sb-gen"), "--tokens", str(tokens)],
+                         capture_output=True, text=True, timeout=60)
+    assert bad.returncode == 2 and "usage" in bad.stderr

@@ -1,0 +1,126 @@
+"""Sampling on the host: the plain sampler against the reference's test vectors, and the
+product's host stages (filters, Philox, Gumbel draw) against the plain sampler."""
+import math
+
+import numpy as np
+import pytest
+
+from plain import sampling_plain as SP
+from sonicboom_amd.sampling import SamplingParams, filter_candidates, gumbel_draw, penalty_items, philox4x32_10
+
+F32 = np.float32
+
+
+def test_philox_known_answer():
+    """/root/reference/tests/core/test_sampling.cpp:42-49 (Random123, zero counter and key)."""
+    want = [0x6627E8D5, 0xE169C58D, 0xBC57AC4C, 0x9B00DBD8]
+    assert SP.philox4x32_10([0, 0, 0, 0], 0) == want
+    assert [int(w) for w in philox4x32_10(0, 0, 0, 0, 0)] == want
+    # the vectorised form agrees with the plain one on other counters and a 64-bit key
+    key = 0x0123456789ABCDEF
+    ids = np.array([0, 1, 77, 152063], dtype=np.uint64)
+    got = philox4x32_10(12345, 6, ids, 0, key)
+    for i, t in enumerate(ids):
+        assert [int(w[i]) for w in got] == SP.philox4x32_10([12345, 6, int(t), 0], key)
+
+
+def test_greedy_and_top_k_one():
+    """test_sampling.cpp:51-69."""
+    assert SP.sample_token(np.array([0.2, 0.2, 0.9, 0.1], F32), 0) == 2
+    assert SP.sample_token(np.array([0.5, 0.5, 0.1], F32), 0) == 0
+    logits = np.array([0.5, 2.5, 1.5, -1.0], F32)
+    for pos in range(32):
+        assert SP.sample_token(logits, pos, temperature=1.0, top_k=1) == 1
+
+
+def test_filter_sets():
+    """test_sampling.cpp:71-117: top-k, min-p and nucleus surviving sets."""
+    assert SP.surviving_ids(np.array([3, 2, 1, 0], F32), 1.0, top_k=2) == [0, 1]
+    assert SP.surviving_ids(np.zeros(4, F32), 1.0, top_k=2) == [0, 1]                 # ties by id
+    z = np.array([0.0, -1.0, -3.0], F32)
+    assert SP.surviving_ids(z, 1.0, min_p=0.1) == [0, 1]                              # ln 0.1 = -2.30
+    assert SP.surviving_ids(z, 1.0, min_p=0.5) == [0]
+    four = np.zeros(4, F32)
+    assert SP.surviving_ids(four, 1.0, top_p=0.6) == [0, 1, 2]
+    assert SP.surviving_ids(four, 1.0, top_p=0.5) == [0, 1]
+    assert SP.surviving_ids(four, 1.0, top_p=0.24) == [0]
+    # the window of 30 below the best z
+    assert SP.surviving_ids(np.array([0.0, -29.0, -31.0], F32), 1.0) == [0, 1]
+    assert SP.surviving_ids(np.array([0.0, -29.0, -31.0], F32), 0.5) == [0]          # z = l / T
+
+
+def test_penalties():
+    """test_sampling.cpp:119-169."""
+    assert SP.sample_token(np.array([1.5, 1.0], F32), 0, repeat_penalty=2.0, history=[0]) == 1
+    assert SP.sample_token(np.array([-0.5, -0.8], F32), 0, repeat_penalty=2.0, history=[0]) == 1
+    assert SP.sample_token(np.array([1.0, 0.9], F32), 0, presence_penalty=0.2, history=[0]) == 1
+    assert SP.sample_token(np.array([1.0, 0.9], F32), 0, frequency_penalty=0.04, history=[0, 0, 0]) == 1
+    # outside the window of repeat_last_n nothing is penalised
+    assert SP.sample_token(np.array([1.0, 0.9], F32), 0, presence_penalty=0.2, repeat_last_n=2,
+                           history=[0, 1, 1]) == 0
+    assert penalty_items([[1, 2, 2, 49], [], [7] * 10], 64, 50) == ([0, 0, 0, 2], [1, 2, 49, 7], [1, 2, 1, 10])
+    assert penalty_items([[1, 2, 3]], 2, 50) == ([0, 0], [2, 3], [1, 1])
+    assert penalty_items([[1, 99]], 64, 50) == ([0], [1], [1])
+
+
+def test_candidate_cap_and_order():
+    """test_sampling.cpp:171-258: 256 candidates, (z descending, id ascending), z = l / T."""
+    r = np.random.default_rng(0)
+    logits = r.standard_normal(1000).astype(F32)
+    logits[10] = logits[500] = 9.0
+    c = SP.select_candidates(logits, 0.7)
+    assert len(c) == 256 and c[0][0] == 10 and c[1][0] == 500
+    assert all((a[1] > b[1]) or (a[1] == b[1] and a[0] < b[0]) for a, b in zip(c, c[1:]))
+    assert all(z == F32(logits[i] / F32(0.7)) for i, z in c)
+
+
+def test_seed_and_position_fix_the_draw():
+    """test_sampling.cpp:260-281."""
+    logits = np.random.default_rng(1).standard_normal(64).astype(F32)
+    a = [SP.sample_token(logits, p, temperature=1.0, seed=7) for p in range(64)]
+    assert a == [SP.sample_token(logits, p, temperature=1.0, seed=7) for p in range(64)]
+    assert a != [SP.sample_token(logits, p, temperature=1.0, seed=8) for p in range(64)]
+    assert len(set(a)) > 8
+
+
+def test_draws_follow_the_softmax():
+    """test_sampling.cpp:283-313 with fewer draws: chi-square of the draw counts against the softmax."""
+    logits = np.array([1.0, 0.5, 0.0, -0.5, -1.0], F32)
+    cands = SP.select_candidates(logits, 1.0)
+    n = 20000
+    counts = np.zeros(5)
+    for pos in range(n):
+        counts[SP.draw(cands, 99, pos)] += 1
+    p = np.exp(logits.astype(np.float64))
+    p /= p.sum()
+    chi2 = (((counts - n * p) ** 2) / (n * p)).sum()
+    assert chi2 < 18.47                       # 4 degrees of freedom, p = 0.001
+
+
+@pytest.mark.parametrize("params", [
+    dict(temperature=0.8), dict(temperature=1.3, top_k=5), dict(temperature=0.5, top_p=0.7),
+    dict(temperature=1.0, min_p=0.2), dict(temperature=0.9, top_k=40, top_p=0.9, min_p=0.01),
+])
+def test_product_host_stages_equal_the_plain_sampler(params):
+    r = np.random.default_rng(5)
+    for trial in range(20):
+        logits = (r.standard_normal(400) * 3).astype(F32)
+        cands = SP.select_candidates(logits, params["temperature"])
+        ids = np.array([c[0] for c in cands], dtype=np.int32)
+        z = np.array([c[1] for c in cands], dtype=np.float32)
+        sp = SamplingParams(seed=trial, **params)
+        kept_ids, kept_z = filter_candidates(ids, z, sp)
+        want = SP.filter_candidates(cands, params.get("top_k", 0), params.get("top_p", 1.0), params.get("min_p", 0.0))
+        assert kept_ids.tolist() == [c[0] for c in want]
+        for pos in (0, 17, 2 ** 33 + 5):
+            assert gumbel_draw(kept_ids, kept_z, trial, pos) == SP.draw(want, trial, pos)
+
+
+def test_params_validation():
+    assert SamplingParams(repeat_penalty=0.0).validated().repeat_penalty == 1.0
+    assert not SamplingParams().has_penalties and SamplingParams(presence_penalty=0.1).has_penalties
+    assert not SamplingParams(presence_penalty=0.1, repeat_last_n=0).has_penalties
+    for bad in (dict(temperature=-1.0), dict(top_p=1.5), dict(min_p=-0.1), dict(top_k=-1), dict(repeat_penalty=-2.0),
+                dict(seed=2 ** 64)):
+        with pytest.raises(ValueError):
+            SamplingParams(**bad).validated()
