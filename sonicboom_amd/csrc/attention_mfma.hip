@@ -49,17 +49,25 @@ constexpr int DT = HD / 16;          // 16-row tiles of O^T
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kPagesPerChunk = 4;
 
+// A wave's running softmax for NC groups of 16 query columns that share positions (and so the
+// mask): in decode one group, the heads of a kv head; in prefill up to four heads of one kv head
+// for the same 16 positions, so that every key and value fragment feeds NC products.
+template <int NC>
 struct WaveState {
-  floatx4_t o[DT];   // O^T[d = 16 dt + 4 g + i][col]
-  float m;           // running maximum of the column (log2 domain), same in the four lane groups
-  float l;           // this lane's share of the running sum
+  floatx4_t o[NC][DT];   // O^T[d = 16 dt + 4 g + i][col]
+  float m[NC];           // running maximum of the column (log2 domain), same in the four lane groups
+  float l[NC];           // this lane's share of the running sum
 };
 
-__device__ __forceinline__ void init_state(WaveState &st) {
+template <int NC>
+__device__ __forceinline__ void init_state(WaveState<NC> &st) {
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) st.o[dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-  st.m = -__builtin_inff();
-  st.l = 0.f;
+  for (int c = 0; c < NC; ++c) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) st.o[c][dt] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+    st.m[c] = -__builtin_inff();
+    st.l[c] = 0.f;
+  }
 }
 
 // Zero the elements of a fragment of 8 consecutive keys from index n_keep on.
@@ -107,86 +115,98 @@ __device__ __forceinline__ void load_half(HalfPage &hp, const bf16_t *__restrict
   for (int dt = 0; dt < DT; ++dt) hp.v[dt] = ld16(vp + size_t(dt * 16 + r) * SB_PAGE + 32 * half + 8 * g, true);
 }
 
-// 32 keys at absolute positions base .. base+31, their fragments in hp, for the wave's 16 columns.
-// col_pos / col_lo: last and first visible key of this lane's column (col_pos < 0: the column is
-// empty).  key_hi / key_lo: the same over all columns of the wave (uniform).
-__device__ __forceinline__ void attend_half(WaveState &st, const bf16x8_t (&qf)[KS], const HalfPage &hp,
+// 32 keys at absolute positions base .. base+31, their fragments in hp, for the wave's NC groups
+// of 16 columns.  col_pos / col_lo: last and first visible key of this lane's column (col_pos < 0:
+// the column is empty); the groups share them.  key_hi / key_lo: the same over all columns of the
+// wave (uniform).
+template <int NC>
+__device__ __forceinline__ void attend_half(WaveState<NC> &st, const bf16x8_t (&qf)[NC][KS], const HalfPage &hp,
                                             int base, int col_pos, int col_lo, int key_lo, int key_hi,
                                             float scale_log2, int lane) {
   const int g = lane >> 4;
-  floatx4_t s[2];
-#pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    s[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) s[t] = mfma16(as_bf16x8(hp.k[t][ks]), qf[ks], s[t]);
-  }
-  // this lane: column lane % 16, keys base + 8 g + e, e = 0..7 (s[0] holds e = 0..3, s[1] e = 4..7)
-  float sc[8];
-  float mx = -__builtin_inff();
   const int k0 = base + 8 * g;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const int j = k0 + e;
-    const bool vis = j <= col_pos && j >= col_lo;
-    const float v = (e < 4 ? s[0][e] : s[1][e - 4]) * scale_log2;
-    sc[e] = vis ? v : -__builtin_inff();
-    mx = fmaxf(mx, sc[e]);
-  }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-  const float m_new = fmaxf(st.m, mx);
-  // a column that has seen no key yet keeps m = -inf: give it a finite stand-in
-  const float m_use = m_new == -__builtin_inff() ? 0.f : m_new;
-  const float alpha = __builtin_amdgcn_exp2f(st.m - m_use);   // st.m = -inf gives 0
-  float p[8];
-  float psum = 0.f;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    p[e] = __builtin_amdgcn_exp2f(sc[e] - m_use);             // -inf gives 0
-    psum += p[e];
-  }
-  st.l = st.l * alpha + psum;
-  st.m = m_new;
-  const uint4 pb = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]),
-                              pack_bf16(p[6], p[7]));
   // values of keys outside [key_lo, key_hi] may be stale or never written: 0 * garbage must not
-  // reach the accumulator, so such keys are cut out of the V fragment as well
+  // reach the accumulator, so such keys are cut out of the V fragments
   const bool cut_hi = base + 31 > key_hi, cut_lo = base < key_lo;
+  uint4 vf[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
     uint4 a = hp.v[dt];
     if (cut_hi) a = keep_first(a, key_hi - k0 + 1);
     if (cut_lo) a = drop_first(a, key_lo - k0);
-    floatx4_t acc = st.o[dt];
-    acc[0] *= alpha; acc[1] *= alpha; acc[2] *= alpha; acc[3] *= alpha;
-    st.o[dt] = mfma16(as_bf16x8(a), as_bf16x8(pb), acc);
+    vf[dt] = a;
+  }
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    floatx4_t s[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      s[t] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) s[t] = mfma16(as_bf16x8(hp.k[t][ks]), qf[c][ks], s[t]);
+    }
+    // this lane: column lane % 16, keys base + 8 g + e, e = 0..7 (s[0] holds e = 0..3, s[1] e = 4..7)
+    float sc[8];
+    float mx = -__builtin_inff();
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int j = k0 + e;
+      const bool vis = j <= col_pos && j >= col_lo;
+      const float v = (e < 4 ? s[0][e] : s[1][e - 4]) * scale_log2;
+      sc[e] = vis ? v : -__builtin_inff();
+      mx = fmaxf(mx, sc[e]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(st.m[c], mx);
+    // a column that has seen no key yet keeps m = -inf: give it a finite stand-in
+    const float m_use = m_new == -__builtin_inff() ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f(st.m[c] - m_use);   // m = -inf gives 0
+    float p[8];
+    float psum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      p[e] = __builtin_amdgcn_exp2f(sc[e] - m_use);                // -inf gives 0
+      psum += p[e];
+    }
+    st.l[c] = st.l[c] * alpha + psum;
+    st.m[c] = m_new;
+    const uint4 pb = make_uint4(pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3]), pack_bf16(p[4], p[5]),
+                                pack_bf16(p[6], p[7]));
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      floatx4_t acc = st.o[c][dt];
+      acc[0] *= alpha; acc[1] *= alpha; acc[2] *= alpha; acc[3] *= alpha;
+      st.o[c][dt] = mfma16(as_bf16x8(vf[dt]), as_bf16x8(pb), acc);
+    }
   }
 }
 
-// One page (64 keys at absolute positions page_pos .. page_pos+63): both halves' fragments are
-// requested before the first product, so a page costs one round trip to memory.
-__device__ __forceinline__ void attend_page(WaveState &st, const bf16x8_t (&qf)[KS],
+// One page (64 keys at absolute positions page_pos .. page_pos+63).  With one column group and a
+// head size up to 128 both halves' fragments are requested before the first product, so a page
+// costs one round trip to memory; otherwise half by half, to stay within the registers.
+template <int NC>
+__device__ __forceinline__ void attend_page(WaveState<NC> &st, const bf16x8_t (&qf)[NC][KS],
                                             const bf16_t *__restrict__ kp, const bf16_t *__restrict__ vp,
                                             int page_pos, int col_pos, int col_lo, int key_lo, int key_hi,
                                             float scale_log2, int lane) {
   const bool use0 = !(page_pos > key_hi || page_pos + 31 < key_lo);
   const bool use1 = !(page_pos + 32 > key_hi || page_pos + 63 < key_lo);
-  if (HD <= 128) {
+  if (HD <= 128 && NC == 1) {
     HalfPage h0, h1;
     if (use0) load_half(h0, kp, vp, 0, lane);
     if (use1) load_half(h1, kp, vp, 1, lane);
-    if (use0) attend_half(st, qf, h0, page_pos, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
-    if (use1) attend_half(st, qf, h1, page_pos + 32, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
+    if (use0) attend_half<NC>(st, qf, h0, page_pos, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
+    if (use1) attend_half<NC>(st, qf, h1, page_pos + 32, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
   } else {
     HalfPage h;
     if (use0) {
       load_half(h, kp, vp, 0, lane);
-      attend_half(st, qf, h, page_pos, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
+      attend_half<NC>(st, qf, h, page_pos, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
     }
     if (use1) {
       load_half(h, kp, vp, 1, lane);
-      attend_half(st, qf, h, page_pos + 32, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
+      attend_half<NC>(st, qf, h, page_pos + 32, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
     }
   }
 }
@@ -201,8 +221,10 @@ __device__ __forceinline__ void load_q(bf16x8_t (&qf)[KS], const bf16_t *qrow, b
 }
 
 // ---------------------------------------------------------------------------------------------
-// Prefill: a wave takes a tile of up to 16 consecutive rows of one sequence and one query head.
-// tiles: int32 [n_tiles][4] = (first row, rows, sequence, unused).
+// Prefill: a wave takes a tile of up to 16 consecutive rows of one sequence and NC query heads
+// of one kv head.  tiles: int32 [n_tiles][4] = (first row, rows, sequence, unused).
+// Grid: x = groups of four row tiles (one per wave), y = kv head x head tile.
+template <int NC>
 __global__ void __launch_bounds__(256)
 attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
                     const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
@@ -213,8 +235,9 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
   // heavy tiles (late rows, long key ranges) first
   const int tile = n_tiles - 1 - (blockIdx.x * 4 + wave);
   if (tile < 0) return;
-  const int head = blockIdx.y;
-  const int kvh = head / (heads_q / heads_kv);
+  const int group = heads_q / heads_kv;
+  const int head_tiles = (group + NC - 1) / NC;
+  const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y - kvh * head_tiles;
   const int row0 = tiles[tile * 4 + 0], n_rows = tiles[tile * 4 + 1], seq = tiles[tile * 4 + 2];
   const int r = lane & 15, g = lane >> 4;
   const bool col_ok = r < n_rows;
@@ -228,29 +251,40 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
   const int key_lo = (window > 0 && pos_first >= window) ? pos_first - window + 1 : 0;
   const int key_hi = pos_last;
 
-  bf16x8_t qf[KS];
-  load_q(qf, q + (size_t(row) * heads_q + head) * HD, col_ok, lane);
-  WaveState st;
-  init_state(st);
+  bf16x8_t qf[NC][KS];
+  int head[NC];
+  bool head_ok[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int hg = ht * NC + c;                      // query head within the kv head's group
+    head_ok[c] = hg < group;
+    head[c] = kvh * group + (head_ok[c] ? hg : 0);
+    load_q(qf[c], q + (size_t(row) * heads_q + head[c]) * HD, col_ok && head_ok[c], lane);
+  }
+  WaveState<NC> st;
+  init_state<NC>(st);
   const int32_t *pt = page_table + size_t(seq) * max_pages;
   for (int pg = key_lo / SB_PAGE; pg <= key_hi / SB_PAGE; ++pg) {
     const int page = pg < max_pages ? pt[pg] : -1;
     if (page < 0 || page >= n_pages_total) continue;
     const size_t off = (size_t(page) * heads_kv + kvh) * SB_PAGE * HD;
-    attend_page(st, qf, k_cache + off, v_cache + off, pg * SB_PAGE, col_pos, col_lo, key_lo, key_hi,
-                scale_log2, lane);
+    attend_page<NC>(st, qf, k_cache + off, v_cache + off, pg * SB_PAGE, col_pos, col_lo, key_lo, key_hi,
+                    scale_log2, lane);
   }
-  float l = st.l;
-  l += __shfl_xor(l, 16, 64);
-  l += __shfl_xor(l, 32, 64);
-  if (!col_ok) return;
-  const float inv = l > 0.f ? 1.f / l : 0.f;
-  bf16_t *orow = out + (size_t(row) * heads_q + head) * HD;
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) {
-    const uint2 v = make_uint2(pack_bf16(st.o[dt][0] * inv, st.o[dt][1] * inv),
-                               pack_bf16(st.o[dt][2] * inv, st.o[dt][3] * inv));
-    *reinterpret_cast<uint2 *>(orow + dt * 16 + 4 * g) = v;
+  for (int c = 0; c < NC; ++c) {
+    float l = st.l[c];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!col_ok || !head_ok[c]) continue;
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    bf16_t *orow = out + (size_t(row) * heads_q + head[c]) * HD;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const uint2 v = make_uint2(pack_bf16(st.o[c][dt][0] * inv, st.o[c][dt][1] * inv),
+                                 pack_bf16(st.o[c][dt][2] * inv, st.o[c][dt][3] * inv));
+      *reinterpret_cast<uint2 *>(orow + dt * 16 + 4 * g) = v;
+    }
   }
 }
 
@@ -280,28 +314,28 @@ attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *
   const int hq = ht * 16 + r;                 // query head within the group
   const bool col_ok = hq < group;
   const int head = kvh * group + (col_ok ? hq : 0);
-  bf16x8_t qf[KS];
-  load_q(qf, q + (size_t(seq) * heads_q + head) * HD, col_ok, lane);
-  WaveState st;
-  init_state(st);
+  bf16x8_t qf[1][KS];
+  load_q(qf[0], q + (size_t(seq) * heads_q + head) * HD, col_ok, lane);
+  WaveState<1> st;
+  init_state<1>(st);
   const int pg = chunk * kPagesPerChunk + wave;
   if (pg >= key_lo / SB_PAGE && pg <= pos / SB_PAGE && pg < max_pages) {
     const int page = page_table[size_t(seq) * max_pages + pg];
     if (page >= 0 && page < n_pages_total) {
       const size_t off = (size_t(page) * heads_kv + kvh) * SB_PAGE * HD;
-      attend_page(st, qf, k_cache + off, v_cache + off, pg * SB_PAGE, col_ok ? pos : -1, key_lo, key_lo, pos,
-                  scale_log2, lane);
+      attend_page<1>(st, qf, k_cache + off, v_cache + off, pg * SB_PAGE, col_ok ? pos : -1, key_lo, key_lo, pos,
+                     scale_log2, lane);
     }
   }
-  float l = st.l;
+  float l = st.l[0];
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) lds_o[wave][(dt * 16 + 4 * g + i) * 16 + r] = st.o[dt][i];
+    for (int i = 0; i < 4; ++i) lds_o[wave][(dt * 16 + 4 * g + i) * 16 + r] = st.o[0][dt][i];
   if (g == 0) {
-    lds_m[wave][r] = st.m;
+    lds_m[wave][r] = st.m[0];
     lds_l[wave][r] = l;
   }
   __syncthreads();
@@ -425,9 +459,21 @@ extern "C" int sb_attn_prefill_bf16(void *out, const void *q, const void *k_cach
   SB_REQUIRE(tiles && n_tiles >= 0, "sb_attn_prefill_bf16: no tiles");
   if (n_tiles == 0) return SB_OK;
   hipStream_t s = (hipStream_t)stream;
-  dim3 grid((n_tiles + 3) / 4, heads_q);
-  attn_prefill_kernel<<<grid, 256, 0, s>>>((bf16_t *)out, (const bf16_t *)q, (const bf16_t *)k_cache,
-                                           (const bf16_t *)v_cache, page_table, max_pages, n_pages_total,
-                                           row_pos, tiles, n_tiles, heads_q, heads_kv, scale * kLog2e, window);
+  const int group = heads_q / heads_kv;
+  // query heads of a kv head that one wave takes together: each key and value fragment it reads
+  // then feeds that many products
+  const int nc = (group >= 4 && HD <= 128) ? 4 : (group >= 2 ? 2 : 1);
+  const int head_tiles = (group + nc - 1) / nc;
+  SB_SUPPORT(heads_kv * head_tiles <= 65535, "sb_attn_prefill_bf16: too many heads");
+  dim3 grid((n_tiles + 3) / 4, heads_kv * head_tiles);
+#define SB_GO(NC)                                                                                      \
+  attn_prefill_kernel<NC><<<grid, 256, 0, s>>>((bf16_t *)out, (const bf16_t *)q, (const bf16_t *)k_cache, \
+                                               (const bf16_t *)v_cache, page_table, max_pages,           \
+                                               n_pages_total, row_pos, tiles, n_tiles, heads_q, heads_kv, \
+                                               scale * kLog2e, window)
+  if (nc == 4) SB_GO(4);
+  else if (nc == 2) SB_GO(2);
+  else SB_GO(1);
+#undef SB_GO
   return sb::check_launch("sb_attn_prefill_bf16");
 }
