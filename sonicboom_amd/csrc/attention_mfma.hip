@@ -291,13 +291,42 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
 // ---------------------------------------------------------------------------------------------
 // Decode: one row per sequence.  Block (chunk, kv head x head tile, sequence); wave w of the
 // block takes page 4 * chunk + w; columns are the query heads of the kv head.
-// part_o: float [seqs][heads_q][n_chunks][HD], part_ml: float [seqs][heads_q][n_chunks][2].
+//
+// Partial results, when a row's keys span several chunks, go to
+//   part_o  float [seqs][tiles][n_chunks][HD][16]   (unnormalised sums, column fastest)
+//   part_ml float [seqs][tiles][n_chunks][2][16]    (maximum, sum)
+// and are merged in ascending chunk order by attn_decode_merge_kernel.  (Merging in the block
+// that finishes last was tried and dropped: the device-scope fences it needs write back and
+// invalidate whole L2 caches on this multi-die GPU and cost far more than the second launch.)
+// Element e = d * 16 + column of a (sequence, tile): the chunks' partial sums, rescaled to the
+// common maximum and added in ascending chunk order.
+__device__ __forceinline__ void merge_element(bf16_t *__restrict__ out, const float *__restrict__ po,
+                                              const float *__restrict__ pml, int e, int first, int last,
+                                              int seq, int heads_q, int kvh, int ht, int group) {
+  const int c = e & 15, d = e >> 4;
+  const int hh = ht * 16 + c;
+  if (hh >= group) return;
+  float m = -__builtin_inff();
+#pragma unroll 4
+  for (int ch = first; ch <= last; ++ch) m = fmaxf(m, pml[size_t(ch) * 32 + c]);
+  const float m_use = m == -__builtin_inff() ? 0.f : m;
+  float o = 0.f, l = 0.f;
+#pragma unroll 4
+  for (int ch = first; ch <= last; ++ch) {
+    const float f = __builtin_amdgcn_exp2f(pml[size_t(ch) * 32 + c] - m_use);
+    o += po[size_t(ch) * (HD * 16) + e] * f;
+    l += pml[size_t(ch) * 32 + 16 + c] * f;
+  }
+  out[(size_t(seq) * heads_q + kvh * group + hh) * HD + d] = f32_to_bf16(l > 0.f ? o / l : 0.f);
+}
+
 __global__ void __launch_bounds__(256)
 attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
-                   const bf16_t *__restrict__ q, const bf16_t *__restrict__ k_cache,
-                   const bf16_t *__restrict__ v_cache, const int32_t *__restrict__ page_table,
-                   int max_pages, int n_pages_total, const int32_t *__restrict__ row_pos, int heads_q,
-                   int heads_kv, int n_chunks, float scale_log2, int window) {
+                   const bf16_t *__restrict__ q,
+                   const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
+                   const int32_t *__restrict__ page_table, int max_pages, int n_pages_total,
+                   const int32_t *__restrict__ row_pos, int heads_q, int heads_kv, int n_chunks,
+                   float scale_log2, int window) {
   __shared__ float lds_o[4][HD * 16];   // [wave][d][col]
   __shared__ float lds_m[4][16], lds_l[4][16];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -307,7 +336,8 @@ attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *
   const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y - kvh * head_tiles;
   const int pos = row_pos[seq];
   const int key_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
-  const int first_chunk = key_lo / (SB_PAGE * kPagesPerChunk), last_chunk = pos / (SB_PAGE * kPagesPerChunk);
+  const int first_chunk = key_lo / (SB_PAGE * kPagesPerChunk);
+  const int last_chunk = min(pos / (SB_PAGE * kPagesPerChunk), n_chunks - 1);
   if (chunk < first_chunk || chunk > last_chunk) return;   // uniform over the block
 
   const int r = lane & 15, g = lane >> 4;
@@ -339,11 +369,13 @@ attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *
     lds_l[wave][r] = l;
   }
   __syncthreads();
-  // merge the four waves (pages in ascending order); thread e owns (d, col)
+  // merge the four waves (pages in ascending order); thread e owns (d, col), column fastest
+  const bool alone = first_chunk == last_chunk;
+  const size_t tile_index = size_t(seq) * gridDim.y + blockIdx.y;
+  float *po = part_o + (tile_index * n_chunks) * (HD * 16);
+  float *pml = part_ml + (tile_index * n_chunks) * 32;
   for (int e = threadIdx.x; e < HD * 16; e += 256) {
     const int c = e & 15, d = e >> 4;
-    const int hh = ht * 16 + c;
-    if (hh >= group) continue;
     float m = -__builtin_inff();
 #pragma unroll
     for (int w = 0; w < 4; ++w) m = fmaxf(m, lds_m[w][c]);
@@ -355,42 +387,39 @@ attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *
       o += lds_o[w][e] * f;
       lsum += lds_l[w][c] * f;
     }
-    const int oh = kvh * group + hh;
-    if (n_chunks == 1) {
-      out[(size_t(seq) * heads_q + oh) * HD + d] = f32_to_bf16(lsum > 0.f ? o / lsum : 0.f);
-    } else {
-      const size_t pi = (size_t(seq) * heads_q + oh) * n_chunks + chunk;
-      part_o[pi * HD + d] = o;
+    if (alone) {
+      const int hh = ht * 16 + c;
+      if (hh < group)
+        out[(size_t(seq) * heads_q + kvh * group + hh) * HD + d] = f32_to_bf16(lsum > 0.f ? o / lsum : 0.f);
+    } else if (ht * 16 + c < group) {
+      po[size_t(chunk) * (HD * 16) + e] = o;
       if (d == 0) {
-        part_ml[pi * 2 + 0] = m;
-        part_ml[pi * 2 + 1] = lsum;
+        pml[size_t(chunk) * 32 + c] = m;
+        pml[size_t(chunk) * 32 + 16 + c] = lsum;
       }
     }
   }
 }
 
-// Merge the chunks of a (sequence, head) in ascending order.
-__global__ void attn_decode_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o,
-                                         const float *__restrict__ part_ml,
-                                         const int32_t *__restrict__ row_pos, int heads_q, int n_chunks,
-                                         int window) {
-  const int seq = blockIdx.y, head = blockIdx.x;
+// Merge the chunks of a (sequence, tile) in ascending order: one thread per (d, column).
+// Grid (HD * 16 / 256, tiles, sequences).
+__global__ void __launch_bounds__(256)
+attn_decode_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o,
+                         const float *__restrict__ part_ml, const int32_t *__restrict__ row_pos,
+                         int heads_q, int heads_kv, int n_chunks, int window) {
+  const int seq = blockIdx.z;
+  const int group = heads_q / heads_kv;
+  const int head_tiles = (group + 15) / 16;
+  const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y - kvh * head_tiles;
   const int pos = row_pos[seq];
   const int key_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
   const int first = key_lo / (SB_PAGE * kPagesPerChunk), last = min(pos / (SB_PAGE * kPagesPerChunk), n_chunks - 1);
-  const size_t base = (size_t(seq) * heads_q + head) * n_chunks;
-  float m = -__builtin_inff();
-  for (int c = first; c <= last; ++c) m = fmaxf(m, part_ml[(base + c) * 2]);
-  const float m_use = m == -__builtin_inff() ? 0.f : m;
-  for (int d = threadIdx.x; d < HD; d += blockDim.x) {
-    float o = 0.f, l = 0.f;
-    for (int c = first; c <= last; ++c) {
-      const float f = __builtin_amdgcn_exp2f(part_ml[(base + c) * 2] - m_use);
-      o += part_o[(base + c) * HD + d] * f;
-      l += part_ml[(base + c) * 2 + 1] * f;
-    }
-    out[(size_t(seq) * heads_q + head) * HD + d] = f32_to_bf16(l > 0.f ? o / l : 0.f);
-  }
+  if (first == last) return;      // the decode kernel has written the result itself
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= HD * 16) return;
+  const size_t tile_index = size_t(seq) * gridDim.y + blockIdx.y;
+  merge_element(out, part_o + (tile_index * n_chunks) * (HD * 16), part_ml + (tile_index * n_chunks) * 32, e,
+                first, last, seq, heads_q, kvh, ht, group);
 }
 
 int check_common(const void *out, const void *q, const void *k, const void *v, const void *pt,
@@ -415,10 +444,19 @@ extern "C" int sb_attn_decode_chunks(int max_pages) {
   return (max_pages + kPagesPerChunk - 1) / kPagesPerChunk;
 }
 
+// Floats of part_o and of part_ml that sb_attn_decode_bf16 needs for these sizes.
+extern "C" size_t sb_attn_decode_part_o(int n_seqs, int heads_q, int heads_kv, int max_pages) {
+  const int tiles = heads_kv * ((heads_q / heads_kv + 15) / 16);
+  return size_t(n_seqs) * tiles * sb_attn_decode_chunks(max_pages) * HD * 16;
+}
+extern "C" size_t sb_attn_decode_part_ml(int n_seqs, int heads_q, int heads_kv, int max_pages) {
+  const int tiles = heads_kv * ((heads_q / heads_kv + 15) / 16);
+  return size_t(n_seqs) * tiles * sb_attn_decode_chunks(max_pages) * 32;
+}
+
 // q, out: bf16 [n_seqs, heads_q * HD], one row per sequence; k_cache bf16 [pages][heads_kv][64][HD],
-// v_cache bf16 [pages][heads_kv][HD][64].  part_o float [n_seqs * heads_q * chunks * HD] and part_ml
-// float [n_seqs * heads_q * chunks * 2] with chunks = sb_attn_decode_chunks(max_pages) (unused, may be
-// NULL, when chunks == 1).
+// v_cache bf16 [pages][heads_kv][HD][64].  part_o / part_ml: float buffers of the sizes the two
+// functions above give (may be NULL when max_pages fits one chunk).
 extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
                                    const int32_t *page_table, int max_pages, int n_pages_total,
                                    const int32_t *row_pos, float *part_o, float *part_ml, int n_seqs,
@@ -442,8 +480,8 @@ extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache
                                           scale * kLog2e, window);
   rc = sb::check_launch("sb_attn_decode_bf16");
   if (rc != SB_OK || n_chunks == 1) return rc;
-  attn_decode_merge_kernel<<<dim3(heads_q, n_seqs), HD < 64 ? 64 : HD, 0, s>>>(
-      (bf16_t *)out, part_o, part_ml, row_pos, heads_q, n_chunks, window);
+  attn_decode_merge_kernel<<<dim3((HD * 16 + 255) / 256, heads_kv * head_tiles, n_seqs), 256, 0, s>>>(
+      (bf16_t *)out, part_o, part_ml, row_pos, heads_q, heads_kv, n_chunks, window);
   return sb::check_launch("sb_attn_decode_bf16 (merge)");
 }
 

@@ -229,16 +229,24 @@ Plan plan_for(int n_rows, int n_out, int n_in, int gated) {
   Plan p;
   p.TT = n_rows <= 16 ? 1 : (n_rows <= 32 ? 2 : 4);
   const int tiles = (n_out + 15) / 16;
-  // measured on MI355X: one row tile per block streams best up to 16 rows; more rows reuse each
-  // X fragment for several row tiles
-  p.R = p.TT == 1 ? 1 : (tiles >= 2048 ? 4 : (tiles >= 1024 ? 2 : 1));
-  if (gated && p.R == 4) p.R = 2;   // gate and up double the fragments a wave holds
+  // Measured on MI355X.  Up to 16 rows: one row tile per block streams best, and K is cut
+  // into slices until about a thousand blocks exist.  More rows: every X fragment a wave loads
+  // must serve several row tiles (it comes from L2, and there are TT of them per W fragment), so
+  // a wave takes four row tiles (two gated pairs) and fewer, fatter blocks are better.
+  const int n_steps = (n_in + kStepK - 1) / kStepK;
+  int want_blocks;
+  if (p.TT == 1) {
+    p.R = 1;
+    want_blocks = 1024;
+  } else {
+    p.R = gated ? 2 : 4;
+    want_blocks = 224;
+  }
   if (g_force_r) p.R = g_force_r;
   const int blocks = (tiles + p.R - 1) / p.R;
-  const int n_steps = (n_in + kStepK - 1) / kStepK;
   int slices = 1;
-  if (blocks < 1024) {
-    slices = (1024 + blocks - 1) / blocks;
+  if (blocks < want_blocks) {
+    slices = (want_blocks + blocks - 1) / blocks;
     const int most = n_steps / (kWaves * 4);   // every wave keeps at least four steps
     if (slices > most) slices = most;
     if (slices > 8) slices = 8;     // what the kernels that add the slices take

@@ -409,11 +409,13 @@ def attention_decode_mfma(q, k_cache, v_cache, page_table, seq_pos, heads_q, hea
     out = torch.empty_like(q)
     part_o = part_ml = None
     if chunks > 1:
-        part_o = torch.empty((n * heads_q * chunks * head_dim,), dtype=torch.float32, device=q.device)
-        part_ml = torch.empty((n * heads_q * chunks * 2,), dtype=torch.float32, device=q.device)
+        part_o = torch.empty((lib.sb_attn_decode_part_o(n, heads_q, heads_kv, max_pages),), dtype=torch.float32,
+                             device=q.device)
+        part_ml = torch.empty((lib.sb_attn_decode_part_ml(n, heads_q, heads_kv, max_pages),), dtype=torch.float32,
+                              device=q.device)
     check(lib.sb_attn_decode_bf16(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(page_table), max_pages,
-                                  k_cache.shape[0], _p(seq_pos), _p(part_o), _p(part_ml), n, heads_q, heads_kv,
-                                  float(scale), int(window), _stream()), lib, "sb_attn_last_error")
+                                  k_cache.shape[0], _p(seq_pos), _p(part_o), _p(part_ml), n, heads_q,
+                                  heads_kv, float(scale), int(window), _stream()), lib, "sb_attn_last_error")
     return out
 
 

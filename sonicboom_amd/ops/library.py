@@ -105,6 +105,9 @@ def attention_library(head_dim: int):
                     raise KernelLibraryError(f"cannot load the attention kernels for head size {head_dim}: {e}") from e
                 lib.sb_attn_last_error.restype = c_char_p
                 _declare(lib, _ATTN_SIGNATURES)
+                for fn in (lib.sb_attn_decode_part_o, lib.sb_attn_decode_part_ml):
+                    fn.argtypes = [_I, _I, _I, _I]
+                    fn.restype = c_size_t
                 lib._sb_path = path
                 _attn[head_dim] = lib
     return lib

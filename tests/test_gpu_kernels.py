@@ -317,6 +317,9 @@ def test_attention_decode_matrix_cores(hq, hkv, hd, window):
     pos = torch.tensor([p for _, p in rows], dtype=torch.int32)
     got = ops.attention_decode_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), hq, hkv, hd, scale, window)
     close(got, want, atol=1.5e-2, rtol=1e-2, what="decode")
+    for _ in range(3):                       # launch after launch, the same bits
+        again = ops.attention_decode_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), hq, hkv, hd, scale, window)
+        assert torch.equal(got, again)
 
 
 @pytest.mark.parametrize("hq, hkv, hd", MFMA_SHAPES)
