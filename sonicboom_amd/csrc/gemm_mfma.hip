@@ -2,27 +2,26 @@
 // on the matrix cores, with the model's epilogues fused: bias, float32
 // residual, SiLU gate, float32 or bfloat16 output.
 //
-// A block of 256 threads (2 x 2 waves) owns a 128 x 128 tile of Y and walks K
-// in steps of 64.  Both operand tiles go global -> registers -> LDS, the next
-// step's loads being issued before the current step's MFMAs (two LDS buffers,
-// one barrier per step).  An LDS row holds 64 k (128 bytes, eight 16-byte
-// chunks); chunk c of row r is stored at chunk c ^ (r & 7), which makes the
-// 16-byte fragment reads of eight consecutive lanes fall on distinct banks.
-// A wave owns 64 x 64: 2 x 2 tiles of v_mfma_f32_32x32x16_bf16, A = rows of X,
-// B = rows of W, so a lane holds one output column of 16 rows.
+// A block of 256 threads (2 x 2 waves) owns a BM x 128 tile of Y (BM = 128 or
+// 256 rows) and walks K in stages of BK (32 or 64).  Both operand tiles go
+// global -> registers -> LDS, the next stage's loads being issued before the
+// current stage's MFMAs (two LDS buffers, one barrier per stage).  An LDS row
+// holds BK k (BK / 8 chunks of 16 bytes); chunk c of row r is stored at chunk
+// c ^ f(r), f chosen so that the 16-byte fragment reads of sixteen consecutive
+// rows fall on distinct banks.  A wave owns (BM / 2) x 64: MT x 2 tiles of
+// v_mfma_f32_32x32x16_bf16, A = rows of X, B = rows of W, so a lane holds one
+// output column of 16 rows.  The taller tile halves the LDS reads per MFMA;
+// the launcher picks it when the grid still fills the chip.
 //
 // Block order: consecutive block numbers go to different XCDs (each with its
 // own L2).  The grid is walked so that the blocks one XCD runs at a time share
 // their X rows and neighbouring W rows.
+#include <type_traits>
+
 #include "mfma.cuh"
 
 namespace {
 
-constexpr int BM = 128, BN = 128, BK = 64;
-constexpr int kThreads = 256;
-constexpr int kChunksPerRow = BK / 8;                       // 16-byte chunks in an LDS row
-constexpr int kLoadsA = BM * kChunksPerRow / kThreads;      // 4
-constexpr int kLoadsB = BN * kChunksPerRow / kThreads;      // 4
 constexpr int kXcds = 8;
 
 struct Args {
@@ -39,17 +38,33 @@ struct Args {
   int w_steps;     // packed W: 32-wide k-steps (ceil(n_in / 32))
 };
 
-__device__ __forceinline__ int swz(int row, int chunk) { return row * kChunksPerRow + (chunk ^ (row & 7)); }
+// index (in 16-byte chunks) of chunk `chunk` of LDS row `row`, CPR chunks per row
+template <int CPR>
+__device__ __forceinline__ int swz(int row, int chunk) {
+  return row * CPR + (chunk ^ ((row / (16 / CPR)) & (CPR - 1)));
+}
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
 // PACKED: W comes in the packed tile layout (1 KB blocks of 16 rows x 32 k in fragment order,
 // zero padded), which makes its global loads contiguous and free of bounds checks.
-template <int GATED, bool PACKED>
-__global__ void __launch_bounds__(kThreads)
+// MT: 32-row tiles of a wave (the block has two waves along M), NW: waves along N (64 columns
+// each), DEPTH: stages the global loads run ahead of the products.
+template <int MT, int NW, int BK, int DEPTH, int GATED, bool PACKED, bool EVEN_K>
+__global__ void __launch_bounds__(128 * NW)
 gemm_mfma_kernel(Args a) {
-  __shared__ uint4 lds_a[2][BM * kChunksPerRow];
-  __shared__ uint4 lds_b[2][BN * kChunksPerRow];
+  constexpr int BM = 64 * MT, BN = 64 * NW, kThreads = 128 * NW;
+  constexpr int CPR = BK / 8;                       // 16-byte chunks in an LDS row
+  constexpr int kLoadsA = BM * CPR / kThreads;
+  constexpr int kLoadsB = BN * CPR / kThreads;
+  constexpr int kLoads = kLoadsA + kLoadsB;
+  constexpr int kSteps32 = BK / 32;                 // packed k-steps in a stage
+  constexpr int kSteps16 = BK / 16;                 // MFMA k-steps in a stage
+  constexpr int kMfmas = 2 * MT;                    // MFMAs of a wave per k-step
+  // 16-byte chunks travel as first-class vectors, so the staging arrays stay in registers
+  extern __shared__ bf16x8_t lds[];
+  bf16x8_t *lds_a0 = lds, *lds_a1 = lds + BM * CPR;
+  bf16x8_t *lds_b0 = lds + 2 * BM * CPR, *lds_b1 = lds_b0 + BN * CPR;
 
   // XCD-aware order: hardware sends block b to XCD b % 8.  When the count divides, XCD x
   // gets the contiguous run of tiles [x * per, (x + 1) * per), which share rows of X and W in
@@ -63,29 +78,39 @@ gemm_mfma_kernel(Args a) {
   const int n0 = tn * (GATED ? BN / 2 : BN);
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / NW, wn = wave % NW;
 
-  // global -> register staging: thread handles chunk ids tid + 256 * i
-  const bf16_t *ga[kLoadsA];
-  const bf16_t *gb[kLoadsB];
-  bool oka[kLoadsA], okb[kLoadsB];
-  int sa[kLoadsA], sb_[kLoadsB], ca[kLoadsA], cb[kLoadsB];
+  // Global -> register staging: load i of a thread takes chunk id tid + kThreads * i of the
+  // stage.  Buffer loads: a descriptor per operand in scalar registers, one 32-bit byte offset
+  // per load, the stage's offset along K as the scalar offset; what lies past the operand's end
+  // reads as zero, which covers the rows past the last one.  Chunks past the end of K inside a
+  // row have to be zeroed by hand (EVEN_K: there are none).  Load i + 1 lands kThreads chunks
+  // after load i in LDS (its rows are a multiple of 16 further on, so the swizzle term repeats).
+  static_assert((kThreads / CPR) % 16 == 0, "rows per load must keep the swizzle term");
+  uint32_t off[kLoads];       // byte offset of the load at stage 0
+  int kpos[kLoads];           // !EVEN_K: first k of the chunk within the stage (packed: of its k-step)
+  int slot_a0, slot_b0;       // LDS chunk index of loads 0 of A and of B
+  const size_t w_rows_total = size_t(GATED ? 2 : 1) * (PACKED ? size_t(a.w_tiles) * 16 : size_t(a.n_out));
+  const size_t w_row_bytes = PACKED ? size_t(a.w_steps) * 64 : size_t(a.n_in) * 2;
+  const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<bf16_t *>(a.x), 0, uint32_t(size_t(a.n_rows) * a.n_in * 2), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrc_w = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<bf16_t *>(a.w), 0, uint32_t(w_rows_total * w_row_bytes), 0x00020000);
 #pragma unroll
   for (int i = 0; i < kLoadsA; ++i) {
-    const int id = tid + kThreads * i, row = id / kChunksPerRow, c = id % kChunksPerRow;
-    const int t = t0 + row;
-    oka[i] = t < a.n_rows;
-    ga[i] = a.x + size_t(min(t, a.n_rows - 1)) * a.n_in + c * 8;
-    sa[i] = swz(row, c);
-    ca[i] = c * 8;
+    const int id = tid + kThreads * i, row = id / CPR, c = id % CPR;
+    const int t = min(t0 + row, a.n_rows);          // n_rows: one past the end, reads zeros
+    off[i] = uint32_t((size_t(t) * a.n_in + c * 8) * 2);
+    if (i == 0) slot_a0 = swz<CPR>(row, c);
+    kpos[i] = c * 8;
   }
-  int step_b[kLoadsB];    // packed: which of the two k-steps of a BK stage this load takes
 #pragma unroll
   for (int i = 0; i < kLoadsB; ++i) {
+    const int id = tid + kThreads * i;
     if (PACKED) {
       // load id -> 1 KB block (id / 64) = (row tile of the LDS tile, k-step), lane id % 64
-      const int id = tid + kThreads * i, blk = id >> 6, l = id & 63;
-      const int rt = blk >> 1, j = blk & 1;      // LDS rows rt * 16 .., k-step j of the stage
+      const int blk = id >> 6, l = id & 63;
+      const int rt = blk / kSteps32, j = blk % kSteps32;   // LDS rows rt * 16 .., k-step j of the stage
       int tile;
       if (GATED) {
         const int half = rt >> 2, within = rt & 3;
@@ -93,95 +118,162 @@ gemm_mfma_kernel(Args a) {
       } else {
         tile = min(n0 / 16 + rt, a.w_tiles - 1);
       }
-      okb[i] = true;
-      gb[i] = a.w + size_t(tile) * a.w_steps * 512 + size_t(l) * 8;
-      sb_[i] = swz(rt * 16 + (l & 15), j * 4 + (l >> 4));
-      cb[i] = 0;
-      step_b[i] = j;
-      continue;
-    }
-    step_b[i] = 0;
-    const int id = tid + kThreads * i, row = id / kChunksPerRow, c = id % kChunksPerRow;
-    int n;       // output feature, and the row of W that feeds LDS row `row`
-    int wrow;
-    if (GATED) {
-      // LDS rows [0,32) gate of features n0..n0+31, [32,64) up of the same, [64,96) gate of
-      // n0+32.., [96,128) up of the same: a wave's two B tiles are gate and up of 32 features.
-      const int half = row >> 6, within = row & 63, is_up = within >> 5;
-      n = n0 + half * 32 + (within & 31);
-      wrow = is_up * a.n_out + n;
+      off[kLoadsA + i] = uint32_t(((size_t(tile) * a.w_steps + j) * 512 + size_t(l) * 8) * 2);
+      if (i == 0) slot_b0 = swz<CPR>(rt * 16 + (l & 15), j * 4 + (l >> 4));
+      kpos[kLoadsA + i] = j * 32;
     } else {
-      n = n0 + row;
-      wrow = n;
+      const int row = id / CPR, c = id % CPR;
+      int wrow;       // the row of W that feeds LDS row `row`
+      if (GATED) {
+        // LDS rows [0,32) gate of features n0..n0+31, [32,64) up of the same, [64,96) gate of
+        // n0+32.., [96,128) up of the same: a wave's two B tiles are gate and up of 32 features.
+        const int half = row >> 6, within = row & 63, is_up = within >> 5;
+        wrow = is_up * a.n_out + min(n0 + half * 32 + (within & 31), a.n_out - 1);
+      } else {
+        wrow = min(n0 + row, a.n_out - 1);
+      }
+      off[kLoadsA + i] = uint32_t((size_t(wrow) * a.n_in + c * 8) * 2);
+      if (i == 0) slot_b0 = swz<CPR>(row, c);
+      kpos[kLoadsA + i] = c * 8;
     }
-    okb[i] = n < a.n_out;
-    gb[i] = a.w + size_t(okb[i] ? wrow : 0) * a.n_in + c * 8;
-    sb_[i] = swz(row, c);
-    cb[i] = c * 8;
   }
 
-  floatx16_t acc[2][2];
+  floatx16_t acc[MT][2];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < MT; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
 
-  uint4 ra[kLoadsA], rb[kLoadsB];
-  auto load_global = [&](int k0) {
-#pragma unroll
-    for (int i = 0; i < kLoadsA; ++i) ra[i] = ld16(ga[i] + k0, oka[i] && (k0 + ca[i]) < a.n_in);
-#pragma unroll
-    for (int i = 0; i < kLoadsB; ++i) {
-      if (PACKED) {
-        const int ks = k0 / 32 + step_b[i];
-        rb[i] = ld16(gb[i] + size_t(ks) * 512, ks < a.w_steps);
-      } else {
-        rb[i] = ld16(gb[i] + k0, okb[i] && (k0 + cb[i]) < a.n_in);
-      }
+  // DEPTH 2, two register sets: while stage kt is multiplied out of LDS, stage kt + 1 waits in
+  // one set (its loads went out a stage earlier) and the loads of stage kt + 2 go out into the
+  // other.  DEPTH 1, one set: the loads of stage kt + 1 go out in the first half of stage kt.
+  bf16x8_t staged[DEPTH][kLoads];
+  typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+  auto issue_load = [&](auto SET, int i, int kt) {
+    constexpr int set = decltype(SET)::value;
+    const bool is_a = i < kLoadsA;
+    // uniform part of the address: the stage's offset along K
+    const int stage_off = (PACKED && !is_a) ? kt * (kSteps32 * 1024) : kt * (BK * 2);
+    bf16x8_t v = __builtin_bit_cast(
+        bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(is_a ? rsrc_x : rsrc_w, int(off[i]), stage_off, 0));
+    if (!EVEN_K) {
+      const bool ok = (PACKED && !is_a) ? (kt * BK + kpos[i] < a.w_steps * 32) : (kt * BK + kpos[i] < a.n_in);
+      if (!ok) v = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
     }
+    staged[set][i] = v;
   };
-  auto store_lds = [&](int buf) {
-#pragma unroll
-    for (int i = 0; i < kLoadsA; ++i) lds_a[buf][sa[i]] = ra[i];
-#pragma unroll
-    for (int i = 0; i < kLoadsB; ++i) lds_b[buf][sb_[i]] = rb[i];
+  auto store_lds = [&](auto SET, int i, int buf) {
+    constexpr int set = decltype(SET)::value;
+    if (i < kLoadsA) (buf ? lds_a1 : lds_a0)[slot_a0 + i * kThreads] = staged[set][i];
+    else (buf ? lds_b1 : lds_b0)[slot_b0 + (i - kLoadsA) * kThreads] = staged[set][i];
   };
 
   const int n_k = (a.n_in + BK - 1) / BK;
-  load_global(0);
-  store_lds(0);
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+#pragma unroll
+  for (int i = 0; i < kLoads; ++i) issue_load(Set0{}, i, 0);
+  if (DEPTH == 2 && n_k > 1) {
+#pragma unroll
+    for (int i = 0; i < kLoads; ++i) issue_load(std::integral_constant<int, DEPTH - 1>{}, i, 1);
+  }
+#pragma unroll
+  for (int i = 0; i < kLoads; ++i) store_lds(Set0{}, i, 0);
   __syncthreads();
 
-  const int frag_row = lane & 31, frag_c = lane >> 5;   // row within a 32-row tile, chunk within a k16 step
-  for (int kt = 0; kt < n_k; ++kt) {
-    const int buf = kt & 1;
-    if (kt + 1 < n_k) load_global((kt + 1) * BK);
+  // fragment reads: lane -> row lane % 32 of a 32-row tile, chunk 2 * ks + lane / 32 of the stage
+  const int frag_row = lane & 31, frag_c = lane >> 5;
+  const int frag_sw = (frag_row / (16 / CPR)) & (CPR - 1);     // swizzle term, equal for all tiles of a wave
+  const int a_row0 = (wm * (32 * MT) + frag_row) * CPR, b_row0 = (wn * 64 + frag_row) * CPR;
+
+  // One stage.  CUR: LDS buffer of this stage (and with two register sets the free one); LOAD: the
+  // stage to load (kt + DEPTH) exists, STORE: stage kt + 1 exists.  The memory operations are spread between the MFMAs in the source
+  // so that the matrix pipe keeps running while they issue.
+  auto stage = [&](auto CUR, auto LOAD, auto STORE, int kt) {
+    constexpr int cur = decltype(CUR)::value;
+    constexpr bool do_load = decltype(LOAD)::value, do_store = decltype(STORE)::value;
+    using SetCur = std::integral_constant<int, DEPTH == 2 ? cur : 0>;          // set to load into
+    using SetNext = std::integral_constant<int, DEPTH == 2 ? (cur ^ 1) : 0>;   // set to store from
+    const bf16x8_t *la = cur ? lds_a1 : lds_a0, *lb = cur ? lds_b1 : lds_b0;
+    bf16x8_t frag[2][MT + 2];
+    auto read_frag = [&](int fs, int ks, int f) {
+      const int c = (ks * 2 + frag_c) ^ frag_sw;
+      frag[fs][f] = f < MT ? la[a_row0 + f * 32 * CPR + c] : lb[b_row0 + (f - MT) * 32 * CPR + c];
+    };
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      const int c = ks * 2 + frag_c;
-      bf16x8_t fa[2], fb[2];
+    for (int f = 0; f < MT + 2; ++f) read_frag(0, 0, f);
+    constexpr int kSlots = kSteps16 * kMfmas;           // MFMAs of the stage = places to put other work
+    constexpr int kHalf = kSlots / 2;
 #pragma unroll
-      for (int i = 0; i < 2; ++i) fa[i] = as_bf16x8(lds_a[buf][swz(wm * 64 + i * 32 + frag_row, c)]);
+    for (int ks = 0; ks < kSteps16; ++ks) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) fb[j] = as_bf16x8(lds_b[buf][swz(wn * 64 + j * 32 + frag_row, c)]);
+      for (int m = 0; m < kMfmas; ++m) {
+        const int i = m >> 1, j = m & 1, at = ks * kMfmas + m;
+        acc[i][j] = mfma32(frag[ks & 1][i], frag[ks & 1][MT + j], acc[i][j]);
+        // fragments of the next k-step, one read after each of the first MFMAs
+        if (ks + 1 < kSteps16 && m < MT + 2) read_frag((ks + 1) & 1, ks + 1, m);
+        // loads of stage kt + DEPTH over the first half of the stage
+        if (do_load && at < kHalf) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+          for (int l = 0; l < kLoads; ++l)
+            if (l >= at * kLoads / kHalf && l < (at + 1) * kLoads / kHalf) issue_load(SetCur{}, l, kt + DEPTH);
+        }
+        // stage kt + 1 into the other LDS buffer over the second half: nobody reads that buffer
+        // since the last barrier
+        if (do_store && at >= kHalf) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = mfma32(fa[i], fb[j], acc[i][j]);
+          for (int l = 0; l < kLoads; ++l)
+            if (l >= (at - kHalf) * kLoads / kHalf && l < (at - kHalf + 1) * kLoads / kHalf)
+              store_lds(SetNext{}, l, cur ^ 1);
+        }
+        // keep this order: left alone, the scheduler gathers the memory operations into lumps
+        // and reads each fragment right before its MFMA, and the matrix pipe waits on both
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
-    if (kt + 1 < n_k) store_lds(buf ^ 1);
     __syncthreads();
+  };
+  using Yes = std::true_type;
+  using No = std::false_type;
+  int kt = 0;
+  if (DEPTH == 2) {
+    for (; kt + 3 < n_k; kt += 2) {
+      stage(Set0{}, Yes{}, Yes{}, kt);
+      stage(Set1{}, Yes{}, Yes{}, kt + 1);
+    }
+    const int rest = n_k - kt;
+    if (rest == 3) {
+      stage(Set0{}, Yes{}, Yes{}, kt);
+      stage(Set1{}, No{}, Yes{}, kt + 1);
+      stage(Set0{}, No{}, No{}, kt + 2);
+    } else if (rest == 2) {
+      stage(Set0{}, No{}, Yes{}, kt);
+      stage(Set1{}, No{}, No{}, kt + 1);
+    } else if (rest == 1) {
+      stage(Set0{}, No{}, No{}, kt);
+    }
+  } else {
+    for (; kt + 2 < n_k; kt += 2) {
+      stage(Set0{}, Yes{}, Yes{}, kt);
+      stage(Set1{}, Yes{}, Yes{}, kt + 1);
+    }
+    if (n_k - kt == 2) {
+      stage(Set0{}, Yes{}, Yes{}, kt);
+      stage(Set1{}, No{}, No{}, kt + 1);
+    } else {
+      stage(Set0{}, No{}, No{}, kt);
+    }
   }
 
   // Epilogue.  acc[i][j][e]: row = 8 * (e / 4) + 4 * (lane / 32) + e % 4, column = lane % 32.
   const int col = lane & 31, row_base = (lane >> 5) * 4;
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
+  for (int i = 0; i < MT; ++i) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      const int t = t0 + wm * 64 + i * 32 + 8 * (e >> 2) + row_base + (e & 3);
+      const int t = t0 + wm * (32 * MT) + i * 32 + 8 * (e >> 2) + row_base + (e & 3);
       if (t >= a.n_rows) continue;
       if (GATED) {
         const int n = n0 + wn * 32 + col;
@@ -208,6 +300,60 @@ gemm_mfma_kernel(Args a) {
   }
 }
 
+constexpr int kCus = 256;
+int g_force_variant = -1;
+
+template <int MT, int NW, int BK, int DEPTH, int GATED, bool PACKED, bool EVEN_K>
+int launch_one(const Args &a, long long blocks, hipStream_t s) {
+  constexpr int lds_bytes = 2 * (64 * MT + 64 * NW) * (BK / 8) * 16;
+  static bool raised = false;     // per instantiation; harmless if repeated
+  if (lds_bytes > 48 * 1024 && !raised) {
+    const hipError_t e =
+        hipFuncSetAttribute((const void *)gemm_mfma_kernel<MT, NW, BK, DEPTH, GATED, PACKED, EVEN_K>,
+                            hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
+    SB_REQUIRE(e == hipSuccess, "sb_gemm_mfma_bf16: cannot reserve %d bytes of LDS: %s", lds_bytes,
+               hipGetErrorString(e));
+    raised = true;
+  }
+  gemm_mfma_kernel<MT, NW, BK, DEPTH, GATED, PACKED, EVEN_K><<<unsigned(blocks), 128 * NW, lds_bytes, s>>>(a);
+  return SB_OK;
+}
+
+template <int MT, int NW, int BK, int DEPTH>
+int launch(const Args &a, long long blocks, int packed, hipStream_t s) {
+  const int which = (a.gated ? 4 : 0) + (packed ? 2 : 0) + (a.n_in % BK == 0 ? 1 : 0);
+  switch (which) {
+    case 7: return launch_one<MT, NW, BK, DEPTH, 1, true, true>(a, blocks, s);
+    case 6: return launch_one<MT, NW, BK, DEPTH, 1, true, false>(a, blocks, s);
+    case 5: return launch_one<MT, NW, BK, DEPTH, 1, false, true>(a, blocks, s);
+    case 4: return launch_one<MT, NW, BK, DEPTH, 1, false, false>(a, blocks, s);
+    case 3: return launch_one<MT, NW, BK, DEPTH, 0, true, true>(a, blocks, s);
+    case 2: return launch_one<MT, NW, BK, DEPTH, 0, true, false>(a, blocks, s);
+    case 1: return launch_one<MT, NW, BK, DEPTH, 0, false, true>(a, blocks, s);
+    default: return launch_one<MT, NW, BK, DEPTH, 0, false, false>(a, blocks, s);
+  }
+}
+
+// Tile shapes the launcher chooses from: rows x columns of Y per block.
+struct Shape { int bm, bn; };
+constexpr Shape kShapes[3] = {{128, 128}, {256, 128}, {256, 256}};
+
+// Rough cost of a shape for a problem: rounds of the grid over the CUs times the work of a block,
+// the bigger tiles getting credit for the operand traffic they save.
+int pick_shape(int n_rows, int n_out, int gated) {
+  double best = 0;
+  int pick = 0;
+  const double speed[3] = {1.0, 1.2, 1.3};    // measured rate of a full grid, relative
+  for (int v = 0; v < 3; ++v) {
+    const int bn = gated ? kShapes[v].bn / 2 : kShapes[v].bn;
+    const long long blocks = (long long)((n_rows + kShapes[v].bm - 1) / kShapes[v].bm) * ((n_out + bn - 1) / bn);
+    const long long rounds = (blocks + kCus - 1) / kCus;
+    const double cost = double(rounds) * kShapes[v].bm * kShapes[v].bn / speed[v];
+    if (v == 0 || cost < best) { best = cost; pick = v; }
+  }
+  return pick;
+}
+
 }  // namespace
 
 // Y = X W^T (+bias) (+resid), or gated: Y = silu(X Wg^T) * (X Wu^T), W = [Wg; Wu].
@@ -230,17 +376,30 @@ extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void
   a.y = y; a.y_dtype = y_dtype; a.x = (const bf16_t *)x; a.w = (const bf16_t *)w;
   a.bias = bias; a.bias_dtype = bias_dtype; a.resid = resid;
   a.n_rows = n_rows; a.n_out = n_out; a.n_in = n_in; a.gated = gated ? 1 : 0;
-  a.tiles_m = (n_rows + BM - 1) / BM;
-  const int bn = gated ? BN / 2 : BN;
+  int variant = pick_shape(n_rows, n_out, a.gated);
+  if (g_force_variant >= 0 && g_force_variant < 3) variant = g_force_variant;
+  const int bm = kShapes[variant].bm, bn = gated ? kShapes[variant].bn / 2 : kShapes[variant].bn;
+  a.tiles_m = (n_rows + bm - 1) / bm;
   a.tiles_n = (n_out + bn - 1) / bn;
   const long long blocks = (long long)a.tiles_m * a.tiles_n;
   SB_SUPPORT(blocks <= 0x7fffffffLL, "sb_gemm_mfma_bf16: too many tiles");
+  // the kernel addresses both operands with 32-bit byte offsets
+  const unsigned long long w_rows = (unsigned long long)((n_out + 15) / 16 * 16) * (gated ? 2 : 1);
+  const unsigned long long k_padded = (unsigned long long)((n_in + 31) / 32 * 32);
+  SB_SUPPORT(((unsigned long long)n_rows + 1) * n_in * 2 < (1ull << 32) - (1ull << 20) &&
+                 w_rows * k_padded * 2 < (1ull << 32) - (1ull << 20),
+             "sb_gemm_mfma_bf16: an operand of 4 GiB or more (rows=%d out=%d in=%d)", n_rows, n_out, n_in);
   hipStream_t s = (hipStream_t)stream;
   a.w_tiles = (n_out + 15) / 16;
   a.w_steps = (n_in + 31) / 32;
-  if (gated && packed) gemm_mfma_kernel<1, true><<<unsigned(blocks), kThreads, 0, s>>>(a);
-  else if (gated) gemm_mfma_kernel<1, false><<<unsigned(blocks), kThreads, 0, s>>>(a);
-  else if (packed) gemm_mfma_kernel<0, true><<<unsigned(blocks), kThreads, 0, s>>>(a);
-  else gemm_mfma_kernel<0, false><<<unsigned(blocks), kThreads, 0, s>>>(a);
+  int rc;
+  if (variant == 0) rc = launch<2, 2, 64, 2>(a, blocks, packed, s);
+  else if (variant == 1) rc = launch<4, 2, 64, 2>(a, blocks, packed, s);
+  else rc = launch<4, 4, 64, 1>(a, blocks, packed, s);
+  if (rc != SB_OK) return rc;
   return sb::check_launch("sb_gemm_mfma_bf16");
 }
+
+// Measurement hook: -1 lets the launcher choose; 0, 1, 2 force the 128 x 128, 256 x 128 and
+// 256 x 256 tiles.
+extern "C" void sb_gemm_mfma_force(int variant) { g_force_variant = variant; }

@@ -9,6 +9,8 @@ a missing library or a refused size raises
 """
 from __future__ import annotations
 
+import contextlib
+
 from typing import Optional
 
 import torch
@@ -381,6 +383,18 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], re
         check(lib.sb_gemm_mfma_bf16(_p(out), _dt(out), _p(x), _p(w), _p(bias), bdt, _p(resid), t, n, k,
                                     1 if gated else 0, packed, _stream()))
     return out
+
+
+@contextlib.contextmanager
+def gemm_tile_shape(shape: Optional[int]):
+    """For tests and measurements: inside the block the tiled product uses tile shape ``shape``
+    (0: 128 x 128, 1: 256 x 128, 2: 256 x 256 outputs per block) instead of choosing one."""
+    lib = library.core()
+    lib.sb_gemm_mfma_force(-1 if shape is None else int(shape))
+    try:
+        yield
+    finally:
+        lib.sb_gemm_mfma_force(-1)
 
 
 MFMA_MAX_HEAD_DIM = 256

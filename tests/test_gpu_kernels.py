@@ -133,6 +133,29 @@ def test_gemm_bf16_gated(t, inner, k):
     close(got, want, atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"gated t={t}")
 
 
+@pytest.mark.parametrize("shape", [0, 1, 2])
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("t, n, k", [(65, 100, 96), (300, 224, 200), (520, 264, 128), (257, 1000, 448), (130, 72, 2368)])
+def test_gemm_bf16_every_tile_shape(shape, packed, t, n, k):
+    """Each tile shape of the tiled product, with K a multiple of the stage or not, rows and
+    columns that end inside a tile, plain and packed weights, plain and gated."""
+    from sonicboom_amd import ops
+    x, w = randn(t, k, dtype=BF16), randn(n, k, dtype=BF16, scale=0.05)
+    bias, resid = randn(n, scale=0.1), randn(t, n)
+    wd = w.to(DEV)
+    with ops.gemm_tile_shape(shape):
+        got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(wd) if packed else wd, bias.to(DEV), resid.to(DEV), F32,
+                            packed_shape=(n, k) if packed else None)
+        close(got, ref_gemm(x, w, bias, resid), atol=3e-5 * math.sqrt(k), rtol=1e-5, what=f"shape {shape}")
+        inner = n // 2
+        gu = x.double() @ w[:2 * inner].double().T
+        g, u = gu[:, :inner], gu[:, inner:]
+        wg = wd[:2 * inner].contiguous()
+        got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(wg, True) if packed else wg, None, None, F32, gated=True,
+                            packed_shape=(2 * inner, k) if packed else None)
+        close(got, g / (1.0 + torch.exp(-g)) * u, atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"gated shape {shape}")
+
+
 def test_gemm_bf16_refuses_what_it_cannot_take():
     from sonicboom_amd import ops
     x, w = randn(4, 100, dtype=BF16).to(DEV), randn(8, 100, dtype=BF16).to(DEV)
