@@ -24,6 +24,8 @@
 // Order of summation: keys are visited in ascending order, 32 at a time, within
 // a wave; decode merges waves (pages) and then blocks (chunks of 4 pages) in
 // ascending order.  It depends on positions only, not on the batch.
+#include <type_traits>
+
 #include "mfma.cuh"
 
 #ifndef SB_HEAD_DIM
@@ -48,6 +50,7 @@ constexpr int KS = (HD + 31) / 32;   // k-steps of the score product
 constexpr int DT = HD / 16;          // 16-row tiles of O^T
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kPagesPerChunk = 4;
+constexpr float kMaxSlack = 8.f;
 
 // A wave's running softmax for NC groups of 16 query columns that share positions (and so the
 // mask): in decode one group, the heads of a kv head; in prefill up to four heads of one kv head
@@ -221,23 +224,200 @@ __device__ __forceinline__ void load_q(bf16x8_t (&qf)[KS], const bf16_t *qrow, b
 }
 
 // ---------------------------------------------------------------------------------------------
-// Prefill: a wave takes a tile of up to 16 consecutive rows of one sequence and NC query heads
-// of one kv head.  tiles: int32 [n_tiles][4] = (first row, rows, sequence, unused).
-// Grid: x = groups of four row tiles (one per wave), y = kv head x head tile.
-template <int NC>
-__global__ void __launch_bounds__(256)
+// Prefill: a block takes a tile of up to 16 consecutive rows of one sequence and one kv head; its
+// WAVES (4 or 8) waves take NC query heads of that kv head each (head tile WAVES * y + wave).
+// Eight waves are two per SIMD: one's matrix products run under the other's softmax arithmetic.  Every page of
+// keys and values is copied once per block into LDS (two buffers: the next page's loads are in
+// flight while this one is multiplied) and read from there by all four waves.
+// tiles: int32 [n_tiles][4] = (first row, rows, sequence, unused).  Grid: one dimension, the
+// block number counting (kv head, group of four head tiles) fastest and row tiles from the last
+// one down: the heavy (late) tiles of all heads start first and the short ones fill the gaps.
+constexpr int CPRK = HD / 8;                       // 16-byte chunks in a row of keys
+constexpr int kSwzK = CPRK % 16 == 0 ? 16 : (CPRK % 8 == 0 ? 8 : (CPRK % 4 == 0 ? 4 : 2));
+constexpr int kPageChunks = SB_PAGE * HD / 8;      // 16-byte chunks of a page of keys (= of values)
+
+// LDS position (in chunks) of chunk `chunk` of key row `key`: the sixteen rows a fragment read
+// touches at once (key bits 0, 1, 3, 4) land in distinct banks.
+__device__ __forceinline__ int k_slot(int key, int chunk) {
+  const int f = ((key & 3) | (((key >> 3) & 3) << 2)) & (kSwzK - 1);
+  return key * CPRK + (chunk ^ f);
+}
+// ... and of chunk `chunk` (8 keys) of value row d.
+__device__ __forceinline__ int v_slot(int d, int chunk) { return d * 8 + (chunk ^ ((d >> 1) & 7)); }
+
+__device__ __forceinline__ void load_half_lds(HalfPage &hp, const uint4 *kl, const uint4 *vl, int half, int lane) {
+  const int r = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int key = 32 * half + 8 * (r >> 2) + 4 * t + (r & 3);
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 32 + g * 8;
+      hp.k[t][ks] = d < HD ? kl[k_slot(key, ks * 4 + g)] : make_uint4(0u, 0u, 0u, 0u);
+    }
+  }
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) hp.v[dt] = vl[v_slot(dt * 16 + r, 4 * half + g)];
+}
+
+// One page (64 keys at page_pos ..) out of LDS for the wave's NC groups of 16 columns, the softmax
+// step taken over all 64 keys at once.  MASKED = false: every key of the page is visible from every
+// column of the wave (the common case below the diagonal), so no score is tested and no value cut.
+// PIN: keep the order written here (all fragments requested early), for a wave that has its SIMD
+// to itself; otherwise the compiler reads each fragment where it is used and a second wave of
+// the SIMD fills the waits.
+template <int NC, bool MASKED, bool PIN>
+__device__ __forceinline__ void attend_page64(WaveState<NC> &st, const bf16x8_t (&qf)[NC][KS], const uint4 *kl,
+                                              const uint4 *vl, int page_pos, int col_pos, int col_lo, int key_lo,
+                                              int key_hi, float scale_log2, int lane) {
+  const int r = lane & 15, g = lane >> 4;
+  auto read_k = [&](uint4 (&kf)[2][KS], int h) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      // A row r = 4 gg + i of score tile t is key 8 gg + 4 t + i of the 32
+      const int key = 32 * h + 8 * (r >> 2) + 4 * t + (r & 3);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d = ks * 32 + g * 8;
+        kf[t][ks] = d < HD ? kl[k_slot(key, ks * 4 + g)] : make_uint4(0u, 0u, 0u, 0u);
+      }
+    }
+  };
+  floatx4_t s[NC][2][2];      // [group][half][score tile]
+  auto scores = [&](const uint4 (&kf)[2][KS], int h) {
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        floatx4_t a = floatx4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) a = mfma16(as_bf16x8(kf[t][ks]), qf[c][ks], a);
+        s[c][h][t] = a;
+      }
+  };
+  uint4 vf[PIN ? DT : 1][2];
+  if (PIN) {
+    // All key fragments of the page are requested first, so that the wave waits for LDS once; the
+    // second half's arrive while the first half is multiplied.
+    uint4 kf[2][2][KS];
+    read_k(kf[0], 0);
+    read_k(kf[1], 1);
+    __builtin_amdgcn_sched_barrier(0);
+    scores(kf[0], 0);
+    scores(kf[1], 1);
+    __builtin_amdgcn_sched_barrier(0);
+    // the value fragments travel while the softmax is worked out
+#pragma unroll
+    for (int dt = 0; dt < (PIN ? DT : 1); ++dt)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) vf[dt][h] = vl[v_slot(dt * 16 + r, 4 * h + g)];
+    __builtin_amdgcn_sched_barrier(0);
+  } else {
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      uint4 kf[2][KS];
+      read_k(kf, h);
+      scores(kf, h);
+    }
+  }
+  // this lane: column lane % 16, keys page_pos + 32 h + 8 g + e, e = 0..7
+  // The running maximum only moves when a score exceeds it by more than kMaxSlack (in log2
+  // units): until then the probabilities are taken relative to the old maximum (at most
+  // 2^kMaxSlack, no trouble for float32 sums or bf16 operands) and the sums need no rescaling.
+  // The quotient o / l at the end is the same; only the rounding differs.
+  float alpha[NC];
+  uint4 pb[NC][2];
+  bool rescale = false;
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    float sc[16];
+    float mx = -__builtin_inff();
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float v = e < 4 ? s[c][h][0][e] : s[c][h][1][e - 4];
+        if (MASKED) {
+          const int j = page_pos + 32 * h + 8 * g + e;
+          v = (j <= col_pos && j >= col_lo) ? v : -__builtin_inff();
+        }
+        sc[8 * h + e] = v;
+        mx = fmaxf(mx, v);
+      }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx *= scale_log2;                                              // the scale is positive
+    const float m_old = st.m[c];
+    const bool move = mx > m_old + kMaxSlack;                      // also the first key of a column
+    const float m_new = move ? mx : m_old;
+    // a column that has seen no key yet keeps m = -inf: give it a finite stand-in
+    const float m_use = m_new == -__builtin_inff() ? 0.f : m_new;
+    alpha[c] = move ? __builtin_amdgcn_exp2f(m_old - m_use) : 1.f; // m_old = -inf gives 0
+    rescale = rescale || move;
+    float p[16];
+    float psum = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      p[e] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[e], scale_log2, -m_use));   // -inf gives 0
+      psum += p[e];
+    }
+    st.l[c] = st.l[c] * alpha[c] + psum;
+    st.m[c] = m_new;
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      pb[c][h] = make_uint4(pack_bf16(p[8 * h + 0], p[8 * h + 1]), pack_bf16(p[8 * h + 2], p[8 * h + 3]),
+                            pack_bf16(p[8 * h + 4], p[8 * h + 5]), pack_bf16(p[8 * h + 6], p[8 * h + 7]));
+  }
+  // the old sums shrink by alpha; once the maxima have settled no column of the wave moves
+  if (__any(rescale)) {
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        st.o[c][dt][0] *= alpha[c]; st.o[c][dt][1] *= alpha[c];
+        st.o[c][dt][2] *= alpha[c]; st.o[c][dt][3] *= alpha[c];
+      }
+  }
+  if (PIN) __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt) {
+    uint4 va[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      uint4 a = PIN ? vf[PIN ? dt : 0][h] : vl[v_slot(dt * 16 + r, 4 * h + g)];
+      if (MASKED) {
+        // values of keys outside [key_lo, key_hi] may be stale or never written: 0 * garbage must
+        // not reach the accumulator
+        const int k0 = page_pos + 32 * h + 8 * g;
+        a = drop_first(keep_first(a, key_hi - k0 + 1), key_lo - k0);
+      }
+      va[h] = a;
+    }
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      floatx4_t acc = mfma16(as_bf16x8(va[0]), as_bf16x8(pb[c][0]), st.o[c][dt]);
+      st.o[c][dt] = mfma16(as_bf16x8(va[1]), as_bf16x8(pb[c][1]), acc);
+    }
+  }
+}
+
+template <int NC, int WAVES>
+__global__ void __launch_bounds__(64 * WAVES, (WAVES == 8 || NC == 1) ? 2 : 1)
 attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
                     const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
                     const int32_t *__restrict__ page_table, int max_pages, int n_pages_total,
                     const int32_t *__restrict__ row_pos, const int32_t *__restrict__ tiles, int n_tiles,
-                    int heads_q, int heads_kv, float scale_log2, int window) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  // heavy tiles (late rows, long key ranges) first
-  const int tile = n_tiles - 1 - (blockIdx.x * 4 + wave);
-  if (tile < 0) return;
+                    int heads_q, int heads_kv, int head_tiles, int y_per_kv, float scale_log2, int window) {
+  constexpr int kThreads = 64 * WAVES;
+  constexpr int kStageLoads = (kPageChunks + kThreads - 1) / kThreads;
+  extern __shared__ uint4 lds_pages[];               // [2 buffers][keys | values][kPageChunks]
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int n_y = heads_kv * y_per_kv;
+  const int tile = n_tiles - 1 - int(blockIdx.x) / n_y, by = int(blockIdx.x) % n_y;
   const int group = heads_q / heads_kv;
-  const int head_tiles = (group + NC - 1) / NC;
-  const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y - kvh * head_tiles;
+  const int kvh = by / y_per_kv, yb = by - kvh * y_per_kv;
+  const int ht = yb * WAVES + wave;                      // this wave's head tile
+  const bool active = ht < head_tiles;
   const int row0 = tiles[tile * 4 + 0], n_rows = tiles[tile * 4 + 1], seq = tiles[tile * 4 + 2];
   const int r = lane & 15, g = lane >> 4;
   const bool col_ok = r < n_rows;
@@ -250,6 +430,8 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
   const int pos_first = row_pos[row0], pos_last = row_pos[row0 + n_rows - 1];
   const int key_lo = (window > 0 && pos_first >= window) ? pos_first - window + 1 : 0;
   const int key_hi = pos_last;
+  // first key that every row of the tile sees (the last row's window start)
+  const int lo_last = (window > 0 && pos_last >= window) ? pos_last - window + 1 : 0;
 
   bf16x8_t qf[NC][KS];
   int head[NC];
@@ -257,19 +439,102 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
 #pragma unroll
   for (int c = 0; c < NC; ++c) {
     const int hg = ht * NC + c;                      // query head within the kv head's group
-    head_ok[c] = hg < group;
+    head_ok[c] = active && hg < group;
     head[c] = kvh * group + (head_ok[c] ? hg : 0);
     load_q(qf[c], q + (size_t(row) * heads_q + head[c]) * HD, col_ok && head_ok[c], lane);
   }
   WaveState<NC> st;
   init_state<NC>(st);
+
   const int32_t *pt = page_table + size_t(seq) * max_pages;
-  for (int pg = key_lo / SB_PAGE; pg <= key_hi / SB_PAGE; ++pg) {
-    const int page = pg < max_pages ? pt[pg] : -1;
-    if (page < 0 || page >= n_pages_total) continue;
-    const size_t off = (size_t(page) * heads_kv + kvh) * SB_PAGE * HD;
-    attend_page<NC>(st, qf, k_cache + off, v_cache + off, pg * SB_PAGE, col_pos, col_lo, key_lo, key_hi,
-                    scale_log2, lane);
+  const int pg_hi = min(key_hi / SB_PAGE, max_pages - 1);
+  // the next page from pg on that the table holds (uniform over the block)
+  auto next_valid = [&](int pg) {
+    while (pg <= pg_hi) {
+      const int page = pt[pg];
+      if (page >= 0 && page < n_pages_total) break;
+      ++pg;
+    }
+    return pg;
+  };
+  // Two register sets: while page p is multiplied out of LDS, page p + 1 waits in one set (its
+  // loads went out a page earlier) and the loads of page p + 2 go out into the other.
+  bf16x8_t stage_k[2][kStageLoads], stage_v[2][kStageLoads];
+  auto issue = [&](auto SET, int pg) {
+    constexpr int set = decltype(SET)::value;
+    const size_t off = (size_t(pt[pg]) * heads_kv + kvh) * SB_PAGE * HD;
+    const bf16x8_t *kp = reinterpret_cast<const bf16x8_t *>(k_cache + off);
+    const bf16x8_t *vp = reinterpret_cast<const bf16x8_t *>(v_cache + off);
+#pragma unroll
+    for (int j = 0; j < kStageLoads; ++j) {
+      const int id = tid + kThreads * j;
+      if (kPageChunks % kThreads == 0 || id < kPageChunks) {
+        stage_k[set][j] = kp[id];
+        stage_v[set][j] = vp[id];
+      }
+    }
+  };
+  auto store = [&](auto SET, int buf) {
+    constexpr int set = decltype(SET)::value;
+    bf16x8_t *kl = reinterpret_cast<bf16x8_t *>(lds_pages) + buf * 2 * kPageChunks, *vl = kl + kPageChunks;
+#pragma unroll
+    for (int j = 0; j < kStageLoads; ++j) {
+      const int id = tid + kThreads * j;
+      if (kPageChunks % kThreads == 0 || id < kPageChunks) {
+        kl[k_slot(id / CPRK, id % CPRK)] = stage_k[set][j];
+        vl[v_slot(id / 8, id % 8)] = stage_v[set][j];
+      }
+    }
+  };
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+
+  int pg = next_valid(key_lo / SB_PAGE);                      // the page being multiplied
+  int pg1 = pg <= pg_hi ? next_valid(pg + 1) : pg;            // the page after it
+  if (pg <= pg_hi) issue(Set0{}, pg);
+  if (pg1 <= pg_hi) issue(Set1{}, pg1);
+  if (pg <= pg_hi) store(Set0{}, 0);
+  __syncthreads();
+  int buf = 0;
+  // One page: FREE is the register set whose page already lies in LDS.
+  auto step = [&](auto FREE) {
+    constexpr int free_set = decltype(FREE)::value;
+    using SetFree = std::integral_constant<int, free_set>;
+    using SetHeld = std::integral_constant<int, free_set ^ 1>;
+    const int pg2 = pg1 <= pg_hi ? next_valid(pg1 + 1) : pg1;
+    if (pg2 <= pg_hi) issue(SetFree{}, pg2);
+    if (active) {
+      const uint4 *kl = lds_pages + buf * 2 * kPageChunks, *vl = kl + kPageChunks;
+      const int page_pos = pg * SB_PAGE;
+      if (HD > 128) {
+        // too many fragments for the registers at once: half a page at a time
+        HalfPage h;
+        if (!(page_pos > key_hi || page_pos + 31 < key_lo)) {
+          load_half_lds(h, kl, vl, 0, lane);
+          attend_half<NC>(st, qf, h, page_pos, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
+        }
+        if (!(page_pos + 32 > key_hi || page_pos + 63 < key_lo)) {
+          load_half_lds(h, kl, vl, 1, lane);
+          attend_half<NC>(st, qf, h, page_pos + 32, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
+        }
+      } else if (page_pos + SB_PAGE - 1 <= pos_first && page_pos >= lo_last) {
+        attend_page64<NC, false, WAVES == 4 && NC != 1>(st, qf, kl, vl, page_pos, col_pos, col_lo, key_lo, key_hi,
+                                             scale_log2, lane);
+      } else {
+        attend_page64<NC, true, WAVES == 4 && NC != 1>(st, qf, kl, vl, page_pos, col_pos, col_lo, key_lo, key_hi,
+                                            scale_log2, lane);
+      }
+    }
+    if (pg1 <= pg_hi) store(SetHeld{}, buf ^ 1);
+    __syncthreads();
+    pg = pg1;
+    pg1 = pg2;
+    buf ^= 1;
+  };
+  while (pg <= pg_hi) {
+    step(Set0{});
+    if (pg > pg_hi) break;
+    step(Set1{});
   }
 #pragma unroll
   for (int c = 0; c < NC; ++c) {
@@ -422,6 +687,8 @@ attn_decode_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ par
                 first, last, seq, heads_q, kvh, ht, group);
 }
 
+int g_force_nc = 0, g_force_waves = 0;
+
 int check_common(const void *out, const void *q, const void *k, const void *v, const void *pt,
                  const void *row_pos, int max_pages, int n_pages_total, int heads_q, int heads_kv,
                  int window, const char *who) {
@@ -485,6 +752,9 @@ extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache
   return sb::check_launch("sb_attn_decode_bf16 (merge)");
 }
 
+// Measurement hook: heads per wave and waves per block in prefill (0: chosen from the group size).
+extern "C" void sb_attn_prefill_force(int nc, int waves) { g_force_nc = nc; g_force_waves = waves; }
+
 // q, out: bf16 [n_rows, heads_q * HD]; tiles int32 [n_tiles][4] = (first row, rows <= 16, sequence, 0),
 // every tile inside one sequence and its rows at consecutive positions.
 extern "C" int sb_attn_prefill_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
@@ -498,20 +768,40 @@ extern "C" int sb_attn_prefill_bf16(void *out, const void *q, const void *k_cach
   if (n_tiles == 0) return SB_OK;
   hipStream_t s = (hipStream_t)stream;
   const int group = heads_q / heads_kv;
-  // query heads of a kv head that one wave takes together: each key and value fragment it reads
-  // then feeds that many products
-  const int nc = (group >= 4 && HD <= 128) ? 4 : (group >= 2 ? 2 : 1);
+  // Waves of a block and query heads of a kv head that one wave takes together: the block's
+  // waves cover the group, eight of them (two per SIMD) when the group is big enough to use them,
+  // as far as the accumulators fit the registers.
+  int waves = (group >= 5 && group <= 8 && HD <= 128) ? 8 : 4;
+  if (g_force_waves == 4) waves = 4;
+  int nc = (group + waves - 1) / waves;
+  const int nc_max = waves == 8 ? 1 : (DT <= 4 ? 4 : (DT <= 12 ? 2 : 1));
+  if (nc > nc_max) nc = nc_max;
+  if (g_force_nc > 0 && g_force_nc <= nc_max) nc = g_force_nc;
   const int head_tiles = (group + nc - 1) / nc;
-  SB_SUPPORT(heads_kv * head_tiles <= 65535, "sb_attn_prefill_bf16: too many heads");
-  dim3 grid((n_tiles + 3) / 4, heads_kv * head_tiles);
-#define SB_GO(NC)                                                                                      \
-  attn_prefill_kernel<NC><<<grid, 256, 0, s>>>((bf16_t *)out, (const bf16_t *)q, (const bf16_t *)k_cache, \
-                                               (const bf16_t *)v_cache, page_table, max_pages,           \
-                                               n_pages_total, row_pos, tiles, n_tiles, heads_q, heads_kv, \
-                                               scale * kLog2e, window)
-  if (nc == 4) SB_GO(4);
-  else if (nc == 2) SB_GO(2);
-  else SB_GO(1);
+  const int y_per_kv = (head_tiles + waves - 1) / waves;
+  SB_SUPPORT((long long)n_tiles * heads_kv * y_per_kv <= 0x7fffffffLL, "sb_attn_prefill_bf16: too many blocks");
+  dim3 grid(unsigned(n_tiles) * unsigned(heads_kv * y_per_kv));
+  constexpr int lds_bytes = 2 * 2 * kPageChunks * 16;
+#define SB_GO(NC, WAVES)                                                                                 \
+  do {                                                                                                   \
+    static bool raised = false;                                                                          \
+    if (lds_bytes > 48 * 1024 && !raised) {                                                              \
+      const hipError_t e = hipFuncSetAttribute((const void *)attn_prefill_kernel<NC, WAVES>,             \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);   \
+      SB_REQUIRE(e == hipSuccess, "sb_attn_prefill_bf16: cannot reserve %d bytes of LDS: %s", lds_bytes, \
+                 hipGetErrorString(e));                                                                  \
+      raised = true;                                                                                     \
+    }                                                                                                    \
+    attn_prefill_kernel<NC, WAVES><<<grid, 64 * WAVES, lds_bytes, s>>>(                                  \
+        (bf16_t *)out, (const bf16_t *)q, (const bf16_t *)k_cache, (const bf16_t *)v_cache, page_table,  \
+        max_pages, n_pages_total, row_pos, tiles, n_tiles, heads_q, heads_kv, head_tiles, y_per_kv,      \
+        scale * kLog2e, window);                                                                         \
+  } while (0)
+  if (waves == 8) SB_GO(1, 8);
+  else if (nc == 4) SB_GO(4, 4);
+  else if (nc == 3) SB_GO(3, 4);
+  else if (nc == 2) SB_GO(2, 4);
+  else SB_GO(1, 4);
 #undef SB_GO
   return sb::check_launch("sb_attn_prefill_bf16");
 }

@@ -29,7 +29,10 @@ __device__ __forceinline__ uint4 ld16(const void *p, bool ok) {
   return ok ? *reinterpret_cast<const uint4 *>(p) : make_uint4(0u, 0u, 0u, 0u);
 }
 
-// Two floats to two bf16 packed in 32 bits (low half first).
+// Two floats to two bf16 packed in 32 bits (low half first), round to nearest even: one
+// v_cvt_pk_bf16_f32.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  return uint32_t(f32_to_bf16(lo)) | (uint32_t(f32_to_bf16(hi)) << 16);
+  const bf16x2_t v = {(__bf16)lo, (__bf16)hi};
+  return __builtin_bit_cast(uint32_t, v);
 }
