@@ -319,19 +319,25 @@ int launch_one(const Args &a, long long blocks, hipStream_t s) {
   return SB_OK;
 }
 
-template <int MT, int NW, int BK, int DEPTH>
+template <int MT, int NW, int BK, int DEPTH, bool PLAIN_TOO>
 int launch(const Args &a, long long blocks, int packed, hipStream_t s) {
   const int which = (a.gated ? 4 : 0) + (packed ? 2 : 0) + (a.n_in % BK == 0 ? 1 : 0);
   switch (which) {
     case 7: return launch_one<MT, NW, BK, DEPTH, 1, true, true>(a, blocks, s);
     case 6: return launch_one<MT, NW, BK, DEPTH, 1, true, false>(a, blocks, s);
-    case 5: return launch_one<MT, NW, BK, DEPTH, 1, false, true>(a, blocks, s);
-    case 4: return launch_one<MT, NW, BK, DEPTH, 1, false, false>(a, blocks, s);
     case 3: return launch_one<MT, NW, BK, DEPTH, 0, true, true>(a, blocks, s);
     case 2: return launch_one<MT, NW, BK, DEPTH, 0, true, false>(a, blocks, s);
-    case 1: return launch_one<MT, NW, BK, DEPTH, 0, false, true>(a, blocks, s);
-    default: return launch_one<MT, NW, BK, DEPTH, 0, false, false>(a, blocks, s);
+    default: break;
   }
+  if constexpr (PLAIN_TOO) {
+    switch (which) {
+      case 5: return launch_one<MT, NW, BK, DEPTH, 1, false, true>(a, blocks, s);
+      case 4: return launch_one<MT, NW, BK, DEPTH, 1, false, false>(a, blocks, s);
+      case 1: return launch_one<MT, NW, BK, DEPTH, 0, false, true>(a, blocks, s);
+      default: return launch_one<MT, NW, BK, DEPTH, 0, false, false>(a, blocks, s);
+    }
+  }
+  return sb::fail(SB_ERR_UNSUPPORTED, "sb_gemm_mfma_bf16: this tile shape takes packed weights only");
 }
 
 // Tile shapes the launcher chooses from: rows x columns of Y per block.
@@ -378,6 +384,7 @@ extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void
   a.n_rows = n_rows; a.n_out = n_out; a.n_in = n_in; a.gated = gated ? 1 : 0;
   int variant = pick_shape(n_rows, n_out, a.gated);
   if (g_force_variant >= 0 && g_force_variant < 3) variant = g_force_variant;
+  if (!packed) variant = 0;       // the bigger tiles are built for packed weights only
   const int bm = kShapes[variant].bm, bn = gated ? kShapes[variant].bn / 2 : kShapes[variant].bn;
   a.tiles_m = (n_rows + bm - 1) / bm;
   a.tiles_n = (n_out + bn - 1) / bn;
@@ -393,9 +400,9 @@ extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void
   a.w_tiles = (n_out + 15) / 16;
   a.w_steps = (n_in + 31) / 32;
   int rc;
-  if (variant == 0) rc = launch<2, 2, 64, 2>(a, blocks, packed, s);
-  else if (variant == 1) rc = launch<4, 2, 64, 2>(a, blocks, packed, s);
-  else rc = launch<4, 4, 64, 1>(a, blocks, packed, s);
+  if (variant == 0) rc = launch<2, 2, 64, 2, true>(a, blocks, packed, s);
+  else if (variant == 1) rc = launch<4, 2, 64, 2, false>(a, blocks, packed, s);
+  else rc = launch<4, 4, 64, 1, false>(a, blocks, packed, s);
   if (rc != SB_OK) return rc;
   return sb::check_launch("sb_gemm_mfma_bf16");
 }

@@ -143,6 +143,7 @@ def test_gemm_bf16_every_tile_shape(shape, packed, t, n, k):
     x, w = randn(t, k, dtype=BF16), randn(n, k, dtype=BF16, scale=0.05)
     bias, resid = randn(n, scale=0.1), randn(t, n)
     wd = w.to(DEV)
+    # plain (unpacked) weights always take the 128 x 128 tile
     with ops.gemm_tile_shape(shape):
         got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(wd) if packed else wd, bias.to(DEV), resid.to(DEV), F32,
                             packed_shape=(n, k) if packed else None)
