@@ -79,20 +79,20 @@ class DecoderModel:
     @classmethod
     def from_folder(cls, folder: str, dtype: str = "bfloat16", device=None, fast_kernels: bool = True):
         """The model of a folder with config.json and model.safetensors; its class is chosen by config.json."""
-        dev = require_gpu(device)
-        arch, cfg = load_config(folder)
+        arch, cfg = load_config(folder)          # configuration errors first: they need no GPU
         spec = arch.build_spec(cfg)
+        dev = require_gpu(device)
         tensors = load_tensors(folder, spec, dtype, dev)
         return cls(spec, tensors, Runtime(dev, DTYPES[dtype], fast_kernels), cfg)
 
     @classmethod
     def from_random(cls, config, seed: int, dtype: str = "bfloat16", device=None, fast_kernels: bool = True):
         """Random weights drawn on the device, for a typed configuration or a config.json dict."""
-        dev = require_gpu(device)
         d = config if isinstance(config, dict) else config.to_dict()
         arch = architecture_of(d)
         cfg = arch.config_class.from_dict(d)
         spec = arch.build_spec(cfg)
+        dev = require_gpu(device)
         tensors = random_tensors(spec, seed, dtype, dev)
         return cls(spec, tensors, Runtime(dev, DTYPES[dtype], fast_kernels), cfg)
 

@@ -1,0 +1,110 @@
+"""The C interface (sonicboom_amd/capi): the header is plain C, failures are statuses with
+messages, and what a C program gets equals what the package gives."""
+import os
+import shutil
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CAPI = os.path.join(ROOT, "sonicboom_amd", "capi")
+HERE = os.path.join(ROOT, "tests", "capi")
+
+pytestmark = pytest.mark.skipif(shutil.which("gcc") is None, reason="no C compiler")
+
+
+def compile_c(source, tmp_path):
+    from sonicboom_amd.capi import build
+    lib, _ = build.build()
+    exe = str(tmp_path / os.path.splitext(os.path.basename(source))[0])
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-O1", source, f"-I{CAPI}", f"-L{os.path.dirname(lib)}",
+                        "-lsonicboom_amd", f"-Wl,-rpath,{os.path.dirname(lib)}", "-o", exe],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    return exe
+
+
+def run(cmd, **kw):
+    env = dict(os.environ, SONICBOOM_AMD_ROOT=ROOT)
+    return subprocess.run(cmd, capture_output=True, text=True, env=env, timeout=600, **kw)
+
+
+def test_header_is_plain_c():
+    r = subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror", "-fsyntax-only", "-x", "c",
+                        os.path.join(CAPI, "sonicboom_amd.h")], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+
+
+def test_failures_are_statuses_with_messages(tmp_path):
+    exe = compile_c(os.path.join(HERE, "check_errors.c"), tmp_path)
+    r = run([exe])
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stdout + r.stderr
+
+
+def test_command_line_usage_and_errors(tmp_path):
+    from sonicboom_amd.capi import build
+    _, cmd = build.build()
+    r = run([cmd])
+    assert r.returncode == 2 and "usage: sb-gen" in r.stderr
+    r = run([cmd, "--bogus", "1"])
+    assert r.returncode == 2 and "unknown option" in r.stderr
+    tokens = tmp_path / "p.txt"
+    tokens.write_text("1 2 3\n")
+    r = run([cmd, "-m", str(tmp_path / "nowhere"), "--tokens", str(tokens)])
+    assert r.returncode == 1 and "config.json" in r.stderr
+    r = run([cmd, "-m", "x", "--tokens", str(tmp_path / "missing.txt")])
+    assert r.returncode == 2 and "tokens file not found" in r.stderr
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_c_program_gets_what_the_package_gives(tmp_path, model_folders, dtype):
+    import torch
+    from sonicboom_amd.api import Model
+    folder = model_folders["B"]
+    exe = compile_c(os.path.join(HERE, "generate.c"), tmp_path)
+    r = run([exe, folder, dtype])
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stdout + r.stderr
+    got = r.stdout.strip().splitlines()
+
+    model = Model.load(folder, dtype=dtype)
+    session = model.session(512)
+    want = [f"arch {model.arch}", f"vocab {model.vocab_size}", "eos" + "".join(f" {t}" for t in model.eos)]
+    s0, s1 = session.alloc_slot(), session.alloc_slot()
+    logits = session.step([(s0, [5, 17, 3, 9, 250], [0, 4]), (s1, [7, 7], [1])]).float().cpu()
+    for row in range(3):
+        best = int(torch.argmax(logits[row]))
+        want.append(f"step row {row} argmax {best} logit {float(logits[row, best]):.6f}")
+    session.free_slot(s0)
+    session.free_slot(s1)
+    prompts = [[1, 2, 3], [4, 5, 6, 7, 8, 9, 10], [11]]
+    seen = [0]
+
+    def cb(i, t):
+        if i == 1:
+            seen[0] += 1
+            return seen[0] >= 3
+        return False
+    outs = session.generate(prompts, max_tokens=6, stop_tokens=[], callback=cb)
+    assert len(outs[1]) == 3
+    want += [f"greedy {i}:" + "".join(f" {t}" for t in o) for i, o in enumerate(outs)]
+    outs = session.generate(prompts, max_tokens=6, stop_tokens=[], temperature=0.8, seed=7, top_k=40)
+    want += [f"sampled {i}:" + "".join(f" {t}" for t in o) for i, o in enumerate(outs)]
+    want.append("ok")
+    assert got == want
+
+
+@pytest.mark.gpu
+def test_both_command_lines_agree(tmp_path, model_folders):
+    from sonicboom_amd.capi import build
+    _, cmd = build.build()
+    tokens = tmp_path / "prompts.txt"
+    tokens.write_text("1 2 3 4\n9 8 7\n5\n")
+    args = ["-m", model_folders["A"], "--tokens", str(tokens), "-n", "5", "--dtype", "float32", "--temperature", "0.7",
+            "--sample-seed", "3", "--top-p", "0.9", "--stop", "1000000"]
+    native = run([cmd, *args])
+    assert native.returncode == 0, native.stderr
+    script = run([sys.executable, os.path.join(ROOT, "bin", "sb-gen"), *args])
+    assert script.returncode == 0, script.stderr
+    assert native.stdout == script.stdout and len(native.stdout.splitlines()) == 3
