@@ -157,6 +157,27 @@ def test_gemm_bf16_every_tile_shape(shape, packed, t, n, k):
         close(got, g / (1.0 + torch.exp(-g)) * u, atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"gated shape {shape}")
 
 
+@pytest.mark.parametrize("t", [17, 40, 64])
+def test_gemm_bf16_wide_matrix_with_few_rows(t):
+    """17 to 64 rows against a matrix of 256 tiles or more go to the tiled kernel (packed
+    weights), plain and gated; one tile less stays with the weight-streaming kernel."""
+    from sonicboom_amd import ops
+    from sonicboom_amd.ops import kernels
+    k = 64
+    x = randn(t, k, dtype=BF16)
+    for n in (kernels.TILED_MIN_TILES * 128, kernels.TILED_MIN_TILES * 128 - 128):
+        w = randn(n, k, dtype=BF16, scale=0.05)
+        got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(w.to(DEV)), None, None, F32, packed_shape=(n, k))
+        close(got, ref_gemm(x, w), atol=3e-5 * math.sqrt(k), rtol=1e-5, what=f"wide n={n}")
+    for inner in (kernels.TILED_MIN_TILES * 64, kernels.TILED_MIN_TILES * 64 - 64):   # gated tiles hold 64 outputs
+        w = randn(2 * inner, k, dtype=BF16, scale=0.05)
+        gu = x.double() @ w.double().T
+        g, u = gu[:, :inner], gu[:, inner:]
+        got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(w.to(DEV), True), None, None, F32, gated=True,
+                            packed_shape=(2 * inner, k))
+        close(got, g / (1.0 + torch.exp(-g)) * u, atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"wide gated {inner}")
+
+
 def test_gemm_bf16_refuses_what_it_cannot_take():
     from sonicboom_amd import ops
     x, w = randn(4, 100, dtype=BF16).to(DEV), randn(8, 100, dtype=BF16).to(DEV)
