@@ -440,6 +440,50 @@ def test_a_far_key_among_hundreds_is_found():
             assert torch.allclose(out[0, h * hd:(h + 1) * hd], vals[0][far, h // 2], atol=1e-4), (far, h)
 
 
+@pytest.mark.parametrize("hq, hkv, hd", [(14, 2, 128), (4, 2, 64), (3, 1, 32)])
+@pytest.mark.parametrize("shape", ["climbing", "falling", "far key"])
+def test_attention_matrix_cores_when_the_maximum_moves(hq, hkv, hd, shape):
+    """Scores made to climb page after page (the running maximum has to follow, in steps), to
+    fall from the first key on (it never moves again), or to peak at one key far back among
+    hundreds of small ones: prefill rows and decode rows against the plain softmax."""
+    from sonicboom_amd import ops
+    n, group = 600, hq // hkv
+    scale = 1.0 / math.sqrt(hd)
+    keys = randn(n, hkv, hd, scale=0.05, seed=11)
+    vals = randn(n, hkv, hd, seed=12)
+    rows_pos = list(range(552, 600))                 # 552 keys cached, 48 rows asking
+    q = randn(len(rows_pos), hq * hd, scale=0.05, seed=13)
+    q.view(len(rows_pos), hq, hd)[:, :, 0] = 8.0      # every head looks along coordinate 0
+    ramp = torch.arange(n, dtype=torch.float32) / n   # 0 .. 1 over the sequence
+    rise = 56.0 / (8.0 * scale)                       # scores span about 56 (81 in log2 units)
+    if shape == "climbing":
+        keys[:, :, 0] = (ramp * rise)[:, None]
+    elif shape == "falling":
+        keys[:, :, 0] = ((1.0 - ramp) * rise)[:, None]
+    else:
+        keys[389, :, 0] = rise
+    keys, vals, q = keys.to(BF16).float(), vals.to(BF16).float(), q.to(BF16)
+    table = torch.tensor([[7, 2, 9, 4, 0, 5, 1, 8, 3, 6]], dtype=torch.int32)
+    kc, vc = fill_cache_from([keys], [vals], table, BF16)
+    want = plain.attention(q.float().numpy(), keys.reshape(n, -1).numpy(), vals.reshape(n, -1).numpy(), rows_pos,
+                           np.arange(n), hq, hkv, hd, scale, causal=True, window=0)
+    pos = torch.tensor(rows_pos, dtype=torch.int32)
+    tiles = torch.tensor([(r0, min(16, len(rows_pos) - r0), 0, 0) for r0 in range(0, len(rows_pos), 16)],
+                         dtype=torch.int32)
+    got = ops.attention_prefill_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), tiles.to(DEV), hq, hkv, hd,
+                                     scale, 0)
+    close(got, want, atol=1.5e-2, rtol=1e-2, what=f"prefill, {shape}")
+    # the same rows as single decode rows of sequences that share the pages
+    for r in (0, 17, 47):
+        got1 = ops.attention_decode_mfma(q[r:r + 1].to(DEV), kc, vc, table.to(DEV), pos[r:r + 1].to(DEV), hq, hkv,
+                                         hd, scale, 0)
+        close(got1, want[r:r + 1], atol=1.5e-2, rtol=1e-2, what=f"decode row {r}, {shape}")
+    if shape == "far key":
+        # the far key takes all the weight: the output is its value
+        v_far = vals[389].repeat_interleave(group, dim=0).reshape(1, -1)
+        close(got[-1:], v_far.numpy(), atol=2e-2, rtol=1e-2, what="far key's value")
+
+
 @pytest.mark.parametrize("vocab", [5, 256, 1000, 152064])
 def test_argmax_first_maximum(vocab):
     from sonicboom_amd import ops
