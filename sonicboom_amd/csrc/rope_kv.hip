@@ -30,10 +30,11 @@ __device__ __forceinline__ float qkv_at(const TI *r, size_t e, int n_slices, siz
   return v;
 }
 
-constexpr int kHeadsPerBlock = 4;
-
-// Block (row, head group): heads [4 y, 4 y + 4) of the row's heads_q query heads, heads_kv key
-// heads and heads_kv value heads, in that order.
+// Block (row, head group): heads [hpb y, hpb (y + 1)) of the row's heads_q query heads, heads_kv
+// key heads and heads_kv value heads, in that order.  Few rows (decode): groups of four heads,
+// to have enough blocks; many rows (prefill): all heads of a row in one block, so that the
+// row's cosines and sines and its page look-up are worked out once and every thread has
+// several pairs to move.
 template <typename TI, typename TQ, typename TC>
 __global__ void __launch_bounds__(256)
 rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_stride, int n_slices,
@@ -42,7 +43,7 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
                int rot_dims, const int32_t *__restrict__ row_pos,
                const int32_t *__restrict__ row_seq, TC *__restrict__ k_cache,
                TC *__restrict__ v_cache, const int32_t *__restrict__ page_table, int max_pages,
-               int n_pages_total, int heads_q, int heads_kv, int head_dim) {
+               int n_pages_total, int heads_q, int heads_kv, int head_dim, int heads_per_block) {
   const int row = blockIdx.x;
   const int pos = row_pos[row];
   const TI *r = qkv + size_t(row) * row_stride;
@@ -50,7 +51,7 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
   const int q_width = heads_q * head_dim;
   TQ *qo = q_out + size_t(row) * q_width;
   const int n_heads = heads_q + 2 * heads_kv;
-  const int h_begin = blockIdx.y * kHeadsPerBlock, h_end = min(h_begin + kHeadsPerBlock, n_heads);
+  const int h_begin = blockIdx.y * heads_per_block, h_end = min(h_begin + heads_per_block, n_heads);
 
   // Where this row's key and value go.
   int page_of_row = 0;
@@ -156,13 +157,16 @@ extern "C" int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int q
                "sb_rope_kv_store: a layer that stores keys needs a cache and a page table");
   if (n_rows == 0) return SB_OK;
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid(n_rows, (heads_q + 2 * heads_kv + kHeadsPerBlock - 1) / kHeadsPerBlock);
+  const int n_heads = heads_q + 2 * heads_kv;
+  const int heads_per_block = n_rows >= 512 ? n_heads : 4;
+  const dim3 grid(n_rows, (n_heads + heads_per_block - 1) / heads_per_block);
   SB_SUPPORT(grid.y <= 65535, "sb_rope_kv_store: too many heads");
 #define SB_GO(TI, TQ, TC)                                                                        \
   rope_kv_kernel<TI, TQ, TC><<<grid, 256, 0, s>>>(                                              \
       (TQ *)q_out, (const TI *)qkv, row_stride, n_slices, slice_stride, bias, inv_freq, freq_factors,   \
       rot_dims, row_pos, row_seq,                                                                    \
-      (TC *)k_cache, (TC *)v_cache, page_table, max_pages, n_pages_total, heads_q, heads_kv, head_dim)
+      (TC *)k_cache, (TC *)v_cache, page_table, max_pages, n_pages_total, heads_q, heads_kv, head_dim,  \
+      heads_per_block)
   const int key = qkv_dtype * 4 + q_dtype * 2 + cache_dtype;
   switch (key) {
     case 0: SB_GO(float, float, float); break;

@@ -251,6 +251,31 @@ def test_rope_kv_store(hq, hkv, hd, rot, dtype):
     assert torch.isnan(kc.float()).sum().item() == kc.numel() - n * kvw
 
 
+@pytest.mark.parametrize("hq, hkv, hd, rot", [(7, 1, 48, 0), (28, 4, 128, 0), (3, 3, 64, 32)])
+def test_rope_kv_store_many_rows_equals_few_rows(hq, hkv, hd, rot):
+    """A prompt of 700 rows in one call (all heads of a row in one block) gives bitwise what the
+    same rows give in calls of 100 (groups of four heads)."""
+    from sonicboom_amd import ops
+    n = 700
+    qkv = randn(n, (hq + 2 * hkv) * hd).to(DEV)
+    bias = randn((hq + 2 * hkv) * hd, scale=0.1, seed=3).to(DEV)
+    pos = torch.arange(n, dtype=torch.int32, device=DEV)
+    seq = torch.zeros(n, dtype=torch.int32, device=DEV)
+    table = torch.tensor([[4, 9, 1, 7, 3, 10, 0, 6, 2, 8, 5]], dtype=torch.int32, device=DEV)
+    dims = rot or hd
+    inv = torch.exp(-2.0 * torch.arange(dims // 2, dtype=F32) / dims * math.log(1e6)).to(DEV)
+    results = []
+    for step in (n, 100):
+        kc, vc = make_cache(11, hkv, hd, BF16, fill=0.0)
+        qs = [ops.rope_kv_store(qkv[r0:r0 + step], BF16, inv, None, dims, pos[r0:r0 + step], seq[r0:r0 + step], kc, vc,
+                                table, hq, hkv, hd, bias=bias) for r0 in range(0, n, step)]
+        results.append((torch.cat(qs), kc, vc))
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    want_q = plain.rope_neox((qkv.cpu() + bias.cpu())[:, :hq * hd].numpy(), pos.cpu().numpy(), hd, 1e6, rot, None)
+    close(results[0][0], want_q, atol=2e-2, rtol=8e-3, what="q of the long prompt")
+
+
 def test_rope_reference_vectors():
     """/root/reference/tests/core/test_nn.cpp:221-290: position 0 is the identity; with
     head size 2 and an angle of pi/2, [1,0] turns into [0,1]; pairs are (i, i+half)."""
