@@ -30,14 +30,15 @@ constexpr int kMaxSlices = 8;  // K slices of a product that the fused kernel ad
 // Sum of the squares of a block's kept values: per thread in ascending order, a fixed butterfly
 // over the wave, then wave by wave in ascending order; all in double
 // (/root/reference/core/src/nn/cpu_reduce.h:55-57 sums float products in double).
+template <int WAVES = kNormWaves>
 __device__ __forceinline__ double block_sum(double part) {
-  __shared__ double wave_part[kNormWaves];
+  __shared__ double wave_part[WAVES];
   part = wave_sum(part);
   if ((threadIdx.x & 63) == 0) wave_part[threadIdx.x >> 6] = part;
   __syncthreads();
   double total = 0.0;
 #pragma unroll
-  for (int k = 0; k < kNormWaves; ++k) total += wave_part[k];
+  for (int k = 0; k < WAVES; ++k) total += wave_part[k];
   return total;
 }
 
@@ -56,11 +57,13 @@ __device__ __forceinline__ void write_normed(TO *yr, const float4 &v, int g, flo
   }
 }
 
-// One block per row.  A thread takes float4 groups tid and tid + 1024; its loads are issued
+// One block per row.  A thread takes float4 groups tid, tid + THREADS, ...; its loads are issued
 // unconditionally (from a clamped address) so that all are in flight together, and the groups
-// stay in registers for the second pass.  Rows wider than 8192, or not readable in groups of
-// four, go through the scalar tail loops.
-template <typename TO>
+// stay in registers for the second pass.  Rows wider than 4 * KEEP * THREADS, or not readable in
+// groups of four, go through the scalar tail loops.  Few rows: 1024 threads keeping two groups
+// each, to have the row's loads in flight at once; many rows: 256 threads keeping four, so
+// that eight rows share a CU.
+template <typename TO, int kNormThreads, int kNormKeep>
 __global__ void __launch_bounds__(kNormThreads)
 rmsnorm_kernel(TO *__restrict__ y, const float *__restrict__ x, const void *__restrict__ w,
                int w_dtype, const int32_t *__restrict__ rows, int width, float eps) {
@@ -87,7 +90,7 @@ rmsnorm_kernel(TO *__restrict__ y, const float *__restrict__ x, const void *__re
     const float v = xr[i];
     part += double(v * v);
   }
-  const double total = block_sum(part);
+  const double total = block_sum<kNormThreads / 64>(part);
   const float mean = float(total / double(width));
   const float inv = 1.0f / sqrtf(mean + eps);
 #pragma unroll
@@ -211,9 +214,13 @@ extern "C" int sb_rmsnorm(void *y, int out_dtype, const float *x, const void *w,
   SB_REQUIRE(eps >= 0.0f, "sb_rmsnorm: eps must not be negative");
   if (n_rows == 0) return SB_OK;
   hipStream_t s = (hipStream_t)stream;
-  if (out_dtype == SB_F32)
-    rmsnorm_kernel<float><<<n_rows, kNormThreads, 0, s>>>((float *)y, x, w, w_dtype, rows, width, eps);
-  else
-    rmsnorm_kernel<bf16_t><<<n_rows, kNormThreads, 0, s>>>((bf16_t *)y, x, w, w_dtype, rows, width, eps);
+  const bool many = n_rows >= 256;
+  if (out_dtype == SB_F32) {
+    if (many) rmsnorm_kernel<float, 256, 4><<<n_rows, 256, 0, s>>>((float *)y, x, w, w_dtype, rows, width, eps);
+    else rmsnorm_kernel<float, 1024, 2><<<n_rows, 1024, 0, s>>>((float *)y, x, w, w_dtype, rows, width, eps);
+  } else {
+    if (many) rmsnorm_kernel<bf16_t, 256, 4><<<n_rows, 256, 0, s>>>((bf16_t *)y, x, w, w_dtype, rows, width, eps);
+    else rmsnorm_kernel<bf16_t, 1024, 2><<<n_rows, 1024, 0, s>>>((bf16_t *)y, x, w, w_dtype, rows, width, eps);
+  }
   return sb::check_launch("sb_rmsnorm");
 }

@@ -43,11 +43,12 @@ def test_embed(dtype):
     assert torch.isnan(bad).all()          # an id outside the table never reads memory it does not own
 
 
-@pytest.mark.parametrize("width", [64, 201, 338, 3584])
+@pytest.mark.parametrize("n_rows", [7, 300])       # few rows and many rows take different block shapes
+@pytest.mark.parametrize("width", [64, 201, 338, 3584, 5000])
 @pytest.mark.parametrize("out_dtype, w_dtype", [(F32, F32), (BF16, BF16), (BF16, F32)])
-def test_rmsnorm(width, out_dtype, w_dtype):
+def test_rmsnorm(width, out_dtype, w_dtype, n_rows):
     from sonicboom_amd import ops
-    x = randn(7, width, scale=3.0)
+    x = randn(n_rows, width, scale=3.0)
     w = (1.0 + randn(width, scale=0.1)).to(w_dtype)
     eps = 1e-5
     want = plain.rms_norm(x.numpy(), w.float().numpy(), eps)
