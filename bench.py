@@ -2,6 +2,7 @@
 on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
+                    [--sizes 7b|14b|72b] [--prompt T] [--context C]
 
 A "step" is one decode step: every sequence of the batch goes on by one token
 (step function, greedy choice on the device, the token fed back).  The default
@@ -28,6 +29,12 @@ CONFIG_7B = {
     "max_position_embeddings": 32768, "tie_word_embeddings": False, "use_sliding_window": False,
     "hidden_act": "silu",
 }
+# the other sizes the baseline names, for runs beyond the default one (--sizes)
+CONFIG_14B = dict(CONFIG_7B, num_hidden_layers=48, hidden_size=5120, num_attention_heads=40,
+                  num_key_value_heads=8, intermediate_size=13824)
+CONFIG_72B = dict(CONFIG_7B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
+                  num_key_value_heads=8, intermediate_size=29568)
+SIZES = {"7b": ("Qwen2.5-7B", CONFIG_7B), "14b": ("Qwen2.5-14B", CONFIG_14B), "72b": ("Qwen2.5-72B", CONFIG_72B)}
 CONTEXT = 4096
 PROMPT = 2048
 
@@ -57,12 +64,16 @@ def decode_bytes(m, batch, lengths):
 
 
 def main() -> int:
+    global PROMPT, CONTEXT
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--layers", type=int, default=0, help="run fewer layers than the configuration has")
+    ap.add_argument("--sizes", choices=sorted(SIZES), default="7b", help="layer sizes (default: the benchmark's)")
+    ap.add_argument("--prompt", type=int, default=PROMPT, help="cached prompt tokens per sequence")
+    ap.add_argument("--context", type=int, default=CONTEXT, help="cache size per sequence")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--no-graph", action="store_true", help="launch decode steps kernel by kernel")
     a = ap.parse_args()
@@ -76,7 +87,9 @@ def main() -> int:
     from sonicboom_amd.engine import DecoderModel, Engine, StepEntry
     from sonicboom_amd.engine.decode import DecodeLoop
 
-    cfg = dict(CONFIG_7B)
+    PROMPT, CONTEXT = a.prompt, max(a.context, a.prompt + a.steps + a.warmup + 64)
+    model_name, base_cfg = SIZES[a.sizes]
+    cfg = dict(base_cfg)
     full_layers = cfg["num_hidden_layers"]
     if a.layers:
         cfg["num_hidden_layers"] = a.layers
@@ -98,7 +111,7 @@ def main() -> int:
         torch.cuda.synchronize()
         return time.perf_counter() - t
 
-    # ---- prefill of one 2,048-token prompt ------------------------------------------------
+    # ---- prefill of one prompt (2,048 tokens unless --prompt says otherwise) ----------------
     engine = Engine(model, max_tokens=CONTEXT)
     times = []
     for i in range(5):
@@ -154,12 +167,12 @@ def main() -> int:
             print(f"[bench] decode b{b}: {points[f'decode_b{b}']} tok/s", file=sys.stderr, flush=True)
 
     line = {
-        "metric": "decode tokens/s, Qwen2.5-7B sizes, batch 8, 2048-token cached prompts",
+        "metric": f"decode tokens/s, {model_name} sizes, batch {a.batch}, {PROMPT}-token cached prompts",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
         "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {
-            "model": "Qwen2.5-7B sizes, random bf16 weights", "layers": cfg["num_hidden_layers"],
+            "model": f"{model_name} sizes, random bf16 weights", "layers": cfg["num_hidden_layers"],
             "layers_of_configuration": full_layers, "hidden_size": m["d"], "num_attention_heads": m["hq"],
             "num_key_value_heads": m["hkv"], "head_dim": m["hd"], "intermediate_size": m["ff"],
             "vocab_size": m["v"], "rope_theta": cfg["rope_theta"], "rms_norm_eps": cfg["rms_norm_eps"],
