@@ -108,7 +108,8 @@ rmsnorm_kernel(TO *__restrict__ y, const float *__restrict__ x, const void *__re
 // x[t,:] += sum_s partial[s][t][:] (+ bias), then optionally y[t,:] = rmsnorm(x[t,:]) * w.
 // The slices are added in ascending order, then the bias, then the residual: the order of the
 // unfused kernels (product, bias, residual).  width % 4 == 0 and width <= 8192 (host-checked).
-template <typename TO>
+// KEEP: float4 groups of the row per thread (1 for rows up to 4096 wide: nothing is loaded twice).
+template <typename TO, int KEEP>
 __global__ void __launch_bounds__(kNormThreads)
 reduce_resid_norm_kernel(TO *__restrict__ y, float *__restrict__ x, const float *__restrict__ partial,
                          int n_slices, size_t slice_stride, const void *__restrict__ bias, int bias_dtype,
@@ -119,10 +120,10 @@ reduce_resid_norm_kernel(TO *__restrict__ y, float *__restrict__ x, const float 
   const int tid = threadIdx.x;
   const int n_groups = width / 4;
 
-  float4 keep[kNormKeep];
+  float4 keep[KEEP];
   double part = 0.0;
 #pragma unroll
-  for (int i = 0; i < kNormKeep; ++i) {
+  for (int i = 0; i < KEEP; ++i) {
     const int g = tid + i * kNormThreads;
     const int gc = min(g, n_groups - 1);
     float4 p[kMaxSlices];
@@ -151,7 +152,7 @@ reduce_resid_norm_kernel(TO *__restrict__ y, float *__restrict__ x, const float 
   const float inv = 1.0f / sqrtf(mean + eps);
   TO *yr = y + size_t(r) * width;
 #pragma unroll
-  for (int i = 0; i < kNormKeep; ++i) {
+  for (int i = 0; i < KEEP; ++i) {
     const int g = tid + i * kNormThreads;
     if (g < n_groups) write_normed(yr, keep[i], g, inv, w, w_dtype);
   }
@@ -181,12 +182,18 @@ extern "C" int sb_reduce_resid_norm(void *y, int y_dtype, float *x, const float 
   if (n_rows == 0) return SB_OK;
   hipStream_t s = (hipStream_t)stream;
   const size_t stride = size_t(n_rows) * width;
-  if (!do_norm || y_dtype == SB_F32)
-    reduce_resid_norm_kernel<float><<<n_rows, kNormThreads, 0, s>>>(
-        (float *)y, x, partial, n_slices, stride, bias, bias_dtype, w, w_dtype, width, eps, do_norm);
-  else
-    reduce_resid_norm_kernel<bf16_t><<<n_rows, kNormThreads, 0, s>>>(
-        (bf16_t *)y, x, partial, n_slices, stride, bias, bias_dtype, w, w_dtype, width, eps, do_norm);
+#define SB_GO(TO, KEEP)                                                                \
+  reduce_resid_norm_kernel<TO, KEEP><<<n_rows, kNormThreads, 0, s>>>(                 \
+      (TO *)y, x, partial, n_slices, stride, bias, bias_dtype, w, w_dtype, width, eps, do_norm)
+  const bool narrow = width <= 4 * kNormThreads;
+  if (!do_norm || y_dtype == SB_F32) {
+    if (narrow) SB_GO(float, 1);
+    else SB_GO(float, kNormKeep);
+  } else {
+    if (narrow) SB_GO(bf16_t, 1);
+    else SB_GO(bf16_t, kNormKeep);
+  }
+#undef SB_GO
   return sb::check_launch("sb_reduce_resid_norm");
 }
 

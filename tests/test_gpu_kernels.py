@@ -60,6 +60,31 @@ def test_rmsnorm(width, out_dtype, w_dtype, n_rows):
     assert torch.equal(picked.cpu(), got.cpu()[rows.long()])
 
 
+@pytest.mark.parametrize("width", [64, 100, 3584, 5120, 8192])
+@pytest.mark.parametrize("n_slices", [1, 5, 8])
+@pytest.mark.parametrize("out_dtype", [F32, BF16])
+def test_reduce_resid_norm(width, n_slices, out_dtype):
+    """x += slices (+ bias), then the norm of the new x, in one pass: rows narrower and wider than
+    what a thread keeps in one group of four."""
+    from sonicboom_amd import ops
+    rows, eps = 9, 1e-6
+    partial = randn(n_slices, rows, width, seed=1)
+    x = randn(rows, width, scale=2.0, seed=2)
+    bias = randn(width, scale=0.1, seed=3)
+    w = 1.0 + randn(width, scale=0.1, seed=4)
+    new_x = x.double() + partial.double().sum(0) + bias.double()
+    want_y = plain.rms_norm(new_x.float().numpy(), w.numpy(), eps)
+    xd = x.to(DEV)
+    y = ops.reduce_resid_norm(partial.to(DEV), bias.to(DEV), xd, w.to(DEV), eps, out_dtype)
+    close(xd, new_x, atol=2e-6 * n_slices, rtol=2e-6, what="residual")
+    tol = dict(atol=2e-5, rtol=2e-5) if out_dtype == F32 else dict(atol=1e-2, rtol=8e-3)
+    close(y, want_y, what="normed", **tol)
+    # without a norm: only the sum
+    xd2 = x.to(DEV)
+    assert ops.reduce_resid_norm(partial.to(DEV), None, xd2, None, eps, None) is None
+    close(xd2, x.double() + partial.double().sum(0), atol=2e-6 * n_slices, rtol=2e-6, what="sum only")
+
+
 def test_rmsnorm_reference_vectors():
     """/root/reference/tests/core/test_nn.cpp:172-219."""
     from sonicboom_amd import ops
