@@ -109,7 +109,8 @@ rmsnorm_kernel(TO *__restrict__ y, const float *__restrict__ x, const void *__re
 // The slices are added in ascending order, then the bias, then the residual: the order of the
 // unfused kernels (product, bias, residual).  width % 4 == 0 and width <= 8192 (host-checked).
 // KEEP: float4 groups of the row per thread (1 for rows up to 4096 wide: nothing is loaded twice).
-template <typename TO, int KEEP>
+// SLICES: how many slices the unrolled loop loads (the count itself, or 8 for "up to 8").
+template <typename TO, int KEEP, int SLICES>
 __global__ void __launch_bounds__(kNormThreads)
 reduce_resid_norm_kernel(TO *__restrict__ y, float *__restrict__ x, const float *__restrict__ partial,
                          int n_slices, size_t slice_stride, const void *__restrict__ bias, int bias_dtype,
@@ -126,14 +127,14 @@ reduce_resid_norm_kernel(TO *__restrict__ y, float *__restrict__ x, const float 
   for (int i = 0; i < KEEP; ++i) {
     const int g = tid + i * kNormThreads;
     const int gc = min(g, n_groups - 1);
-    float4 p[kMaxSlices];
+    float4 p[SLICES];
 #pragma unroll
-    for (int s = 0; s < kMaxSlices; ++s)
+    for (int s = 0; s < SLICES; ++s)
       p[s] = reinterpret_cast<const float4 *>(pr + min(s, n_slices - 1) * slice_stride)[gc];
     const float4 old = reinterpret_cast<const float4 *>(xr)[gc];
     float4 acc = p[0];
 #pragma unroll
-    for (int s = 1; s < kMaxSlices; ++s)
+    for (int s = 1; s < SLICES; ++s)
       if (s < n_slices) { acc.x += p[s].x; acc.y += p[s].y; acc.z += p[s].z; acc.w += p[s].w; }
     if (bias) {
       acc.x += ld_dyn(bias, bias_dtype, gc * 4 + 0); acc.y += ld_dyn(bias, bias_dtype, gc * 4 + 1);
@@ -182,9 +183,17 @@ extern "C" int sb_reduce_resid_norm(void *y, int y_dtype, float *x, const float 
   if (n_rows == 0) return SB_OK;
   hipStream_t s = (hipStream_t)stream;
   const size_t stride = size_t(n_rows) * width;
-#define SB_GO(TO, KEEP)                                                                \
-  reduce_resid_norm_kernel<TO, KEEP><<<n_rows, kNormThreads, 0, s>>>(                 \
+#define SB_GO2(TO, KEEP, SLICES)                                                       \
+  reduce_resid_norm_kernel<TO, KEEP, SLICES><<<n_rows, kNormThreads, 0, s>>>(         \
       (TO *)y, x, partial, n_slices, stride, bias, bias_dtype, w, w_dtype, width, eps, do_norm)
+  // the usual slice counts have loops of their own length, so that no slice is loaded twice
+#define SB_GO(TO, KEEP)                          \
+  do {                                           \
+    if (n_slices == 1) SB_GO2(TO, KEEP, 1);      \
+    else if (n_slices <= 4) SB_GO2(TO, KEEP, 4); \
+    else if (n_slices == 5) SB_GO2(TO, KEEP, 5); \
+    else SB_GO2(TO, KEEP, kMaxSlices);           \
+  } while (0)
   const bool narrow = width <= 4 * kNormThreads;
   if (!do_norm || y_dtype == SB_F32) {
     if (narrow) SB_GO(float, 1);
@@ -194,6 +203,7 @@ extern "C" int sb_reduce_resid_norm(void *y, int y_dtype, float *x, const float 
     else SB_GO(bf16_t, kNormKeep);
   }
 #undef SB_GO
+#undef SB_GO2
   return sb::check_launch("sb_reduce_resid_norm");
 }
 

@@ -16,15 +16,16 @@ constexpr int kMaxPairs = 256;   // rotated pairs of a head at most (head sizes 
 constexpr int kMaxSlices = 8;    // K slices of the projection that are added on load
 
 // Element e of a qkv row: the sum of the product's K slices in ascending order, then the bias.
-template <typename TI>
+// SLICES: length of the unrolled loop (1, 4 or 8: at least n_slices).
+template <int SLICES, typename TI>
 __device__ __forceinline__ float qkv_at(const TI *r, size_t e, int n_slices, size_t slice_stride,
                                         const float *bias) {
-  float p[kMaxSlices];
+  float p[SLICES];
 #pragma unroll
-  for (int s = 0; s < kMaxSlices; ++s) p[s] = s < n_slices ? ld_f(r + s * slice_stride, e) : 0.f;
+  for (int s = 0; s < SLICES; ++s) p[s] = s < n_slices ? ld_f(r + s * slice_stride, e) : 0.f;
   float v = p[0];
 #pragma unroll
-  for (int s = 1; s < kMaxSlices; ++s)
+  for (int s = 1; s < SLICES; ++s)
     if (s < n_slices) v += p[s];
   if (bias) v = v + bias[e];
   return v;
@@ -35,7 +36,7 @@ __device__ __forceinline__ float qkv_at(const TI *r, size_t e, int n_slices, siz
 // to have enough blocks; many rows (prefill): all heads of a row in one block, so that the
 // row's cosines and sines and its page look-up are worked out once and every thread has
 // several pairs to move.
-template <typename TI, typename TQ, typename TC>
+template <typename TI, typename TQ, typename TC, int SLICES>
 __global__ void __launch_bounds__(256)
 rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_stride, int n_slices,
                size_t slice_stride, const float *__restrict__ bias,
@@ -96,7 +97,7 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
 #pragma unroll 1
       for (int d = w; d < head_dim; d += per_head)
         st_f(v_cache, v_base + kh * head_step + size_t(d) * SB_PAGE,
-             qkv_at(r, hoff + d, n_slices, slice_stride, bias));
+             qkv_at<SLICES>(r, hoff + d, n_slices, slice_stride, bias));
       continue;
     }
     const bool is_q = head < heads_q;
@@ -105,8 +106,8 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
     if (rotate && w < half) {
       const int i = w;
       const float c = cs[i], sv = sn[i];
-      const float x0 = qkv_at(r, hoff + i, n_slices, slice_stride, bias);
-      const float x1 = qkv_at(r, hoff + i + half, n_slices, slice_stride, bias);
+      const float x0 = qkv_at<SLICES>(r, hoff + i, n_slices, slice_stride, bias);
+      const float x1 = qkv_at<SLICES>(r, hoff + i + half, n_slices, slice_stride, bias);
       const float y0 = x0 * c - x1 * sv;
       const float y1 = x0 * sv + x1 * c;
       if (is_q) {
@@ -118,7 +119,7 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
       }
     } else {
       const int d = first_plain + (w - (rotate ? half : 0));
-      const float v = qkv_at(r, hoff + d, n_slices, slice_stride, bias);
+      const float v = qkv_at<SLICES>(r, hoff + d, n_slices, slice_stride, bias);
       if (is_q) st_f(qo, hoff + d, v);
       else st_f(k_cache, k_base + kh * head_step + d, v);
     }
@@ -162,7 +163,11 @@ extern "C" int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int q
   const dim3 grid(n_rows, (n_heads + heads_per_block - 1) / heads_per_block);
   SB_SUPPORT(grid.y <= 65535, "sb_rope_kv_store: too many heads");
 #define SB_GO(TI, TQ, TC)                                                                        \
-  rope_kv_kernel<TI, TQ, TC><<<grid, 256, 0, s>>>(                                              \
+  if (n_slices == 1) SB_GO2(TI, TQ, TC, 1);                                                        \
+  else if (n_slices <= 4) SB_GO2(TI, TQ, TC, 4);                                                   \
+  else SB_GO2(TI, TQ, TC, kMaxSlices)
+#define SB_GO2(TI, TQ, TC, SLICES)                                                               \
+  rope_kv_kernel<TI, TQ, TC, SLICES><<<grid, 256, 0, s>>>(                                      \
       (TQ *)q_out, (const TI *)qkv, row_stride, n_slices, slice_stride, bias, inv_freq, freq_factors,   \
       rot_dims, row_pos, row_seq,                                                                    \
       (TC *)k_cache, (TC *)v_cache, page_table, max_pages, n_pages_total, heads_q, heads_kv, head_dim,  \
@@ -179,5 +184,6 @@ extern "C" int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int q
     default: SB_GO(bf16_t, bf16_t, bf16_t); break;
   }
 #undef SB_GO
+#undef SB_GO2
   return sb::check_launch("sb_rope_kv_store");
 }
