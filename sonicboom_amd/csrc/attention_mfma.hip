@@ -599,6 +599,9 @@ attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *
   const int group = heads_q / heads_kv;
   const int head_tiles = (group + 15) / 16;
   const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y - kvh * head_tiles;
+  // the wave's page number does not depend on the position: both look-ups go out together
+  const int pg = chunk * kPagesPerChunk + wave;
+  const int page_looked_up = page_table[size_t(seq) * max_pages + min(pg, max_pages - 1)];
   const int pos = row_pos[seq];
   const int key_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
   const int first_chunk = key_lo / (SB_PAGE * kPagesPerChunk);
@@ -613,9 +616,8 @@ attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *
   load_q(qf[0], q + (size_t(seq) * heads_q + head) * HD, col_ok, lane);
   WaveState<1> st;
   init_state<1>(st);
-  const int pg = chunk * kPagesPerChunk + wave;
   if (pg >= key_lo / SB_PAGE && pg <= pos / SB_PAGE && pg < max_pages) {
-    const int page = page_table[size_t(seq) * max_pages + pg];
+    const int page = page_looked_up;
     if (page >= 0 && page < n_pages_total) {
       const size_t off = (size_t(page) * heads_kv + kvh) * SB_PAGE * HD;
       attend_page<1>(st, qf, k_cache + off, v_cache + off, pg * SB_PAGE, col_ok ? pos : -1, key_lo, key_lo, pos,
