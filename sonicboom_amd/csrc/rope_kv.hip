@@ -54,6 +54,27 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
   const int n_heads = heads_q + 2 * heads_kv;
   const int h_begin = blockIdx.y * heads_per_block, h_end = min(h_begin + heads_per_block, n_heads);
 
+  const bool rotate = inv_freq != nullptr;
+  const int first_plain = rotate ? rot_dims : 0;
+  const int plain = head_dim - first_plain;
+  // work items of a head: `half` rotated pairs, then `plain` elements that are copied
+  const int per_head = (rotate ? half : 0) + plain;
+  const int n_items = (h_end - h_begin) * per_head;
+
+  // The operands of a thread's first rotated pair do not depend on the position: their loads go
+  // out before the cosines are worked out, not after.
+  float pre0 = 0.f, pre1 = 0.f;
+  bool preloaded = false;
+  if (rotate && int(threadIdx.x) < n_items) {
+    const int head = h_begin + int(threadIdx.x) / per_head, w = int(threadIdx.x) % per_head;
+    if (head < heads_q + heads_kv && w < half) {
+      const size_t hoff = size_t(head) * head_dim;
+      pre0 = qkv_at<SLICES>(r, hoff + w, n_slices, slice_stride, bias);
+      pre1 = qkv_at<SLICES>(r, hoff + w + half, n_slices, slice_stride, bias);
+      preloaded = true;
+    }
+  }
+
   // Where this row's key and value go.
   int page_of_row = 0;
   bool store = heads_kv > 0;
@@ -69,23 +90,19 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
   const size_t k_base = page_base + size_t(pos % SB_PAGE) * head_dim;   // keys   [position][d]
   const size_t v_base = page_base + size_t(pos % SB_PAGE);              // values [d][position]
 
-  // The angle of pair i is the same for every head of the row: cosine and sine once per block.
+  // The angle of pair i is the same for every head of the row: cosine and sine once per block,
+  // the cosines by one half of the threads that take part, the sines by the other.
   __shared__ float cs[kMaxPairs], sn[kMaxPairs];
-  const bool rotate = inv_freq != nullptr;
   if (rotate && h_begin < heads_q + heads_kv) {
-    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    for (int j = threadIdx.x; j < 2 * half; j += blockDim.x) {
+      const int i = j < half ? j : j - half;
       float theta = float(pos) * inv_freq[i];
       if (freq_factors) theta = theta / freq_factors[i];
-      cs[i] = cosf(theta);
-      sn[i] = sinf(theta);
+      if (j < half) cs[i] = cosf(theta);
+      else sn[i] = sinf(theta);
     }
   }
   __syncthreads();
-  const int first_plain = rotate ? rot_dims : 0;
-  const int plain = head_dim - first_plain;
-  // work items of a head: `half` rotated pairs, then `plain` elements that are copied
-  const int per_head = (rotate ? half : 0) + plain;
-  const int n_items = (h_end - h_begin) * per_head;
 #pragma unroll 2
   for (int it = threadIdx.x; it < n_items; it += blockDim.x) {
     const int head = h_begin + it / per_head, w = it % per_head;
@@ -106,8 +123,9 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
     if (rotate && w < half) {
       const int i = w;
       const float c = cs[i], sv = sn[i];
-      const float x0 = qkv_at<SLICES>(r, hoff + i, n_slices, slice_stride, bias);
-      const float x1 = qkv_at<SLICES>(r, hoff + i + half, n_slices, slice_stride, bias);
+      const bool have = preloaded && it == int(threadIdx.x);
+      const float x0 = have ? pre0 : qkv_at<SLICES>(r, hoff + i, n_slices, slice_stride, bias);
+      const float x1 = have ? pre1 : qkv_at<SLICES>(r, hoff + i + half, n_slices, slice_stride, bias);
       const float y0 = x0 * c - x1 * sv;
       const float y1 = x0 * sv + x1 * c;
       if (is_q) {
