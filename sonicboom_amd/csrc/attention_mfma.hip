@@ -187,15 +187,16 @@ __device__ __forceinline__ void attend_half(WaveState<NC> &st, const bf16x8_t (&
 
 // One page (64 keys at absolute positions page_pos .. page_pos+63).  With one column group and a
 // head size up to 128 both halves' fragments are requested before the first product, so a page
-// costs one round trip to memory; otherwise half by half, to stay within the registers.
-template <int NC>
+// costs one round trip to memory (BOTH); otherwise half by half, to stay within the registers
+// (or, when there are many more blocks than the GPU holds at once, to let more of them in).
+template <int NC, bool BOTH = true>
 __device__ __forceinline__ void attend_page(WaveState<NC> &st, const bf16x8_t (&qf)[NC][KS],
                                             const bf16_t *__restrict__ kp, const bf16_t *__restrict__ vp,
                                             int page_pos, int col_pos, int col_lo, int key_lo, int key_hi,
                                             float scale_log2, int lane) {
   const bool use0 = !(page_pos > key_hi || page_pos + 31 < key_lo);
   const bool use1 = !(page_pos + 32 > key_hi || page_pos + 63 < key_lo);
-  if (HD <= 128 && NC == 1) {
+  if (BOTH && HD <= 128 && NC == 1) {
     HalfPage h0, h1;
     if (use0) load_half(h0, kp, vp, 0, lane);
     if (use1) load_half(h1, kp, vp, 1, lane);
@@ -585,6 +586,7 @@ __device__ __forceinline__ void merge_element(bf16_t *__restrict__ out, const fl
   out[(size_t(seq) * heads_q + kvh * group + hh) * HD + d] = f32_to_bf16(l > 0.f ? o / l : 0.f);
 }
 
+template <bool BOTH>
 __global__ void __launch_bounds__(256)
 attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
                    const bf16_t *__restrict__ q,
@@ -620,8 +622,8 @@ attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *
     const int page = page_looked_up;
     if (page >= 0 && page < n_pages_total) {
       const size_t off = (size_t(page) * heads_kv + kvh) * SB_PAGE * HD;
-      attend_page<1>(st, qf, k_cache + off, v_cache + off, pg * SB_PAGE, col_ok ? pos : -1, key_lo, key_lo, pos,
-                     scale_log2, lane);
+      attend_page<1, BOTH>(st, qf, k_cache + off, v_cache + off, pg * SB_PAGE, col_ok ? pos : -1, key_lo, key_lo,
+                           pos, scale_log2, lane);
     }
   }
   float l = st.l[0];
@@ -743,10 +745,21 @@ extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache
   hipStream_t s = (hipStream_t)stream;
   dim3 grid(n_chunks, heads_kv * head_tiles, n_seqs);
   SB_SUPPORT(heads_kv * head_tiles <= 65535, "sb_attn_decode_bf16: too many heads");
-  attn_decode_kernel<<<grid, 256, 0, s>>>((bf16_t *)out, part_o, part_ml, (const bf16_t *)q,
-                                          (const bf16_t *)k_cache, (const bf16_t *)v_cache, page_table,
-                                          max_pages, n_pages_total, row_pos, heads_q, heads_kv, n_chunks,
-                                          scale * kLog2e, window);
+  // Few blocks: a wave asks for its whole page at once (one round trip to memory).  Many more
+  // blocks than the GPU holds at once: half a page at a time, which takes fewer registers and
+  // lets three blocks share a CU instead of two (measured at 2,048 keys: 65 against 69 us at 64
+  // sequences, no gain at 32).
+  const long long n_blocks = (long long)n_chunks * heads_kv * head_tiles * n_seqs;
+  if (n_blocks <= 1536)
+    attn_decode_kernel<true><<<grid, 256, 0, s>>>((bf16_t *)out, part_o, part_ml, (const bf16_t *)q,
+                                                  (const bf16_t *)k_cache, (const bf16_t *)v_cache, page_table,
+                                                  max_pages, n_pages_total, row_pos, heads_q, heads_kv,
+                                                  n_chunks, scale * kLog2e, window);
+  else
+    attn_decode_kernel<false><<<grid, 256, 0, s>>>((bf16_t *)out, part_o, part_ml, (const bf16_t *)q,
+                                                   (const bf16_t *)k_cache, (const bf16_t *)v_cache, page_table,
+                                                   max_pages, n_pages_total, row_pos, heads_q, heads_kv,
+                                                   n_chunks, scale * kLog2e, window);
   rc = sb::check_launch("sb_attn_decode_bf16");
   if (rc != SB_OK || n_chunks == 1) return rc;
   attn_decode_merge_kernel<<<dim3((HD * 16 + 255) / 256, heads_kv * head_tiles, n_seqs), 256, 0, s>>>(

@@ -418,6 +418,19 @@ def test_attention_decode_matrix_cores(hq, hkv, hd, window):
         assert torch.equal(got, again)
 
 
+def test_attention_decode_matrix_cores_many_sequences():
+    """Two hundred sequences: more blocks than the GPU holds at once, which takes the kernel
+    that reads half a page at a time."""
+    from sonicboom_amd import ops
+    hq, hkv, hd = 8, 4, 32
+    rng = np.random.default_rng(5)
+    lens = [int(n) for n in rng.integers(1, 300, size=200)]
+    q, kc, vc, table, rows, scale, want = attention_case(hq, hkv, hd, lens, [[n - 1] for n in lens], 0, seed=9)
+    pos = torch.tensor([p for _, p in rows], dtype=torch.int32)
+    got = ops.attention_decode_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), hq, hkv, hd, scale, 0)
+    close(got, want, atol=1.5e-2, rtol=1e-2, what="decode, 200 sequences")
+
+
 @pytest.mark.parametrize("hq, hkv, hd", MFMA_SHAPES)
 @pytest.mark.parametrize("window", [0, 70])
 def test_attention_prefill_matrix_cores(hq, hkv, hd, window):
