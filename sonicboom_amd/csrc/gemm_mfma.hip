@@ -36,6 +36,10 @@ struct Args {
   int tiles_m, tiles_n;
   int w_tiles;     // packed W: 16-row tiles of one half (ceil(n_out / 16))
   int w_steps;     // packed W: 32-wide k-steps (ceil(n_in / 32))
+  // K cut over the grid (blockIdx.y): slice s multiplies stages [s * stages_per_slice, ...) and
+  // writes its raw sums to partial [slice][n_rows][n_out]; NULL: one slice, the epilogues below
+  float *partial;
+  int stages_per_slice;
 };
 
 // index (in 16-byte chunks) of chunk `chunk` of LDS row `row`, CPR chunks per row
@@ -170,14 +174,16 @@ gemm_mfma_kernel(Args a) {
     else (buf ? lds_b1 : lds_b0)[slot_b0 + (i - kLoadsA) * kThreads] = staged[set][i];
   };
 
-  const int n_k = (a.n_in + BK - 1) / BK;
+  const int n_k_all = (a.n_in + BK - 1) / BK;
+  const int kt_begin = a.partial ? int(blockIdx.y) * a.stages_per_slice : 0;
+  const int n_k = a.partial ? min(kt_begin + a.stages_per_slice, n_k_all) : n_k_all;   // end of this slice
   using Set0 = std::integral_constant<int, 0>;
   using Set1 = std::integral_constant<int, 1>;
 #pragma unroll
-  for (int i = 0; i < kLoads; ++i) issue_load(Set0{}, i, 0);
-  if (DEPTH == 2 && n_k > 1) {
+  for (int i = 0; i < kLoads; ++i) issue_load(Set0{}, i, kt_begin);
+  if (DEPTH == 2 && kt_begin + 1 < n_k) {
 #pragma unroll
-    for (int i = 0; i < kLoads; ++i) issue_load(std::integral_constant<int, DEPTH - 1>{}, i, 1);
+    for (int i = 0; i < kLoads; ++i) issue_load(std::integral_constant<int, DEPTH - 1>{}, i, kt_begin + 1);
   }
 #pragma unroll
   for (int i = 0; i < kLoads; ++i) store_lds(Set0{}, i, 0);
@@ -237,7 +243,7 @@ gemm_mfma_kernel(Args a) {
   };
   using Yes = std::true_type;
   using No = std::false_type;
-  int kt = 0;
+  int kt = kt_begin;
   if (DEPTH == 2) {
     for (; kt + 3 < n_k; kt += 2) {
       stage(Set0{}, Yes{}, Yes{}, kt);
@@ -275,6 +281,14 @@ gemm_mfma_kernel(Args a) {
     for (int e = 0; e < 16; ++e) {
       const int t = t0 + wm * (32 * MT) + i * 32 + 8 * (e >> 2) + row_base + (e & 3);
       if (t >= a.n_rows) continue;
+      if (!GATED && a.partial) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int n = n0 + wn * 64 + j * 32 + col;
+          if (n < a.n_out) a.partial[(size_t(blockIdx.y) * a.n_rows + t) * a.n_out + n] = acc[i][j][e];
+        }
+        continue;
+      }
       if (GATED) {
         const int n = n0 + wn * 32 + col;
         if (n < a.n_out) {
@@ -315,7 +329,10 @@ int launch_one(const Args &a, long long blocks, hipStream_t s) {
                hipGetErrorString(e));
     raised = true;
   }
-  gemm_mfma_kernel<MT, NW, BK, DEPTH, GATED, PACKED, EVEN_K><<<unsigned(blocks), 128 * NW, lds_bytes, s>>>(a);
+  const int n_k = (a.n_in + BK - 1) / BK;
+  const unsigned slices = a.partial ? unsigned((n_k + a.stages_per_slice - 1) / a.stages_per_slice) : 1u;
+  gemm_mfma_kernel<MT, NW, BK, DEPTH, GATED, PACKED, EVEN_K>
+      <<<dim3(unsigned(blocks), slices), 128 * NW, lds_bytes, s>>>(a);
   return SB_OK;
 }
 
@@ -382,6 +399,7 @@ extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void
   a.y = y; a.y_dtype = y_dtype; a.x = (const bf16_t *)x; a.w = (const bf16_t *)w;
   a.bias = bias; a.bias_dtype = bias_dtype; a.resid = resid;
   a.n_rows = n_rows; a.n_out = n_out; a.n_in = n_in; a.gated = gated ? 1 : 0;
+  a.partial = nullptr; a.stages_per_slice = 0;
   int variant = pick_shape(n_rows, n_out, a.gated);
   if (g_force_variant >= 0 && g_force_variant < 3) variant = g_force_variant;
   if (!packed) variant = 0;       // the bigger tiles are built for packed weights only
@@ -405,6 +423,60 @@ extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void
   else rc = launch<4, 4, 64, 1, false>(a, blocks, packed, s);
   if (rc != SB_OK) return rc;
   return sb::check_launch("sb_gemm_mfma_bf16");
+}
+
+namespace {
+// K slices of the partial form: enough blocks for the GPU (one 128 x 128 tile per CU and slice),
+// every slice at least four stages of 64 long, at most the eight that the consumers add.
+int partial_slices(int n_rows, int n_out, int n_in) {
+  const long long tiles = (long long)((n_rows + 127) / 128) * ((n_out + 127) / 128);
+  const int n_k = (n_in + 63) / 64;
+  long long s = (224 + tiles - 1) / tiles;
+  if (s > n_k / 4) s = n_k / 4;
+  if (s > 8) s = 8;
+  if (s < 1) s = 1;
+  const int per = int((n_k + s - 1) / s);
+  return (n_k + per - 1) / per;
+}
+}  // namespace
+
+// Slices sb_gemm_mfma_partial_bf16 writes for these sizes.
+extern "C" int sb_gemm_mfma_slices(int n_rows, int n_out, int n_in) { return partial_slices(n_rows, n_out, n_in); }
+
+// The raw product X W^T in K slices: partial float [slices][n_rows][n_out], for a consumer that
+// adds the slices itself.  For few rows against a narrow, long matrix, where one slice would not
+// give the GPU enough tiles.  128 x 128 tiles.
+extern "C" int sb_gemm_mfma_partial_bf16(float *partial, const void *x, const void *w, int n_rows, int n_out,
+                                         int n_in, int packed, void *stream) {
+  SB_REQUIRE(partial && x && w, "sb_gemm_mfma_partial_bf16: null pointer");
+  SB_REQUIRE(n_rows >= 0 && n_out > 0 && n_in > 0, "sb_gemm_mfma_partial_bf16: bad sizes rows=%d out=%d in=%d",
+             n_rows, n_out, n_in);
+  SB_SUPPORT(n_in % 8 == 0, "sb_gemm_mfma_partial_bf16: inner size %d is not a multiple of 8", n_in);
+  SB_SUPPORT((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) % 16 == 0,
+             "sb_gemm_mfma_partial_bf16: operands must be 16-byte aligned");
+  if (n_rows == 0) return SB_OK;
+  Args a;
+  a.y = nullptr; a.y_dtype = SB_F32; a.x = (const bf16_t *)x; a.w = (const bf16_t *)w;
+  a.bias = nullptr; a.bias_dtype = 0; a.resid = nullptr;
+  a.n_rows = n_rows; a.n_out = n_out; a.n_in = n_in; a.gated = 0;
+  a.tiles_m = (n_rows + 127) / 128;
+  a.tiles_n = (n_out + 127) / 128;
+  const long long blocks = (long long)a.tiles_m * a.tiles_n;
+  SB_SUPPORT(blocks <= 0x7fffffffLL, "sb_gemm_mfma_partial_bf16: too many tiles");
+  const unsigned long long w_rows = (unsigned long long)((n_out + 15) / 16 * 16);
+  const unsigned long long k_padded = (unsigned long long)((n_in + 31) / 32 * 32);
+  SB_SUPPORT(((unsigned long long)n_rows + 1) * n_in * 2 < (1ull << 32) - (1ull << 20) &&
+                 w_rows * k_padded * 2 < (1ull << 32) - (1ull << 20),
+             "sb_gemm_mfma_partial_bf16: an operand of 4 GiB or more");
+  a.w_tiles = (n_out + 15) / 16;
+  a.w_steps = (n_in + 31) / 32;
+  const int slices = partial_slices(n_rows, n_out, n_in);
+  const int n_k = (n_in + 63) / 64;
+  a.partial = partial;
+  a.stages_per_slice = (n_k + slices - 1) / slices;
+  const int rc = launch<2, 2, 64, 2, true>(a, blocks, packed, (hipStream_t)stream);
+  if (rc != SB_OK) return rc;
+  return sb::check_launch("sb_gemm_mfma_partial_bf16");
 }
 
 // Measurement hook: -1 lets the launcher choose; 0, 1, 2 force the 128 x 128, 256 x 128 and

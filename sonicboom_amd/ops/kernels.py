@@ -288,10 +288,17 @@ def gemm_bf16_partial(x: torch.Tensor, w: torch.Tensor, packed_shape=None) -> Op
     if t > SKINNY_MAX_ROWS or t == 0 or k % 8 or x.data_ptr() % 16 or w.data_ptr() % 16:
         return None
     lib = library.core()
+    packed = 1 if packed_shape is not None else 0
+    if t >= TILED_PARTIAL_MIN_ROWS and packed:
+        # more than a few rows against a narrow, long matrix: the tiled kernel with K cut over the
+        # grid (X goes through LDS once per block instead of once per wave)
+        slices = lib.sb_gemm_mfma_slices(t, n, k)
+        partial = torch.empty((slices, t, n), dtype=torch.float32, device=x.device)
+        check(lib.sb_gemm_mfma_partial_bf16(_p(partial), _p(x), _p(w), t, n, k, packed, _stream()))
+        return partial
     slices = lib.sb_gemm_skinny_slices(t, n, k)
     partial = torch.empty((slices, t, n), dtype=torch.float32, device=x.device)
-    check(lib.sb_gemm_skinny_partial_bf16(_p(partial), _p(x), _p(w), t, n, k, 1 if packed_shape is not None else 0,
-                                          _stream()))
+    check(lib.sb_gemm_skinny_partial_bf16(_p(partial), _p(x), _p(w), t, n, k, packed, _stream()))
     return partial
 
 
@@ -404,6 +411,7 @@ def gemm_tile_shape(shape: Optional[int]):
 
 MFMA_MAX_HEAD_DIM = 256
 TILED_MIN_TILES = 256
+TILED_PARTIAL_MIN_ROWS = 17
 
 
 def attention_mfma_ok(q_dtype, cache_dtype, head_dim: int) -> bool:

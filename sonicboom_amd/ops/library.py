@@ -41,6 +41,8 @@ _OPTIONAL_SIGNATURES = {
     "sb_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _P, _Z, _P],
     "sb_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _P],
     "sb_gemm_mfma_force": [_I],
+    "sb_gemm_mfma_slices": [_I, _I, _I],
+    "sb_gemm_mfma_partial_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
 }
 _ATTN_SIGNATURES = {
     # out, q, k_cache, v_cache, page_table, max_pages, n_pages, row_pos, part_o, part_ml, n_seqs,

@@ -204,6 +204,27 @@ def test_gemm_bf16_wide_matrix_with_few_rows(t):
         close(got, g / (1.0 + torch.exp(-g)) * u, atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"wide gated {inner}")
 
 
+@pytest.mark.parametrize("t", [1, 8, 16, 17, 40, 64])
+@pytest.mark.parametrize("n, k", [(100, 96), (224, 200), (3584, 512), (264, 2368), (72, 18944 // 8)])
+@pytest.mark.parametrize("packed", [False, True])
+def test_gemm_bf16_partial_slices_add_up(t, n, k, packed):
+    """The product in K slices (weight-streaming kernel up to 16 rows, tiled kernel with K cut
+    over the grid from 17 rows on, for packed weights): the slices add up to x w^T, and the
+    consumers that add them give the fused results."""
+    from sonicboom_amd import ops
+    x, w = randn(t, k, dtype=BF16), randn(n, k, dtype=BF16, scale=0.05)
+    wd = w.to(DEV)
+    partial = ops.gemm_bf16_partial(x.to(DEV), ops.pack_weight(wd) if packed else wd,
+                                    packed_shape=(n, k) if packed else None)
+    assert partial is not None and partial.shape[1:] == (t, n) and 1 <= partial.shape[0] <= 8
+    close(partial.double().sum(0), ref_gemm(x, w), atol=3e-5 * math.sqrt(k), rtol=1e-5, what="sum of the slices")
+    if n % 4 == 0:
+        resid, bias = randn(t, n), randn(n, scale=0.1)
+        rd = resid.to(DEV)
+        ops.reduce_resid_norm(partial, bias.to(DEV), rd, None, 1e-6, None)
+        close(rd, ref_gemm(x, w, bias, resid), atol=3e-5 * math.sqrt(k), rtol=1e-5, what="slices + bias + residual")
+
+
 def test_gemm_bf16_refuses_what_it_cannot_take():
     from sonicboom_amd import ops
     x, w = randn(4, 100, dtype=BF16).to(DEV), randn(8, 100, dtype=BF16).to(DEV)
