@@ -168,3 +168,25 @@ def test_no_weights_in_folder(tmp_path, tiny_configs):
     spec = build_spec(Qwen2Config.from_dict(tiny_configs["A"]))
     with pytest.raises(WeightError, match="neither"):
         load_tensors(str(tmp_path), spec, "float32", "cpu")
+
+
+def test_command_writes_a_model_folder(tmp_path, tiny_configs):
+    """bin/sb-random-model: same bytes as write_random_model, an error and status 1 for a bad config."""
+    import json
+    import os
+    import subprocess
+    import sys
+    from sonicboom_amd.weights import write_random_model
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cfg_path = tmp_path / "config.json"
+    cfg_path.write_text(json.dumps(tiny_configs["B"]))
+    cmd = [sys.executable, os.path.join(root, "bin", "sb-random-model")]
+    r = subprocess.run(cmd + [str(cfg_path), str(tmp_path / "a"), "--seed", "11"], capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    write_random_model(str(tmp_path / "b"), dict(tiny_configs["B"]), seed=11)
+    assert (tmp_path / "a" / "model.safetensors").read_bytes() == (tmp_path / "b" / "model.safetensors").read_bytes()
+    bad = dict(tiny_configs["B"])
+    del bad["hidden_size"]
+    cfg_path.write_text(json.dumps(bad))
+    r = subprocess.run(cmd + [str(cfg_path), str(tmp_path / "c")], capture_output=True, text=True)
+    assert r.returncode == 1 and "hidden_size" in r.stderr
