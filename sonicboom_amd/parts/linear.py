@@ -64,7 +64,8 @@ class Linear:
 
     def partial(self, x: torch.Tensor) -> Optional[torch.Tensor]:
         """The raw product in K slices, float32 [slices, rows, out] (bias and residual left to the
-        consumer), when the weight-streaming kernel takes this call; else None."""
+        consumer), when a kernel that cuts K over the grid takes this call (few rows, or a few
+        hundred against a narrow matrix); else None."""
         if self.packed is None or self.gated or x.dtype != torch.bfloat16:
             return None
         return ops.gemm_bf16_partial(x, self.packed, packed_shape=(self.rows, self.n_in))
