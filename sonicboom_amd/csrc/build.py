@@ -38,7 +38,7 @@ FLAGS = [
 
 CORE_SOURCES = [
     "status.hip", "embed_norm.hip", "elementwise.hip", "gemm_plain.hip", "rope_kv.hip",
-    "attention_plain.hip", "sampling.hip", "gemm_skinny.hip", "gemm_mfma.hip",
+    "attention_plain.hip", "sampling.hip", "gemm_skinny.hip", "gemm_stream.hip", "gemm_mfma.hip",
 ]
 HEADERS = ["common.cuh", "sb_hip.h", "mfma.cuh"]
 ATTN_SOURCES = ["attention_mfma.hip"]

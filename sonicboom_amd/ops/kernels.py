@@ -362,8 +362,8 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], re
               out_dtype: torch.dtype, out: Optional[torch.Tensor] = None, gated: bool = False,
               packed_shape=None) -> Optional[torch.Tensor]:
     """bfloat16 product on the matrix cores: y = x w^T (+bias) (+resid), or with ``gated``
-    y = silu(x wg^T) * (x wu^T) for w = [wg; wu].  Up to 64 rows go to the weight-streaming
-    kernel, more to the tiled one.  ``packed_shape`` = (rows of w, inner size) says that ``w`` is
+    y = silu(x wg^T) * (x wu^T) for w = [wg; wu].  Up to 64 rows go to one of the two
+    weight-streaming kernels, more to the tiled one.  ``packed_shape`` = (rows of w, inner size) says that ``w`` is
     in the layout of :func:`pack_weight`.  Returns None when the sizes fit neither kernel (an
     inner size that is not a multiple of 8): the caller then takes the plain kernel."""
     _dev(x, w, bias, resid, out)
@@ -387,12 +387,20 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], re
     lib = library.core()
     bdt = _dt(bias) if bias is not None else 0
     packed = 1 if packed_shape is not None else 0
-    # 17 to 64 rows: the tiled kernel streams the weights of a wide matrix (at least 256 of its
-    # tiles, one per CU) faster than the weight-streaming kernel, whose X fragments then compete
-    # with the weights for loads in flight (measured: gate/up 73 against 85 us at 64 rows, the
-    # head 222 against 296); narrow matrices keep the kernel that can cut K into slices
-    wide = packed and -(-n // (64 if gated else 128)) >= TILED_MIN_TILES
-    if t <= SKINNY_MAX_ROWS and not (t > 16 and wide):
+    # Up to 64 rows: a wide packed matrix (enough 16-row tiles, or gate/up pairs of them, for
+    # STREAM_MIN_BLOCKS blocks of four waves) goes to the kernel whose waves split the output
+    # features and share the rows through LDS; a narrower one to the kernel whose waves split K
+    # and which can cut K over the grid as well.  Measured at Qwen2.5-7B sizes: gate/up at 64
+    # rows 53 us (tiled kernel 74, few-row kernel 85), at 8 rows 48 (few-row kernel 50); the
+    # head at 16 rows 196 (few-row kernel 259).
+    which = _few_rows_kernel[0]
+    if which is None:
+        wave_units = -(-n // 16) if gated else -(-n // 32)
+        which = "stream" if packed and wave_units >= 4 * STREAM_MIN_BLOCKS else "skinny"
+    if t <= SKINNY_MAX_ROWS and which == "stream" and packed:
+        check(lib.sb_gemm_stream_bf16(_p(out), _dt(out), _p(x), _p(w), _p(bias), bdt, _p(resid), t, n, k,
+                                      1 if gated else 0, _stream()))
+    elif t <= SKINNY_MAX_ROWS and which != "tiled":
         need = lib.sb_gemm_skinny_scratch(t, n, k, 1 if gated else 0)
         scratch = torch.empty((need,), dtype=torch.float32, device=x.device) if need else None
         check(lib.sb_gemm_skinny_bf16(_p(out), _dt(out), _p(x), _p(w), _p(bias), bdt, _p(resid), t, n, k,
@@ -415,8 +423,27 @@ def gemm_tile_shape(shape: Optional[int]):
         lib.sb_gemm_mfma_force(-1)
 
 
+@contextlib.contextmanager
+def gemm_few_rows_kernel(which: Optional[str], waves: int = 0):
+    """For tests and measurements: inside the block products of up to 64 rows go to the kernel
+    ``which`` ("stream", "skinny" or "tiled"; "stream" needs packed weights) whatever the sizes,
+    and the stream kernel uses ``waves`` waves per block (4 to 8; 0: its own choice)."""
+    if which not in (None, "stream", "skinny", "tiled"):
+        raise ValueError(f"unknown kernel {which!r}")
+    lib = library.core()
+    before = _few_rows_kernel[0]
+    _few_rows_kernel[0] = which
+    lib.sb_gemm_stream_force(int(waves))
+    try:
+        yield
+    finally:
+        _few_rows_kernel[0] = before
+        lib.sb_gemm_stream_force(0)
+
+
+_few_rows_kernel = [None]
 MFMA_MAX_HEAD_DIM = 256
-TILED_MIN_TILES = 256
+STREAM_MIN_BLOCKS = 192
 TILED_PARTIAL_MIN_ROWS = 17
 
 

@@ -183,19 +183,46 @@ def test_gemm_bf16_every_tile_shape(shape, packed, t, n, k):
         close(got, g / (1.0 + torch.exp(-g)) * u, atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"gated shape {shape}")
 
 
-@pytest.mark.parametrize("t", [17, 40, 64])
+@pytest.mark.parametrize("t", [1, 16, 17, 40, 64])
+@pytest.mark.parametrize("waves", [0, 4, 5, 6, 7, 8])
+@pytest.mark.parametrize("n, k", [(100, 96), (1000, 520), (264, 2368), (4099, 264)])
+def test_gemm_bf16_stream_kernel(t, waves, n, k):
+    """The kernel for few rows against wide matrices, at every count of waves per block: K
+    shorter than one staged chunk, ending inside a chunk and inside a k-step; columns that end
+    inside a tile and inside a block; plain with bias and residual, and gated."""
+    from sonicboom_amd import ops
+    x, w = randn(t, k, dtype=BF16), randn(n, k, dtype=BF16, scale=0.05)
+    bias, resid = randn(n, scale=0.1), randn(t, n)
+    wd = w.to(DEV)
+    with ops.gemm_few_rows_kernel("stream", waves):
+        got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(wd), bias.to(DEV), resid.to(DEV), F32, packed_shape=(n, k))
+        close(got, ref_gemm(x, w, bias, resid), atol=3e-5 * math.sqrt(k), rtol=1e-5, what="stream")
+        got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(wd), None, None, BF16, packed_shape=(n, k))
+        close(got.float(), ref_gemm(x, w), atol=2e-2, rtol=1e-2, what="stream, bfloat16 out")
+        inner = n // 2
+        wg = wd[:2 * inner].contiguous()
+        gu = x.double() @ w[:2 * inner].double().T
+        g, u = gu[:, :inner], gu[:, inner:]
+        got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(wg, True), None, None, F32, gated=True,
+                            packed_shape=(2 * inner, k))
+        close(got, g / (1.0 + torch.exp(-g)) * u, atol=1e-4 * math.sqrt(k), rtol=1e-4, what="stream, gated")
+
+
+@pytest.mark.parametrize("t", [8, 17, 64])
 def test_gemm_bf16_wide_matrix_with_few_rows(t):
-    """17 to 64 rows against a matrix of 256 tiles or more go to the tiled kernel (packed
-    weights), plain and gated; one tile less stays with the weight-streaming kernel."""
+    """Up to 64 rows against a packed matrix wide enough for the stream kernel, and one wave's
+    worth of columns less (which stays with the kernel that splits K), plain and gated: the
+    choice between the kernels changes no result."""
     from sonicboom_amd import ops
     from sonicboom_amd.ops import kernels
     k = 64
     x = randn(t, k, dtype=BF16)
-    for n in (kernels.TILED_MIN_TILES * 128, kernels.TILED_MIN_TILES * 128 - 128):
+    edge = 4 * kernels.STREAM_MIN_BLOCKS
+    for n in (edge * 32, edge * 32 - 32):
         w = randn(n, k, dtype=BF16, scale=0.05)
         got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(w.to(DEV)), None, None, F32, packed_shape=(n, k))
         close(got, ref_gemm(x, w), atol=3e-5 * math.sqrt(k), rtol=1e-5, what=f"wide n={n}")
-    for inner in (kernels.TILED_MIN_TILES * 64, kernels.TILED_MIN_TILES * 64 - 64):   # gated tiles hold 64 outputs
+    for inner in (edge * 16, edge * 16 - 16):
         w = randn(2 * inner, k, dtype=BF16, scale=0.05)
         gu = x.double() @ w.double().T
         g, u = gu[:, :inner], gu[:, inner:]
