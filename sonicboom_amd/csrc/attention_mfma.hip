@@ -118,11 +118,39 @@ __device__ __forceinline__ void load_half(HalfPage &hp, const bf16_t *__restrict
   for (int dt = 0; dt < DT; ++dt) hp.v[dt] = ld16(vp + size_t(dt * 16 + r) * SB_PAGE + 32 * half + 8 * g, true);
 }
 
+// The same without a branch around any load (a branch makes the compiler wait for every load in
+// flight, which a loop that keeps the next half page's loads in flight cannot afford): a chunk
+// past the head size is read from the row's start and replaced by zeros afterwards.
+__device__ __forceinline__ void load_half_straight(HalfPage &hp, const bf16_t *__restrict__ kp,
+                                                   const bf16_t *__restrict__ vp, int half, int lane) {
+  const int r = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int key = 32 * half + 8 * (r >> 2) + 4 * t + (r & 3);
+    const bf16_t *krow = kp + size_t(key) * HD;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 32 + g * 8;
+      if ((ks + 1) * 32 <= HD) {
+        hp.k[t][ks] = *reinterpret_cast<const uint4 *>(krow + d);
+      } else {
+        const uint4 v = *reinterpret_cast<const uint4 *>(krow + (d < HD ? d : 0));
+        hp.k[t][ks] = d < HD ? v : make_uint4(0u, 0u, 0u, 0u);
+      }
+    }
+  }
+#pragma unroll
+  for (int dt = 0; dt < DT; ++dt)
+    hp.v[dt] = *reinterpret_cast<const uint4 *>(vp + size_t(dt * 16 + r) * SB_PAGE + 32 * half + 8 * g);
+}
+
 // 32 keys at absolute positions base .. base+31, their fragments in hp, for the wave's NC groups
 // of 16 columns.  col_pos / col_lo: last and first visible key of this lane's column (col_pos < 0:
 // the column is empty); the groups share them.  key_hi / key_lo: the same over all columns of the
 // wave (uniform).
-template <int NC>
+// MASKED = false: every key of the 32 is visible from every column (and so written): no score is
+// tested and no value cut.
+template <int NC, bool MASKED = true>
 __device__ __forceinline__ void attend_half(WaveState<NC> &st, const bf16x8_t (&qf)[NC][KS], const HalfPage &hp,
                                             int base, int col_pos, int col_lo, int key_lo, int key_hi,
                                             float scale_log2, int lane) {
@@ -130,7 +158,7 @@ __device__ __forceinline__ void attend_half(WaveState<NC> &st, const bf16x8_t (&
   const int k0 = base + 8 * g;
   // values of keys outside [key_lo, key_hi] may be stale or never written: 0 * garbage must not
   // reach the accumulator, so such keys are cut out of the V fragments
-  const bool cut_hi = base + 31 > key_hi, cut_lo = base < key_lo;
+  const bool cut_hi = MASKED && base + 31 > key_hi, cut_lo = MASKED && base < key_lo;
   uint4 vf[DT];
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt) {
@@ -154,7 +182,7 @@ __device__ __forceinline__ void attend_half(WaveState<NC> &st, const bf16x8_t (&
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const int j = k0 + e;
-      const bool vis = j <= col_pos && j >= col_lo;
+      const bool vis = !MASKED || (j <= col_pos && j >= col_lo);
       const float v = (e < 4 ? s[0][e] : s[1][e - 4]) * scale_log2;
       sc[e] = vis ? v : -__builtin_inff();
       mx = fmaxf(mx, sc[e]);
@@ -586,46 +614,34 @@ __device__ __forceinline__ void merge_element(bf16_t *__restrict__ out, const fl
   out[(size_t(seq) * heads_q + kvh * group + hh) * HD + d] = f32_to_bf16(l > 0.f ? o / l : 0.f);
 }
 
-template <bool BOTH>
-__global__ void __launch_bounds__(256)
-attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
-                   const bf16_t *__restrict__ q,
-                   const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
-                   const int32_t *__restrict__ page_table, int max_pages, int n_pages_total,
-                   const int32_t *__restrict__ row_pos, int heads_q, int heads_kv, int n_chunks,
-                   float scale_log2, int window) {
-  __shared__ float lds_o[4][HD * 16];   // [wave][d][col]
-  __shared__ float lds_m[4][16], lds_l[4][16];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int chunk = blockIdx.x, seq = blockIdx.z;
-  const int group = heads_q / heads_kv;
-  const int head_tiles = (group + 15) / 16;
-  const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y - kvh * head_tiles;
-  // the wave's page number does not depend on the position: both look-ups go out together
-  const int pg = chunk * kPagesPerChunk + wave;
-  const int page_looked_up = page_table[size_t(seq) * max_pages + min(pg, max_pages - 1)];
-  const int pos = row_pos[seq];
-  const int key_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
-  const int first_chunk = key_lo / (SB_PAGE * kPagesPerChunk);
-  const int last_chunk = min(pos / (SB_PAGE * kPagesPerChunk), n_chunks - 1);
-  if (chunk < first_chunk || chunk > last_chunk) return;   // uniform over the block
+// Decode grids have one dimension, the block number counting the (kv head x head tile) fastest,
+// then the sequence, the chunk of pages slowest.  Blocks go to the GPU's eight dies in turn by
+// their number; which chunks have work depends on the sequences' lengths, and with the chunk as
+// the fastest dimension the chunks past a row's end would leave whole dies idle (nine busy chunks
+// of sixteen put two ninths of the work on one die).
+struct DecodeBlock {
+  int chunk, seq, tile;   // tile = kv head * head tiles + head tile
+};
+__device__ __forceinline__ DecodeBlock decode_block(int tiles, int n_seqs) {
+  const int per_chunk = tiles * n_seqs;
+  DecodeBlock b;
+  b.chunk = int(blockIdx.x) / per_chunk;
+  const int rem = int(blockIdx.x) - b.chunk * per_chunk;
+  b.seq = rem / tiles;
+  b.tile = rem - b.seq * tiles;
+  return b;
+}
 
+// The end of a decode block: the waves' running sums meet in LDS and are merged in wave order
+// (thread e owns (d, column), column fastest); the result goes to `out` when the row's keys lie
+// in this chunk alone, else to the chunk's place in the partial buffers.
+__device__ __forceinline__ void finish_decode_block(const WaveState<1> &st, float (*lds_o)[HD * 16], float (*lds_m)[16],
+                                                    float (*lds_l)[16], bf16_t *__restrict__ out,
+                                                    float *__restrict__ part_o, float *__restrict__ part_ml,
+                                                    int wave, int lane, int chunk, bool alone, int seq, int kvh,
+                                                    int ht, int group, int heads_q, int n_chunks,
+                                                    size_t tile_index) {
   const int r = lane & 15, g = lane >> 4;
-  const int hq = ht * 16 + r;                 // query head within the group
-  const bool col_ok = hq < group;
-  const int head = kvh * group + (col_ok ? hq : 0);
-  bf16x8_t qf[1][KS];
-  load_q(qf[0], q + (size_t(seq) * heads_q + head) * HD, col_ok, lane);
-  WaveState<1> st;
-  init_state<1>(st);
-  if (pg >= key_lo / SB_PAGE && pg <= pos / SB_PAGE && pg < max_pages) {
-    const int page = page_looked_up;
-    if (page >= 0 && page < n_pages_total) {
-      const size_t off = (size_t(page) * heads_kv + kvh) * SB_PAGE * HD;
-      attend_page<1, BOTH>(st, qf, k_cache + off, v_cache + off, pg * SB_PAGE, col_ok ? pos : -1, key_lo, key_lo,
-                           pos, scale_log2, lane);
-    }
-  }
   float l = st.l[0];
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
@@ -639,8 +655,6 @@ attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *
   }
   __syncthreads();
   // merge the four waves (pages in ascending order); thread e owns (d, col), column fastest
-  const bool alone = first_chunk == last_chunk;
-  const size_t tile_index = size_t(seq) * gridDim.y + blockIdx.y;
   float *po = part_o + (tile_index * n_chunks) * (HD * 16);
   float *pml = part_ml + (tile_index * n_chunks) * 32;
   for (int e = threadIdx.x; e < HD * 16; e += 256) {
@@ -670,19 +684,150 @@ attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *
   }
 }
 
+template <bool BOTH>
+__global__ void __launch_bounds__(256)
+attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
+                   const bf16_t *__restrict__ q,
+                   const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
+                   const int32_t *__restrict__ page_table, int max_pages, int n_pages_total,
+                   const int32_t *__restrict__ row_pos, int heads_q, int heads_kv, int n_chunks,
+                   float scale_log2, int window, int n_seqs) {
+  __shared__ float lds_o[4][HD * 16];   // [wave][d][col]
+  __shared__ float lds_m[4][16], lds_l[4][16];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int group = heads_q / heads_kv;
+  const int head_tiles = (group + 15) / 16;
+  const int tiles = heads_kv * head_tiles;
+  const DecodeBlock blk = decode_block(tiles, n_seqs);
+  const int chunk = blk.chunk, seq = blk.seq;
+  const int kvh = blk.tile / head_tiles, ht = blk.tile - kvh * head_tiles;
+  // the wave's page number does not depend on the position: both look-ups go out together
+  const int pg = chunk * kPagesPerChunk + wave;
+  const int page_looked_up = page_table[size_t(seq) * max_pages + min(pg, max_pages - 1)];
+  const int pos = row_pos[seq];
+  const int key_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
+  const int first_chunk = key_lo / (SB_PAGE * kPagesPerChunk);
+  const int last_chunk = min(pos / (SB_PAGE * kPagesPerChunk), n_chunks - 1);
+  if (chunk < first_chunk || chunk > last_chunk) return;   // uniform over the block
+
+  const int r = lane & 15, g = lane >> 4;
+  const int hq = ht * 16 + r;                 // query head within the group
+  const bool col_ok = hq < group;
+  const int head = kvh * group + (col_ok ? hq : 0);
+  bf16x8_t qf[1][KS];
+  load_q(qf[0], q + (size_t(seq) * heads_q + head) * HD, col_ok, lane);
+  WaveState<1> st;
+  init_state<1>(st);
+  if (pg >= key_lo / SB_PAGE && pg <= pos / SB_PAGE && pg < max_pages) {
+    const int page = page_looked_up;
+    if (page >= 0 && page < n_pages_total) {
+      const size_t off = (size_t(page) * heads_kv + kvh) * SB_PAGE * HD;
+      attend_page<1, BOTH>(st, qf, k_cache + off, v_cache + off, pg * SB_PAGE, col_ok ? pos : -1, key_lo, key_lo,
+                           pos, scale_log2, lane);
+    }
+  }
+  finish_decode_block(st, lds_o, lds_m, lds_l, out, part_o, part_ml, wave, lane, chunk, first_chunk == last_chunk,
+                      seq, kvh, ht, group, heads_q, n_chunks, size_t(seq) * tiles + blk.tile);
+}
+
+// Decode with many more blocks than the GPU holds at once (long contexts, large batches): a wave
+// takes `ppw` consecutive pages instead of one and keeps the next half page's keys and values in
+// flight while it multiplies the current one, so that a block lives long enough to stream and the
+// fixed costs of a block (look-ups, queries, the merge through LDS, the partial results) are paid
+// once per 4 * ppw pages.  Block (chunk of 4 * ppw pages, kv head x head tile, sequence); wave w
+// takes pages chunk * 4 * ppw + w * ppw + 0 .. ppw-1.  Head sizes up to 128.
+__global__ void __launch_bounds__(256, 2)
+attn_decode_long_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
+                        const bf16_t *__restrict__ q,
+                        const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
+                        const int32_t *__restrict__ page_table, int max_pages, int n_pages_total,
+                        const int32_t *__restrict__ row_pos, int heads_q, int heads_kv, int n_chunks,
+                        float scale_log2, int window, int ppw, int n_seqs) {
+  __shared__ float lds_o[4][HD * 16];   // [wave][d][col]
+  __shared__ float lds_m[4][16], lds_l[4][16];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int group = heads_q / heads_kv;
+  const int head_tiles = (group + 15) / 16;
+  const int tiles = heads_kv * head_tiles;
+  const DecodeBlock blk = decode_block(tiles, n_seqs);
+  const int chunk = blk.chunk, seq = blk.seq;
+  const int kvh = blk.tile / head_tiles, ht = blk.tile - kvh * head_tiles;
+  const int pages_per_chunk = kPagesPerChunk * ppw;
+  const int pos = row_pos[seq];
+  const int key_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
+  const int first_chunk = key_lo / (SB_PAGE * pages_per_chunk);
+  const int last_chunk = min(pos / (SB_PAGE * pages_per_chunk), n_chunks - 1);
+  if (chunk < first_chunk || chunk > last_chunk) return;   // uniform over the block
+
+  const int r = lane & 15;
+  const int hq = ht * 16 + r;                 // query head within the group
+  const bool col_ok = hq < group;
+  const int head = kvh * group + (col_ok ? hq : 0);
+  bf16x8_t qf[1][KS];
+  load_q(qf[0], q + (size_t(seq) * heads_q + head) * HD, col_ok, lane);
+  WaveState<1> st;
+  init_state<1>(st);
+
+  const int32_t *pt = page_table + size_t(seq) * max_pages;
+  const int pg_begin = max(chunk * pages_per_chunk + wave * ppw, key_lo / SB_PAGE);
+  const int pg_end = min(min(chunk * pages_per_chunk + (wave + 1) * ppw, pos / SB_PAGE + 1), max_pages);
+  const size_t page_elems = size_t(heads_kv) * SB_PAGE * HD;
+  const size_t head_off = size_t(kvh) * SB_PAGE * HD;
+  // a page number outside the cache: read page 0 and see none of its keys
+  auto page_of = [&](int pg, bool &ok) {
+    const int page = pt[pg];
+    ok = page >= 0 && page < n_pages_total;
+    return size_t(ok ? page : 0) * page_elems + head_off;
+  };
+  if (pg_begin < pg_end) {
+    HalfPage h0, h1;
+    // 32 keys from `base` on: all visible and written (the common case), or tested one by one
+    auto attend = [&](const HalfPage &h, int base, bool ok) {
+      if (ok && base >= key_lo && base + 31 <= pos) {
+        attend_half<1, false>(st, qf, h, base, pos, key_lo, key_lo, pos, scale_log2, lane);
+      } else {
+        // hi < lo for a page that is not there: every value is cut, no key seen
+        attend_half<1, true>(st, qf, h, base, (ok && col_ok) ? pos : -1, key_lo, key_lo, ok ? pos : -1, scale_log2,
+                             lane);
+      }
+    };
+    bool ok;
+    size_t off = page_of(pg_begin, ok);
+    load_half_straight(h0, k_cache + off, v_cache + off, 0, lane);
+    int pg = pg_begin;
+    // every page but the last: the loads of the next half page go out before this half's
+    // products, with no branch between a load and its use
+    for (; pg + 1 < pg_end; ++pg) {
+      load_half_straight(h1, k_cache + off, v_cache + off, 1, lane);
+      attend(h0, pg * SB_PAGE, ok);
+      bool ok_next;
+      off = page_of(pg + 1, ok_next);
+      load_half_straight(h0, k_cache + off, v_cache + off, 0, lane);
+      attend(h1, pg * SB_PAGE + 32, ok);
+      ok = ok_next;
+    }
+    load_half_straight(h1, k_cache + off, v_cache + off, 1, lane);
+    attend(h0, pg * SB_PAGE, ok);
+    attend(h1, pg * SB_PAGE + 32, ok);
+  }
+  finish_decode_block(st, lds_o, lds_m, lds_l, out, part_o, part_ml, wave, lane, chunk, first_chunk == last_chunk,
+                      seq, kvh, ht, group, heads_q, n_chunks, size_t(seq) * tiles + blk.tile);
+}
+
 // Merge the chunks of a (sequence, tile) in ascending order: one thread per (d, column).
 // Grid (HD * 16 / 256, tiles, sequences).
 __global__ void __launch_bounds__(256)
 attn_decode_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o,
                          const float *__restrict__ part_ml, const int32_t *__restrict__ row_pos,
-                         int heads_q, int heads_kv, int n_chunks, int window) {
+                         int heads_q, int heads_kv, int n_chunks, int window, int pages_per_chunk) {
   const int seq = blockIdx.z;
   const int group = heads_q / heads_kv;
   const int head_tiles = (group + 15) / 16;
   const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y - kvh * head_tiles;
   const int pos = row_pos[seq];
   const int key_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
-  const int first = key_lo / (SB_PAGE * kPagesPerChunk), last = min(pos / (SB_PAGE * kPagesPerChunk), n_chunks - 1);
+  const int first = key_lo / (SB_PAGE * pages_per_chunk), last = min(pos / (SB_PAGE * pages_per_chunk), n_chunks - 1);
   if (first == last) return;      // the decode kernel has written the result itself
   const int e = blockIdx.x * 256 + threadIdx.x;
   if (e >= HD * 16) return;
@@ -691,7 +836,7 @@ attn_decode_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ par
                 first, last, seq, heads_q, kvh, ht, group);
 }
 
-int g_force_nc = 0, g_force_waves = 0;
+int g_force_nc = 0, g_force_waves = 0, g_force_ppw = 0;
 
 int check_common(const void *out, const void *q, const void *k, const void *v, const void *pt,
                  const void *row_pos, int max_pages, int n_pages_total, int heads_q, int heads_kv,
@@ -738,34 +883,51 @@ extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache
   SB_REQUIRE(n_seqs >= 0, "sb_attn_decode_bf16: bad batch");
   SB_SUPPORT(n_seqs <= 65535, "sb_attn_decode_bf16: more than 65535 sequences in a step");
   if (n_seqs == 0) return SB_OK;
-  const int n_chunks = sb_attn_decode_chunks(max_pages);
-  SB_REQUIRE(n_chunks == 1 || (part_o && part_ml), "sb_attn_decode_bf16: no buffers for the partial results");
+  const int chunks_1 = sb_attn_decode_chunks(max_pages);      // what the partial buffers are sized for
+  SB_REQUIRE(chunks_1 == 1 || (part_o && part_ml), "sb_attn_decode_bf16: no buffers for the partial results");
   const int group = heads_q / heads_kv;
   const int head_tiles = (group + 15) / 16;
   hipStream_t s = (hipStream_t)stream;
-  dim3 grid(n_chunks, heads_kv * head_tiles, n_seqs);
   SB_SUPPORT(heads_kv * head_tiles <= 65535, "sb_attn_decode_bf16: too many heads");
-  // Few blocks: a wave asks for its whole page at once (one round trip to memory).  Many more
-  // blocks than the GPU holds at once: half a page at a time, which takes fewer registers and
-  // lets three blocks share a CU instead of two (measured at 2,048 keys: 65 against 69 us at 64
-  // sequences, no gain at 32).
-  const long long n_blocks = (long long)n_chunks * heads_kv * head_tiles * n_seqs;
-  if (n_blocks <= 1536)
+  // A wave takes one page and asks for all of it at once (one round trip to memory), or, when
+  // that still leaves a block for every CU, 2, 4 or 8 pages in a row with half a page in flight
+  // while the half before it is multiplied (measured on cold caches, Qwen2.5-7B heads: 64
+  // sequences of 2,060 keys 65 us with eight pages per wave against 82 with one; 8 sequences of
+  // 16,400 keys 57 against 79; one sequence of 32,780 keys 33 against 43).
+  const long long per_chunk = (long long)heads_kv * head_tiles * n_seqs;
+  int ppw = 1;
+  if (HD <= 128)
+    for (int c = 8; c >= 2 && ppw == 1; c /= 2)
+      if ((long long)((max_pages + 4 * c - 1) / (4 * c)) * per_chunk >= 256) ppw = c;
+  if (g_force_ppw > 0 && (g_force_ppw == 1 || HD <= 128)) ppw = g_force_ppw;
+  const int pages_per_chunk = kPagesPerChunk * ppw;
+  const int n_chunks = (max_pages + pages_per_chunk - 1) / pages_per_chunk;
+  SB_SUPPORT((long long)n_chunks * per_chunk <= 0x7fffffffLL, "sb_attn_decode_bf16: too many blocks");
+  const unsigned grid = unsigned((long long)n_chunks * per_chunk);
+  if (ppw > 1)
+    attn_decode_long_kernel<<<grid, 256, 0, s>>>((bf16_t *)out, part_o, part_ml, (const bf16_t *)q,
+                                                 (const bf16_t *)k_cache, (const bf16_t *)v_cache, page_table,
+                                                 max_pages, n_pages_total, row_pos, heads_q, heads_kv, n_chunks,
+                                                 scale * kLog2e, window, ppw, n_seqs);
+  else if ((long long)n_chunks * per_chunk <= 1536)
     attn_decode_kernel<true><<<grid, 256, 0, s>>>((bf16_t *)out, part_o, part_ml, (const bf16_t *)q,
                                                   (const bf16_t *)k_cache, (const bf16_t *)v_cache, page_table,
                                                   max_pages, n_pages_total, row_pos, heads_q, heads_kv,
-                                                  n_chunks, scale * kLog2e, window);
+                                                  n_chunks, scale * kLog2e, window, n_seqs);
   else
     attn_decode_kernel<false><<<grid, 256, 0, s>>>((bf16_t *)out, part_o, part_ml, (const bf16_t *)q,
                                                    (const bf16_t *)k_cache, (const bf16_t *)v_cache, page_table,
                                                    max_pages, n_pages_total, row_pos, heads_q, heads_kv,
-                                                   n_chunks, scale * kLog2e, window);
+                                                   n_chunks, scale * kLog2e, window, n_seqs);
   rc = sb::check_launch("sb_attn_decode_bf16");
   if (rc != SB_OK || n_chunks == 1) return rc;
   attn_decode_merge_kernel<<<dim3((HD * 16 + 255) / 256, heads_kv * head_tiles, n_seqs), 256, 0, s>>>(
-      (bf16_t *)out, part_o, part_ml, row_pos, heads_q, heads_kv, n_chunks, window);
+      (bf16_t *)out, part_o, part_ml, row_pos, heads_q, heads_kv, n_chunks, window, pages_per_chunk);
   return sb::check_launch("sb_attn_decode_bf16 (merge)");
 }
+
+// Measurement hook: pages per wave of the decode kernel (1, 2, 4, 8; 0: chosen from the sizes).
+extern "C" void sb_attn_decode_force(int ppw) { g_force_ppw = (ppw == 1 || ppw == 2 || ppw == 4 || ppw == 8) ? ppw : 0; }
 
 // Measurement hook: heads per wave and waves per block in prefill (0: chosen from the group size).
 extern "C" void sb_attn_prefill_force(int nc, int waves) { g_force_nc = nc; g_force_waves = waves; }

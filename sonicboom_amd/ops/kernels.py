@@ -480,6 +480,20 @@ def attention_decode_mfma(q, k_cache, v_cache, page_table, seq_pos, heads_q, hea
     return out
 
 
+@contextlib.contextmanager
+def attention_decode_pages_per_wave(head_dim: int, pages: int):
+    """For tests and measurements: inside the block the decode attention kernel of this head size
+    gives every wave ``pages`` pages (1, 2, 4 or 8; more than one only up to head size 128)
+    instead of choosing from the sizes."""
+    lib = library.attention_library(head_dim)
+    lib.sb_attn_decode_force.restype = None
+    lib.sb_attn_decode_force(int(pages))
+    try:
+        yield
+    finally:
+        lib.sb_attn_decode_force(0)
+
+
 def attention_prefill_mfma(q, k_cache, v_cache, page_table, row_pos, tiles, heads_q, heads_kv, head_dim, scale,
                            window):
     """bf16 query rows over the cache; ``tiles`` int32 [n, 4] = (first row, rows <= 16, sequence, 0)

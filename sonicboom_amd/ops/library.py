@@ -54,6 +54,7 @@ _ATTN_SIGNATURES = {
     # heads_kv, scale, window, stream
     "sb_attn_prefill_bf16": [_P, _P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _F, _I, _P],
     "sb_attn_decode_chunks": [_I],
+    "sb_attn_decode_force": [_I],
     "sb_attn_head_dim": [],
 }
 

@@ -471,8 +471,7 @@ def test_attention_decode_matrix_cores(hq, hkv, hd, window):
 
 
 def test_attention_decode_matrix_cores_many_sequences():
-    """Two hundred sequences: more blocks than the GPU holds at once, which takes the kernel
-    that reads half a page at a time."""
+    """Two hundred sequences: enough blocks for the kernel whose waves take several pages."""
     from sonicboom_amd import ops
     hq, hkv, hd = 8, 4, 32
     rng = np.random.default_rng(5)
@@ -481,6 +480,28 @@ def test_attention_decode_matrix_cores_many_sequences():
     pos = torch.tensor([p for _, p in rows], dtype=torch.int32)
     got = ops.attention_decode_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), hq, hkv, hd, scale, 0)
     close(got, want, atol=1.5e-2, rtol=1e-2, what="decode, 200 sequences")
+
+
+@pytest.mark.parametrize("hq, hkv, hd", [(4, 2, 16), (5, 5, 48), (6, 2, 80), (28, 4, 128), (40, 2, 64)])
+@pytest.mark.parametrize("window", [0, 70, 1000])
+@pytest.mark.parametrize("pages", [1, 2, 4, 8])
+def test_attention_decode_pages_per_wave(hq, hkv, hd, window, pages):
+    """Every way of dealing pages to waves (one page each, or 2, 4, 8 in a row with the next half
+    page in flight), on lengths around page, wave and chunk edges, a long row, a window that
+    starts inside a later chunk, and a table with a hole: a page number outside the cache in a
+    page that the window has left behind."""
+    from sonicboom_amd import ops
+    lens = [1, 64, 65, 129, 256, 257, 513, 700, 2100]
+    q, kc, vc, table, rows, scale, want = attention_case(hq, hkv, hd, lens, [[n - 1] for n in lens], window, seed=4)
+    pos = torch.tensor([p for _, p in rows], dtype=torch.int32)
+    if window:
+        table[-1, 0] = -1                     # the cache gives such pages back
+        table[-1, 1] = kc.shape[0] + 5
+    with ops.attention_decode_pages_per_wave(hd, pages):
+        got = ops.attention_decode_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), hq, hkv, hd, scale, window)
+        close(got, want, atol=1.5e-2, rtol=1e-2, what=f"decode, {pages} pages per wave")
+        again = ops.attention_decode_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), hq, hkv, hd, scale, window)
+        assert torch.equal(got, again)
 
 
 @pytest.mark.parametrize("hq, hkv, hd", MFMA_SHAPES)
