@@ -70,12 +70,13 @@ gemm_mfma_kernel(Args a) {
   bf16x8_t *lds_a0 = lds, *lds_a1 = lds + BM * CPR;
   bf16x8_t *lds_b0 = lds + 2 * BM * CPR, *lds_b1 = lds_b0 + BN * CPR;
 
-  // XCD-aware order: hardware sends block b to XCD b % 8.  When the count divides, XCD x
-  // gets the contiguous run of tiles [x * per, (x + 1) * per), which share rows of X and W in
-  // that XCD's L2.
+  // XCD-aware order: hardware sends block b to XCD b % 8.  XCD x gets the contiguous run of
+  // tiles [x * per, (x + 1) * per), which share rows of X and W in that XCD's L2; the grid is
+  // padded to a multiple of eight blocks, and the blocks past the last tile leave at once.
   const int n_blocks = a.tiles_m * a.tiles_n;
-  int bid = blockIdx.x;
-  if (n_blocks % kXcds == 0) bid = (bid % kXcds) * (n_blocks / kXcds) + bid / kXcds;
+  const int per_xcd = (n_blocks + kXcds - 1) / kXcds;
+  const int bid = (int(blockIdx.x) % kXcds) * per_xcd + int(blockIdx.x) / kXcds;
+  if (bid >= n_blocks) return;
   // tiles of one column of N (same W rows) are neighbours: m runs fastest
   const int tn = bid / a.tiles_m, tm = bid - tn * a.tiles_m;
   const int t0 = tm * BM;
@@ -332,7 +333,7 @@ int launch_one(const Args &a, long long blocks, hipStream_t s) {
   const int n_k = (a.n_in + BK - 1) / BK;
   const unsigned slices = a.partial ? unsigned((n_k + a.stages_per_slice - 1) / a.stages_per_slice) : 1u;
   gemm_mfma_kernel<MT, NW, BK, DEPTH, GATED, PACKED, EVEN_K>
-      <<<dim3(unsigned(blocks), slices), 128 * NW, lds_bytes, s>>>(a);
+      <<<dim3(unsigned((blocks + kXcds - 1) / kXcds * kXcds), slices), 128 * NW, lds_bytes, s>>>(a);
   return SB_OK;
 }
 
