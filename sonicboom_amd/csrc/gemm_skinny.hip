@@ -42,7 +42,7 @@ __device__ __forceinline__ void store_out(const Epilogue &e, int t, int n, float
 }
 
 // G = 1: plain.  G = 2: rows n and n_out + n of W are gate and up of output n.
-// PACKED: W is stored tile by tile in MFMA fragment order (see sb_hip.h, "packed weights"): the
+// PACKED: W is stored tile by tile in MFMA fragment order (ops.pack_weight lays it out): the
 // fragment of row tile nb and k-step ks is the 1 KB block (nb * n_steps + ks), lane l's eight
 // elements at l * 8; rows and k are padded with zeros to whole tiles.
 template <int R, int TT, int G, bool PACKED>
@@ -274,7 +274,7 @@ extern "C" size_t sb_gemm_skinny_scratch(int n_rows, int n_out, int n_in, int ga
 
 // Y = X W^T (+bias) (+resid), or with gated != 0: Y = silu(X Wg^T) * (X Wu^T) where W = [Wg; Wu]
 // is [2*n_out, n_in].  X [n_rows, n_in] and W are bf16; n_rows <= 64; n_in a multiple of 8.
-// packed != 0: W is in the packed tile layout (sb_pack_weight_bf16).
+// packed != 0: W is in the packed tile layout.
 extern "C" int sb_gemm_skinny_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,
                                    int bias_dtype, const float *resid, int n_rows, int n_out, int n_in,
                                    int gated, int packed, float *scratch, size_t scratch_floats,
