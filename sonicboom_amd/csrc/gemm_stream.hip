@@ -37,6 +37,11 @@ struct StreamArgs {
   int bias_dtype;
   const float *resid;
   int n_rows, n_out, n_in;
+  // K cut over the grid (blockIdx.y): slice s multiplies k-steps [s * steps_per_slice, ...), a
+  // multiple of eight of them, and writes its raw sums to partial [slice][n_rows][n_out]; NULL:
+  // one slice and the epilogues below
+  float *partial;
+  int steps_per_slice;
 };
 
 __device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
@@ -58,6 +63,8 @@ gemm_stream_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ w, S
   const int n_steps = (a.n_in + kStepK - 1) / kStepK;
   const int tiles_out = (a.n_out + 15) / 16;
   const int tile0 = (blockIdx.x * W + wave) * R;
+  const int s0 = a.partial ? int(blockIdx.y) * a.steps_per_slice : 0;
+  const int s1 = a.partial ? min(s0 + a.steps_per_slice, n_steps) : n_steps;
 
   floatx4_t acc[F][TT];
 #pragma unroll
@@ -68,7 +75,7 @@ gemm_stream_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ w, S
   // Every load goes through a buffer descriptor, so that what lies outside (a tile past the
   // last, a k-step past the end, a row past the last) reads as zero without a branch: a branch
   // around a load makes the compiler wait for every load in flight.
-  // W: one descriptor per fragment stream (tile, half): n_steps blocks of 1 KB.
+  // W: one descriptor per fragment stream (tile, half): blocks of 1 KB up to this slice's end.
   __amdgpu_buffer_rsrc_t rsrc_w[F];
 #pragma unroll
   for (int g = 0; g < G; ++g)
@@ -77,7 +84,7 @@ gemm_stream_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ w, S
       const int tile = tile0 + i;
       const bf16_t *base = w + (size_t(g * tiles_out + min(tile, tiles_out - 1)) * n_steps) * 512;
       rsrc_w[g * R + i] = __builtin_amdgcn_make_buffer_rsrc(
-          const_cast<bf16_t *>(base), 0, tile < tiles_out ? uint32_t(n_steps) * 1024u : 0u, 0x00020000);
+          const_cast<bf16_t *>(base), 0, tile < tiles_out ? uint32_t(s1) * 1024u : 0u, 0x00020000);
     }
   const __amdgpu_buffer_rsrc_t rsrc_x = __builtin_amdgcn_make_buffer_rsrc(
       const_cast<bf16_t *>(x), 0, uint32_t(size_t(a.n_rows) * a.n_in * 2), 0x00020000);
@@ -95,7 +102,9 @@ gemm_stream_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ w, S
   }
   constexpr uint32_t kOutside = 0x80000000u;
   uint4 xs[kXLoads];
-  auto issue_x = [&](int chunk) {
+  const int chunk0 = s0 / kAhead;              // slices start on whole chunks
+  auto issue_x = [&](int c) {
+    const int chunk = chunk0 + c;
 #pragma unroll
     for (int i = 0; i < kXLoads; ++i) {
       const uint32_t off = chunk * kChunkK + x_k[i] < a.n_in ? x_off[i] + uint32_t(chunk) * (kChunkK * 2) : kOutside;
@@ -109,7 +118,7 @@ gemm_stream_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ w, S
   };
 
   uint4 ring[kAhead][F];
-  uint32_t w_off = uint32_t(lane) * 16u;       // of the next k-step to ask for
+  uint32_t w_off = uint32_t(lane) * 16u + uint32_t(s0) * 1024u;   // of the next k-step to ask for
 #pragma unroll
   for (int u = 0; u < kAhead; ++u) {
 #pragma unroll
@@ -121,7 +130,7 @@ gemm_stream_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ w, S
   store_x(0);
   __syncthreads();
 
-  const int n_chunks = (n_steps + kAhead - 1) / kAhead;
+  const int n_chunks = (s1 - s0 + kAhead - 1) / kAhead;
   for (int c = 0; c < n_chunks; ++c) {
     const bool more = c + 1 < n_chunks;
     if (more) issue_x(c + 1);
@@ -152,6 +161,13 @@ gemm_stream_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ w, S
       const int t = j * 16 + r;
       if (t >= a.n_rows) continue;
       const size_t row_off = size_t(t) * a.n_out;
+      if (G == 1 && a.partial) {
+        float *dst = a.partial + size_t(blockIdx.y) * a.n_rows * a.n_out + row_off;
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (nb + e < a.n_out) dst[nb + e] = acc[i][j][e];
+        continue;
+      }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int n = nb + e;
@@ -178,7 +194,9 @@ void launch_w(const bf16_t *x, const bf16_t *w, const StreamArgs &a, hipStream_t
     (void)hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, int(lds));
     raised = true;
   }
-  kern<<<(tiles + per_block - 1) / per_block, 64 * W, lds, s>>>(x, w, a);
+  const int n_steps = (a.n_in + kStepK - 1) / kStepK;
+  const unsigned slices = a.partial ? unsigned((n_steps + a.steps_per_slice - 1) / a.steps_per_slice) : 1u;
+  kern<<<dim3((tiles + per_block - 1) / per_block, slices), 64 * W, lds, s>>>(x, w, a);
 }
 
 int g_force_waves = 0;   // measurement hook, see sb_gemm_stream_force
@@ -197,6 +215,45 @@ int waves_for(int tiles, int r) {
   return best;
 }
 
+// K cut over the grid for narrow matrices: waves per block and slices such that the blocks fill
+// whole rounds over the CUs, every slice a whole number of staged chunks.  The cost of a choice:
+// rounds x a block's k-steps (plus what a block costs before it streams) x the bytes a step
+// moves (1 KB of W per wave from memory, 1 KB of X per 16 rows from L2, counted half), plus what
+// the consumer pays per slice it has to add.
+struct Cut {
+  int waves, slices, steps_per_slice;
+};
+inline int row_tiles(int n_rows) { return n_rows <= 16 ? 1 : (n_rows <= 32 ? 2 : 4); }
+int g_force_slices = 0;
+Cut cut_for(int tiles, int n_steps, int tt) {
+  constexpr int n_cu = 256;   // MI355X
+  Cut best{4, 1, (n_steps + kAhead - 1) / kAhead * kAhead};
+  long long best_cost = -1;
+  for (int want = 1; want <= 8; ++want) {
+    if (g_force_slices && want != g_force_slices) continue;
+    const int sps = ((n_steps + want - 1) / want + kAhead - 1) / kAhead * kAhead;
+    const int slices = (n_steps + sps - 1) / sps;
+    for (int w = 4; w <= 8; ++w) {
+      if (g_force_waves >= 4 && g_force_waves <= 8 && w != g_force_waves) continue;
+      const long long blocks = (long long)((tiles + w - 1) / w) * slices;
+      const long long cost = (blocks + n_cu - 1) / n_cu * (sps + 24) * (2 * w + tt) + 12LL * slices;
+      if (best_cost < 0 || cost < best_cost) best = Cut{w, slices, sps}, best_cost = cost;
+    }
+  }
+  return best;
+}
+
+template <int TT>
+void launch_cut(const bf16_t *x, const bf16_t *w, const StreamArgs &a, int waves, hipStream_t s) {
+  switch (waves) {
+    case 4: return launch_w<TT, 1, 1, 4>(x, w, a, s);
+    case 5: return launch_w<TT, 1, 1, 5>(x, w, a, s);
+    case 6: return launch_w<TT, 1, 1, 6>(x, w, a, s);
+    case 7: return launch_w<TT, 1, 1, 7>(x, w, a, s);
+    default: return launch_w<TT, 1, 1, 8>(x, w, a, s);
+  }
+}
+
 template <int TT, int G, int R>
 void launch(const bf16_t *x, const bf16_t *w, const StreamArgs &a, hipStream_t s) {
   switch (waves_for((a.n_out + 15) / 16, R)) {
@@ -212,6 +269,8 @@ void launch(const bf16_t *x, const bf16_t *w, const StreamArgs &a, hipStream_t s
 
 // For measurements: waves per block of every later call (4..8; 0 = choose).
 extern "C" void sb_gemm_stream_force(int waves) { g_force_waves = waves; }
+// ... and the K slices sb_gemm_stream_partial_bf16 aims at (1..8; 0 = choose).
+extern "C" void sb_gemm_stream_force_slices(int slices) { g_force_slices = slices; }
 
 // Rows of X this kernel takes: 17..64 is what it is built for; fewer rows work too.
 extern "C" int sb_gemm_stream_max_rows(void) { return 64; }
@@ -237,7 +296,7 @@ extern "C" int sb_gemm_stream_bf16(void *y, int y_dtype, const void *x, const vo
              "sb_gemm_stream_bf16: inner size %d is too large", n_in);
   if (n_rows == 0) return SB_OK;
   hipStream_t s = (hipStream_t)stream;
-  const StreamArgs a{y, y_dtype, bias, bias_dtype, resid, n_rows, n_out, n_in};
+  const StreamArgs a{y, y_dtype, bias, bias_dtype, resid, n_rows, n_out, n_in, nullptr, 0};
   const bf16_t *xb = (const bf16_t *)x, *wb = (const bf16_t *)w;
   const int tt = n_rows <= 16 ? 1 : (n_rows <= 32 ? 2 : 4);
   if (gated) {
@@ -250,4 +309,33 @@ extern "C" int sb_gemm_stream_bf16(void *y, int y_dtype, const void *x, const vo
     else launch<4, 1, 2>(xb, wb, a, s);
   }
   return sb::check_launch("sb_gemm_stream_bf16");
+}
+
+// K slices sb_gemm_stream_partial_bf16 will produce for these sizes.
+extern "C" int sb_gemm_stream_slices(int n_rows, int n_out, int n_in) {
+  if (n_rows <= 0 || n_out <= 0 || n_in <= 0) return 1;
+  return cut_for((n_out + 15) / 16, (n_in + kStepK - 1) / kStepK, row_tiles(n_rows)).slices;
+}
+
+// The raw product in K slices, for a consumer that adds them (and bias, residual, ...) itself:
+// partial float [slices][n_rows][n_out], slices = sb_gemm_stream_slices(...).  Operands as above.
+extern "C" int sb_gemm_stream_partial_bf16(float *partial, const void *x, const void *w, int n_rows, int n_out,
+                                           int n_in, void *stream) {
+  SB_REQUIRE(partial && x && w, "sb_gemm_stream_partial_bf16: null pointer");
+  SB_REQUIRE(n_rows >= 0 && n_out > 0 && n_in > 0, "sb_gemm_stream_partial_bf16: bad sizes");
+  SB_SUPPORT(n_rows <= 64, "sb_gemm_stream_partial_bf16: %d rows, at most 64", n_rows);
+  SB_SUPPORT(n_in % 8 == 0, "sb_gemm_stream_partial_bf16: inner size %d is not a multiple of 8", n_in);
+  SB_SUPPORT((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) % 16 == 0,
+             "sb_gemm_stream_partial_bf16: operands must be 16-byte aligned");
+  SB_SUPPORT((unsigned long long)(n_rows + 1) * n_in * 2 < (1ull << 31) && (unsigned long long)n_in * 32 < (1ull << 31),
+             "sb_gemm_stream_partial_bf16: inner size %d is too large", n_in);
+  if (n_rows == 0) return SB_OK;
+  const Cut c = cut_for((n_out + 15) / 16, (n_in + kStepK - 1) / kStepK, row_tiles(n_rows));
+  const StreamArgs a{nullptr, SB_F32, nullptr, 0, nullptr, n_rows, n_out, n_in, partial, c.steps_per_slice};
+  const bf16_t *xb = (const bf16_t *)x, *wb = (const bf16_t *)w;
+  hipStream_t s = (hipStream_t)stream;
+  if (n_rows <= 16) launch_cut<1>(xb, wb, a, c.waves, s);
+  else if (n_rows <= 32) launch_cut<2>(xb, wb, a, c.waves, s);
+  else launch_cut<4>(xb, wb, a, c.waves, s);
+  return sb::check_launch("sb_gemm_stream_partial_bf16");
 }

@@ -277,11 +277,14 @@ SKINNY_MAX_ROWS = 64
 def gemm_bf16_partial(x: torch.Tensor, w: torch.Tensor, packed_shape=None) -> Optional[torch.Tensor]:
     """The raw product x w^T of bfloat16 rows in K slices, float32 [slices, rows, out], for a
     consumer that adds the slices itself (:func:`reduce_resid_norm`, :func:`rope_kv_store`).
-    Up to 16 rows (and up to 64 without packed weights): the weight-streaming kernel.  More rows
-    against packed weights: the tiled kernel with K cut over the grid, as long as the cut gives
-    more than one slice (a narrow matrix and up to a few hundred rows: one slice would leave
-    most of the GPU without a tile; measured at 128 rows, output product 18 against 49 us, down
-    36 against 146).  None when neither applies: the caller then takes the whole product."""
+    Packed weights, up to 64 rows: the kernel whose waves split the output features and share
+    the rows through LDS, with K cut over the grid so that the blocks fill the GPU (measured
+    with the kernel that adds the slices, Qwen2.5-7B down product: 31 us at 8 rows, 38 at 64).
+    Packed weights, more rows: the tiled kernel with K cut over the grid, as long as the cut gives
+    more than one slice (a narrow matrix and up to a few hundred rows; one slice would leave most
+    of the GPU without a tile: at 128 rows the output product takes 18 against 49 us, down 36
+    against 146).  Row-major weights, up to 64 rows: the kernel whose waves split K.  None when
+    none applies: the caller then takes the whole product."""
     _dev(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or x.dim() != 2:
         return None
@@ -292,19 +295,25 @@ def gemm_bf16_partial(x: torch.Tensor, w: torch.Tensor, packed_shape=None) -> Op
     if t == 0 or k % 8 or x.data_ptr() % 16 or w.data_ptr() % 16:
         return None
     lib = library.core()
-    packed = 1 if packed_shape is not None else 0
-    if t >= TILED_PARTIAL_MIN_ROWS and packed:
+    which = _few_rows_kernel[0]
+    if packed_shape is not None and t <= SKINNY_MAX_ROWS and which in (None, "stream"):
+        slices = lib.sb_gemm_stream_slices(t, n, k)
+        partial = torch.empty((slices, t, n), dtype=torch.float32, device=x.device)
+        check(lib.sb_gemm_stream_partial_bf16(_p(partial), _p(x), _p(w), t, n, k, _stream()))
+        return partial
+    if packed_shape is not None and (t > SKINNY_MAX_ROWS or which == "tiled"):
         slices = lib.sb_gemm_mfma_slices(t, n, k)
         if slices > 1 or t <= SKINNY_MAX_ROWS:
             partial = torch.empty((slices, t, n), dtype=torch.float32, device=x.device)
-            check(lib.sb_gemm_mfma_partial_bf16(_p(partial), _p(x), _p(w), t, n, k, packed, _stream()))
+            check(lib.sb_gemm_mfma_partial_bf16(_p(partial), _p(x), _p(w), t, n, k, 1, _stream()))
             return partial
         return None
     if t > SKINNY_MAX_ROWS:
         return None
     slices = lib.sb_gemm_skinny_slices(t, n, k)
     partial = torch.empty((slices, t, n), dtype=torch.float32, device=x.device)
-    check(lib.sb_gemm_skinny_partial_bf16(_p(partial), _p(x), _p(w), t, n, k, packed, _stream()))
+    check(lib.sb_gemm_skinny_partial_bf16(_p(partial), _p(x), _p(w), t, n, k, 1 if packed_shape is not None else 0,
+                                          _stream()))
     return partial
 
 
@@ -424,27 +433,29 @@ def gemm_tile_shape(shape: Optional[int]):
 
 
 @contextlib.contextmanager
-def gemm_few_rows_kernel(which: Optional[str], waves: int = 0):
-    """For tests and measurements: inside the block products of up to 64 rows go to the kernel
-    ``which`` ("stream", "skinny" or "tiled"; "stream" needs packed weights) whatever the sizes,
-    and the stream kernel uses ``waves`` waves per block (4 to 8; 0: its own choice)."""
+def gemm_few_rows_kernel(which: Optional[str], waves: int = 0, slices: int = 0):
+    """For tests and measurements: inside the block products of up to 64 rows, whole or in K
+    slices, go to the kernel ``which`` ("stream", "skinny" or "tiled"; "stream" needs packed
+    weights) whatever the sizes, and the stream kernel uses ``waves`` waves per block (4 to 8)
+    and aims at ``slices`` K slices (1 to 8); 0: its own choice."""
     if which not in (None, "stream", "skinny", "tiled"):
         raise ValueError(f"unknown kernel {which!r}")
     lib = library.core()
     before = _few_rows_kernel[0]
     _few_rows_kernel[0] = which
     lib.sb_gemm_stream_force(int(waves))
+    lib.sb_gemm_stream_force_slices(int(slices))
     try:
         yield
     finally:
         _few_rows_kernel[0] = before
         lib.sb_gemm_stream_force(0)
+        lib.sb_gemm_stream_force_slices(0)
 
 
 _few_rows_kernel = [None]
 MFMA_MAX_HEAD_DIM = 256
 STREAM_MIN_BLOCKS = 192
-TILED_PARTIAL_MIN_ROWS = 17
 
 
 def attention_mfma_ok(q_dtype, cache_dtype, head_dim: int) -> bool:

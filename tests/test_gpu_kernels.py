@@ -235,9 +235,9 @@ def test_gemm_bf16_wide_matrix_with_few_rows(t):
 @pytest.mark.parametrize("n, k", [(100, 96), (224, 200), (3584, 512), (264, 2368), (72, 18944 // 8)])
 @pytest.mark.parametrize("packed", [False, True])
 def test_gemm_bf16_partial_slices_add_up(t, n, k, packed):
-    """The product in K slices (weight-streaming kernel up to 16 rows, tiled kernel with K cut
-    over the grid from 17 rows on, for packed weights): the slices add up to x w^T, and the
-    consumers that add them give the fused results."""
+    """The product in K slices (packed weights: the stream kernel up to 64 rows, the tiled kernel
+    beyond; row-major weights: the kernel whose waves split K): the slices add up to x w^T, and
+    the consumers that add them give the fused results."""
     from sonicboom_amd import ops
     x, w = randn(t, k, dtype=BF16), randn(n, k, dtype=BF16, scale=0.05)
     wd = w.to(DEV)
@@ -254,6 +254,24 @@ def test_gemm_bf16_partial_slices_add_up(t, n, k, packed):
         rd = resid.to(DEV)
         ops.reduce_resid_norm(partial, bias.to(DEV), rd, None, 1e-6, None)
         close(rd, ref_gemm(x, w, bias, resid), atol=3e-5 * math.sqrt(k), rtol=1e-5, what="slices + bias + residual")
+
+
+@pytest.mark.parametrize("which, waves, slices", [("stream", 4, 1), ("stream", 5, 3), ("stream", 7, 8), ("stream", 8, 5),
+                                                  ("tiled", 0, 0), ("skinny", 0, 0)])
+@pytest.mark.parametrize("t", [3, 16, 33, 64])
+@pytest.mark.parametrize("n, k", [(100, 96), (1000, 520), (264, 2368), (72, 4744)])
+def test_gemm_bf16_partial_every_kernel(which, waves, slices, t, n, k):
+    """Each kernel that can cut K, at forced cuts: slices that end inside a staged chunk of 256 k
+    and inside a k-step, more slices asked for than K has chunks, columns that end inside a
+    tile."""
+    from sonicboom_amd import ops
+    x, w = randn(t, k, dtype=BF16), randn(n, k, dtype=BF16, scale=0.05)
+    with ops.gemm_few_rows_kernel(which, waves, slices):
+        partial = ops.gemm_bf16_partial(x.to(DEV), ops.pack_weight(w.to(DEV)), packed_shape=(n, k))
+    assert partial is not None and partial.shape[1:] == (t, n) and 1 <= partial.shape[0] <= 8
+    if which == "stream" and slices:
+        assert partial.shape[0] <= slices
+    close(partial.double().sum(0), ref_gemm(x, w), atol=3e-5 * math.sqrt(k), rtol=1e-5, what=f"{which}: sum of the slices")
 
 
 def test_gemm_bf16_refuses_what_it_cannot_take():
