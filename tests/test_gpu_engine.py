@@ -64,3 +64,20 @@ def test_unequal_batches_one_after_another(model_folders, name, dtype):
             assert_logits_close(g[:p], want[:p], dtype, f"{name} batch prompt")
             assert_logits_close(g[p:], want[p:], dtype, f"{name} batch decode")
         assert eng.cache.held_pages() == 0 and not eng.cache.live_slots
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name, n_req", [("A", 40), ("B", 23)])
+def test_many_short_requests_in_one_batch(model_folders, name, n_req, dtype):
+    """Dozens of requests in one batch: the decode steps bring 17 to 64 rows, which take other
+    product kernels than a handful of rows does.  Prompts of 1 to 9 tokens, 2 to 6 decoded."""
+    folder = model_folders[name]
+    eng = engine_for(folder, dtype, max_tokens=64 * 48)
+    rng = np.random.default_rng(77)
+    prompts = [int(n) for n in rng.integers(1, 10, size=n_req)]
+    decoded = [int(n) for n in rng.integers(2, 7, size=n_req)]
+    reqs = requests_for(name, [p + d for p, d in zip(prompts, decoded)], seed=21)
+    got = run_batch(eng, reqs, prompts)
+    for i, (r, g) in enumerate(zip(reqs, got)):
+        assert_logits_close(g, plain_logits(folder, r), dtype, f"{name} request {i} of {n_req}")
+    assert eng.cache.held_pages() == 0 and not eng.cache.live_slots
