@@ -81,3 +81,22 @@ def test_many_short_requests_in_one_batch(model_folders, name, n_req, dtype):
     for i, (r, g) in enumerate(zip(reqs, got)):
         assert_logits_close(g, plain_logits(folder, r), dtype, f"{name} request {i} of {n_req}")
     assert eng.cache.held_pages() == 0 and not eng.cache.live_slots
+
+
+@pytest.mark.parametrize("dtype, pages", [("float32", 0), ("bfloat16", 0), ("bfloat16", 2), ("bfloat16", 8)])
+def test_large_batch_of_longer_requests(model_folders, dtype, pages):
+    """64 requests of 130 to 200 tokens decoded together, through the engine; in bfloat16 also
+    with the decode attention kernel's waves taking 2 and 8 pages in a row, as they do when the
+    page table is wide."""
+    from sonicboom_amd import ops
+    folder = model_folders["A"]
+    eng = engine_for(folder, dtype, max_tokens=64 * 4 * 64)
+    rng = np.random.default_rng(91)
+    prompts = [int(n) for n in rng.integers(120, 190, size=64)]
+    reqs = requests_for("A", [p + 10 for p in prompts], seed=33)
+    head_dim = TINY["A"]["hidden_size"] // TINY["A"]["num_attention_heads"]
+    with ops.attention_decode_pages_per_wave(head_dim, pages):
+        got = run_batch(eng, reqs, prompts)
+    for i, (r, g) in enumerate(zip(reqs, got)):
+        assert_logits_close(g, plain_logits(folder, r), dtype, f"request {i}")
+    assert eng.cache.held_pages() == 0 and not eng.cache.live_slots
