@@ -1,5 +1,6 @@
-// bf16 matrix product for 17 to 64 rows against a wide packed matrix (decode at
-// batch 17..64: the gate/up product, the head):  Y[t,n] = sum_k X[t,k] W[n,k].
+// bf16 matrix product for up to 128 rows against a packed matrix (decode steps and
+// short prompts: the gate/up product, the head; qkv, output and down with K cut
+// over the grid):  Y[t,n] = sum_k X[t,k] W[n,k].
 //
 // Like the few-row kernel it is bound by reading W once, and every wave loads its
 // W fragments straight from global memory into MFMA operands.  With this many rows
@@ -223,7 +224,7 @@ int waves_for(int tiles, int r) {
 struct Cut {
   int waves, slices, steps_per_slice;
 };
-inline int row_tiles(int n_rows) { return n_rows <= 16 ? 1 : (n_rows <= 32 ? 2 : 4); }
+inline int row_tiles(int n_rows) { return n_rows <= 16 ? 1 : (n_rows <= 32 ? 2 : (n_rows <= 64 ? 4 : 8)); }
 int g_force_slices = 0;
 Cut cut_for(int tiles, int n_steps, int tt) {
   constexpr int n_cu = 256;   // MI355X
@@ -272,11 +273,11 @@ extern "C" void sb_gemm_stream_force(int waves) { g_force_waves = waves; }
 // ... and the K slices sb_gemm_stream_partial_bf16 aims at (1..8; 0 = choose).
 extern "C" void sb_gemm_stream_force_slices(int slices) { g_force_slices = slices; }
 
-// Rows of X this kernel takes: 17..64 is what it is built for; fewer rows work too.
-extern "C" int sb_gemm_stream_max_rows(void) { return 64; }
+// Rows of X this kernel takes.
+extern "C" int sb_gemm_stream_max_rows(void) { return 128; }
 
 // Y = X W^T (+bias) (+resid), or with gated != 0: Y = silu(X Wg^T) * (X Wu^T) for the packed
-// halves [Wg; Wu].  X [n_rows, n_in] bf16, n_rows <= 64, n_in a multiple of 8; W in the packed
+// halves [Wg; Wu].  X [n_rows, n_in] bf16, n_rows <= 128, n_in a multiple of 8; W in the packed
 // tile layout (16 x 32 tiles of 1 KB in fragment order, tiles of a row block consecutive in k).
 extern "C" int sb_gemm_stream_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,
                                    int bias_dtype, const float *resid, int n_rows, int n_out, int n_in,
@@ -286,7 +287,7 @@ extern "C" int sb_gemm_stream_bf16(void *y, int y_dtype, const void *x, const vo
              n_rows, n_out, n_in);
   SB_REQUIRE(sb::valid_dtype(y_dtype) && (!bias || sb::valid_dtype(bias_dtype)),
              "sb_gemm_stream_bf16: unknown dtype");
-  SB_SUPPORT(n_rows <= 64, "sb_gemm_stream_bf16: %d rows, at most 64", n_rows);
+  SB_SUPPORT(n_rows <= 128, "sb_gemm_stream_bf16: %d rows, at most 128", n_rows);
   SB_SUPPORT(n_in % 8 == 0, "sb_gemm_stream_bf16: inner size %d is not a multiple of 8", n_in);
   SB_SUPPORT((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) % 16 == 0,
              "sb_gemm_stream_bf16: operands must be 16-byte aligned");
@@ -298,15 +299,17 @@ extern "C" int sb_gemm_stream_bf16(void *y, int y_dtype, const void *x, const vo
   hipStream_t s = (hipStream_t)stream;
   const StreamArgs a{y, y_dtype, bias, bias_dtype, resid, n_rows, n_out, n_in, nullptr, 0};
   const bf16_t *xb = (const bf16_t *)x, *wb = (const bf16_t *)w;
-  const int tt = n_rows <= 16 ? 1 : (n_rows <= 32 ? 2 : 4);
+  const int tt = row_tiles(n_rows);
   if (gated) {
     if (tt == 1) launch<1, 2, 1>(xb, wb, a, s);
     else if (tt == 2) launch<2, 2, 1>(xb, wb, a, s);
-    else launch<4, 2, 1>(xb, wb, a, s);
+    else if (tt == 4) launch<4, 2, 1>(xb, wb, a, s);
+    else launch<8, 2, 1>(xb, wb, a, s);
   } else {
     if (tt == 1) launch<1, 1, 2>(xb, wb, a, s);
     else if (tt == 2) launch<2, 1, 2>(xb, wb, a, s);
-    else launch<4, 1, 2>(xb, wb, a, s);
+    else if (tt == 4) launch<4, 1, 2>(xb, wb, a, s);
+    else launch<8, 1, 2>(xb, wb, a, s);
   }
   return sb::check_launch("sb_gemm_stream_bf16");
 }

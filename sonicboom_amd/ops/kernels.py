@@ -10,6 +10,7 @@ a missing library or a refused size raises
 from __future__ import annotations
 
 import contextlib
+import math
 
 from typing import Optional
 
@@ -396,17 +397,24 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], re
     lib = library.core()
     bdt = _dt(bias) if bias is not None else 0
     packed = 1 if packed_shape is not None else 0
-    # Up to 64 rows: a wide packed matrix (enough 16-row tiles, or gate/up pairs of them, for
-    # STREAM_MIN_BLOCKS blocks of four waves) goes to the kernel whose waves split the output
-    # features and share the rows through LDS; a narrower one to the kernel whose waves split K
-    # and which can cut K over the grid as well.  Measured at Qwen2.5-7B sizes: gate/up at 64
+    # A wide packed matrix (enough 16-row tiles, or gate/up pairs of them, for STREAM_MIN_BLOCKS
+    # blocks of four waves) and up to 128 rows: the kernel whose waves split the output features
+    # and share the rows through LDS.  Other products of up to 64 rows: the kernel whose waves
+    # split K and which can cut K over the grid as well.  The rest: the tiled kernel.  Measured at Qwen2.5-7B sizes: gate/up at 64
     # rows 53 us (tiled kernel 74, few-row kernel 85), at 8 rows 48 (few-row kernel 50); the
     # head at 16 rows 196 (few-row kernel 259).
     which = _few_rows_kernel[0]
     if which is None:
         wave_units = -(-n // 16) if gated else -(-n // 32)
         which = "stream" if packed and wave_units >= 4 * STREAM_MIN_BLOCKS else "skinny"
-    if t <= SKINNY_MAX_ROWS and which == "stream" and packed:
+        if t > SKINNY_MAX_ROWS and which == "stream":
+            # 65 to 128 rows: the tiled kernel's 128 x 128 tiles do as well or better unless their
+            # count leaves the last round over the 256 CUs nearly empty (Qwen2.5-7B gate/up: 296
+            # tiles, 85 us at 128 rows against 70 here; 216, 462 or 1,188 tiles: the tiled kernel)
+            rounds = -(-n // (64 if gated else 128)) / 256.0
+            if math.ceil(rounds) / rounds < 1.4:
+                which = "tiled"
+    if t <= STREAM_MAX_ROWS and which == "stream" and packed:
         check(lib.sb_gemm_stream_bf16(_p(out), _dt(out), _p(x), _p(w), _p(bias), bdt, _p(resid), t, n, k,
                                       1 if gated else 0, _stream()))
     elif t <= SKINNY_MAX_ROWS and which != "tiled":
@@ -456,6 +464,7 @@ def gemm_few_rows_kernel(which: Optional[str], waves: int = 0, slices: int = 0):
 _few_rows_kernel = [None]
 MFMA_MAX_HEAD_DIM = 256
 STREAM_MIN_BLOCKS = 192
+STREAM_MAX_ROWS = 128
 
 
 def attention_mfma_ok(q_dtype, cache_dtype, head_dim: int) -> bool:

@@ -183,7 +183,7 @@ def test_gemm_bf16_every_tile_shape(shape, packed, t, n, k):
         close(got, g / (1.0 + torch.exp(-g)) * u, atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"gated shape {shape}")
 
 
-@pytest.mark.parametrize("t", [1, 16, 17, 40, 64])
+@pytest.mark.parametrize("t", [1, 16, 17, 40, 64, 65, 100, 128])
 @pytest.mark.parametrize("waves", [0, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("n, k", [(100, 96), (1000, 520), (264, 2368), (4099, 264)])
 def test_gemm_bf16_stream_kernel(t, waves, n, k):
@@ -208,9 +208,9 @@ def test_gemm_bf16_stream_kernel(t, waves, n, k):
         close(got, g / (1.0 + torch.exp(-g)) * u, atol=1e-4 * math.sqrt(k), rtol=1e-4, what="stream, gated")
 
 
-@pytest.mark.parametrize("t", [8, 17, 64])
+@pytest.mark.parametrize("t", [8, 17, 64, 100])
 def test_gemm_bf16_wide_matrix_with_few_rows(t):
-    """Up to 64 rows against a packed matrix wide enough for the stream kernel, and one wave's
+    """Up to 128 rows against a packed matrix wide enough for the stream kernel, and one wave's
     worth of columns less (which stays with the kernel that splits K), plain and gated: the
     choice between the kernels changes no result."""
     from sonicboom_amd import ops
