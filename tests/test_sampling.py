@@ -6,7 +6,8 @@ import numpy as np
 import pytest
 
 from plain import sampling_plain as SP
-from sonicboom_amd.sampling import SamplingParams, filter_candidates, gumbel_draw, penalty_items, philox4x32_10
+from sonicboom_amd.sampling import (SamplingParams, draw_rows, filter_candidates, gumbel_draw, penalty_items,
+                                    philox4x32_10)
 
 F32 = np.float32
 
@@ -114,6 +115,37 @@ def test_product_host_stages_equal_the_plain_sampler(params):
         assert kept_ids.tolist() == [c[0] for c in want]
         for pos in (0, 17, 2 ** 33 + 5):
             assert gumbel_draw(kept_ids, kept_z, trial, pos) == SP.draw(want, trial, pos)
+
+
+@pytest.mark.parametrize("params", [
+    dict(temperature=0.8), dict(temperature=1.3, top_k=5), dict(temperature=0.5, top_p=0.7),
+    dict(temperature=1.0, min_p=0.2), dict(temperature=0.9, top_k=40, top_p=0.9, min_p=0.01),
+    dict(temperature=0.05, top_p=0.5), dict(temperature=2.0, top_k=1), dict(temperature=1.0, top_p=1e-9, min_p=1.0),
+])
+def test_all_rows_at_once_equal_the_plain_sampler_row_by_row(params):
+    """A step's rows filtered and drawn together: every row gets the token the plain sampler
+    gives it alone, whatever the other rows hold (flat and peaked rows, ties, far positions)."""
+    r = np.random.default_rng(11)
+    rows = []
+    for i in range(24):
+        logits = (r.standard_normal(400) * (0.2 if i % 5 == 0 else 3.0)).astype(F32)
+        if i % 7 == 3:
+            logits[10:20] = logits[5]                    # ties among the best
+        if i % 6 == 1:
+            logits[3] = 80.0                             # one candidate far above the window
+        rows.append(logits)
+    cands = [SP.select_candidates(l, params["temperature"]) for l in rows]
+    ids = np.array([[c[0] for c in cs] for cs in cands], dtype=np.int32)
+    z = np.array([[c[1] for c in cs] for cs in cands], dtype=np.float32)
+    positions = [int(q) for q in r.integers(0, 5000, size=len(rows))]
+    positions[0], positions[1] = 0, 2 ** 33 + 5
+    sp = SamplingParams(seed=77, **params)
+    got = draw_rows(ids, z, positions, sp)
+    for i, cs in enumerate(cands):
+        kept = SP.filter_candidates(cs, params.get("top_k", 0), params.get("top_p", 1.0), params.get("min_p", 0.0))
+        assert got[i] == SP.draw(kept, 77, positions[i]), f"row {i}"
+        one = draw_rows(ids[i:i + 1], z[i:i + 1], positions[i:i + 1], sp)
+        assert one == [got[i]]
 
 
 def test_params_validation():
