@@ -114,70 +114,129 @@ __device__ __forceinline__ uint64_t cand_key(float logit, float temperature, int
   return (uint64_t(float_key(__fdiv_rn(logit, temperature))) << 32) | uint64_t(0xffffffffu - uint32_t(id));
 }
 
-// One block per row.  Eight radix passes over the 64-bit keys find the key of
-// rank k exactly; every key at or above it is a candidate; a bitonic sort in
-// shared memory orders them.
-__global__ void __launch_bounds__(kSelThreads)
-top_candidates_kernel(int32_t *__restrict__ cand_id, float *__restrict__ cand_z,
-                      const float *__restrict__ logits, int vocab, int k, float temperature) {
-  __shared__ uint32_t hist[kSelWaves][256];
-  __shared__ uint64_t sel[kMaxCand];
-  __shared__ uint64_t prefix_s;
-  __shared__ int remaining_s;
-  __shared__ int count_s;
-  const float *x = logits + size_t(blockIdx.x) * vocab;
-  const int tid = threadIdx.x, wave = tid >> 6;
-  const int want = min(k, vocab);
-  if (tid == 0) {
-    prefix_s = 0;
-    remaining_s = want;
-    count_s = 0;
-  }
-  for (int i = tid; i < kMaxCand; i += kSelThreads) sel[i] = 0;
+// The key of rank `want` (1 = largest) among the keys a block's threads hold in registers, PER per
+// thread: eight radix passes from the top byte down, each a histogram of the keys that share the
+// bytes found so far (one histogram per wave, then added up), and a look for the bucket that
+// holds the rank.  A key of 0 stands for "nothing" and lies below every real key; `want` must not
+// exceed the number of real keys.  Every thread of the block calls it and gets the same key.
+struct SelectShared {
+  uint32_t hist[kSelWaves][256];
+  uint32_t wave_total[4];
+  uint64_t prefix;
+  int remaining;
+};
 
+template <int PER>
+__device__ __forceinline__ uint64_t select_kth(const uint64_t (&mine)[PER], int want, SelectShared &sh) {
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  if (tid == 0) {
+    sh.prefix = 0;
+    sh.remaining = want;
+  }
   for (int pass = 7; pass >= 0; --pass) {
     const int shift = pass * 8;
-    for (int i = tid; i < kSelWaves * 256; i += kSelThreads) (&hist[0][0])[i] = 0;
+    for (int i = tid; i < kSelWaves * 256; i += kSelThreads) (&sh.hist[0][0])[i] = 0;
     __syncthreads();
-    const uint64_t prefix = prefix_s;
-    for (int i = tid; i < vocab; i += kSelThreads) {
-      const uint64_t key = cand_key(x[i], temperature, i);
+    const uint64_t prefix = sh.prefix;
+    const uint32_t remaining = uint32_t(sh.remaining);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const uint64_t key = mine[j];
       if (pass == 7 || (key >> (shift + 8)) == (prefix >> (shift + 8)))
-        atomicAdd(&hist[wave][(key >> shift) & 0xffu], 1u);
+        atomicAdd(&sh.hist[wave][(key >> shift) & 0xffu], 1u);
     }
+    __syncthreads();
+    // thread b < 256 owns bucket b: its count, and by a suffix sum over the wave and the waves
+    // above the count of all higher buckets; the bucket that holds the rank is the one with
+    // fewer than `remaining` keys above it and at least that many with its own
+    uint32_t mine_n = 0;
+    if (tid < 256)
+      for (int wv = 0; wv < kSelWaves; ++wv) mine_n += sh.hist[wv][tid];
+    uint32_t suffix = mine_n;           // buckets tid .. end of the wave
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const uint32_t other = __shfl_down(suffix, off, 64);
+      if (lane + off < 64) suffix += other;
+    }
+    if (tid < 256 && lane == 0) sh.wave_total[wave] = suffix;
     __syncthreads();
     if (tid < 256) {
-      uint32_t total = 0;
-      for (int wv = 0; wv < kSelWaves; ++wv) total += hist[wv][tid];
-      hist[0][tid] = total;
-    }
-    __syncthreads();
-    if (tid == 0) {
-      int remaining = remaining_s;
-      uint32_t above = 0;
-      int chosen = 0;
-      for (int b = 255; b >= 0; --b) {
-        const uint32_t n = hist[0][b];
-        if (above + n >= uint32_t(remaining)) {
-          chosen = b;
-          break;
-        }
-        above += n;
+      uint32_t above = suffix - mine_n;
+      for (int wv = wave + 1; wv < 4; ++wv) above += sh.wave_total[wv];
+      if (above < remaining && above + mine_n >= remaining) {
+        sh.remaining = int(remaining - above);
+        sh.prefix = prefix | (uint64_t(tid) << shift);
       }
-      remaining_s = remaining - int(above);
-      prefix_s = prefix | (uint64_t(chosen) << shift);
     }
     __syncthreads();
   }
+  return sh.prefix;
+}
 
-  const uint64_t kth = prefix_s;
-  for (int i = tid; i < vocab; i += kSelThreads) {
-    const uint64_t key = cand_key(x[i], temperature, i);
-    if (key >= kth) {
-      const int slot = atomicAdd(&count_s, 1);
-      if (slot < kMaxCand) sel[slot] = key;
-    }
+// Stage 1 for long rows: block (part, row) finds the kMaxCand largest keys among kPartElems
+// elements of its row and writes them, in no order, to part_keys [row][part][kMaxCand] (zeros fill
+// what a short part leaves); the row's kMaxCand largest are among them.
+constexpr int kPartElems = 4096;
+__global__ void __launch_bounds__(kSelThreads)
+top_part_kernel(uint64_t *__restrict__ part_keys, const float *__restrict__ logits, int vocab, float temperature) {
+  __shared__ SelectShared sh;
+  __shared__ int count_s;
+  constexpr int PER = kPartElems / kSelThreads;
+  const int tid = threadIdx.x;
+  const float *x = logits + size_t(blockIdx.y) * vocab;
+  const int first = blockIdx.x * kPartElems;
+  uint64_t mine[PER];
+#pragma unroll
+  for (int j = 0; j < PER; ++j) {
+    const int i = first + j * kSelThreads + tid;
+    mine[j] = i < vocab ? cand_key(x[i], temperature, i) : 0ull;
   }
+  uint64_t *out = part_keys + (size_t(blockIdx.y) * gridDim.x + blockIdx.x) * kMaxCand;
+  if (tid < kMaxCand) out[tid] = 0;
+  if (tid == 0) count_s = 0;
+  const int real = min(kPartElems, vocab - first);
+  const uint64_t kth = select_kth<PER>(mine, min(kMaxCand, real), sh);   // syncs inside
+#pragma unroll
+  for (int j = 0; j < PER; ++j)
+    if (mine[j] >= kth && mine[j] != 0) {
+      const int slot = atomicAdd(&count_s, 1);
+      if (slot < kMaxCand) out[slot] = mine[j];
+    }
+}
+
+// Stage 2, or the only stage of a short row: one block per row finds the k largest keys among the
+// row's (FROM_KEYS: among the n_keys that stage 1 left in part_keys, at most kRowKeys * 1024; else
+// among the keys of its vocab <= kRowKeys * 1024 logits), sorts them (bitonic, in shared memory)
+// and writes ids and z.
+constexpr int kRowKeys = 16;
+template <bool FROM_KEYS>
+__global__ void __launch_bounds__(kSelThreads)
+top_candidates_kernel(int32_t *__restrict__ cand_id, float *__restrict__ cand_z,
+                      const float *__restrict__ logits, const uint64_t *__restrict__ part_keys, int n_keys,
+                      int vocab, int k, float temperature) {
+  __shared__ SelectShared sh;
+  __shared__ uint64_t sel[kMaxCand];
+  __shared__ int count_s;
+  const float *x = logits + size_t(blockIdx.x) * vocab;
+  const uint64_t *pk = part_keys + size_t(blockIdx.x) * n_keys;
+  const int n_scan = FROM_KEYS ? n_keys : vocab;
+  const int tid = threadIdx.x;
+  const int want = min(k, vocab);
+  uint64_t mine[kRowKeys];
+#pragma unroll
+  for (int j = 0; j < kRowKeys; ++j) {
+    const int i = j * kSelThreads + tid;
+    mine[j] = i < n_scan ? (FROM_KEYS ? pk[i] : cand_key(x[i], temperature, i)) : 0ull;
+  }
+  if (tid == 0) count_s = 0;
+  for (int i = tid; i < kMaxCand; i += kSelThreads) sel[i] = 0;
+  const uint64_t kth = select_kth<kRowKeys>(mine, want, sh);              // syncs inside
+#pragma unroll
+  for (int j = 0; j < kRowKeys; ++j)
+    if (mine[j] >= kth && mine[j] != 0) {
+      const int slot = atomicAdd(&count_s, 1);
+      if (slot < kMaxCand) sel[slot] = mine[j];
+    }
   __syncthreads();
 
   // Bitonic sort of 256 keys, descending; empty slots (0) sink to the end.
@@ -248,14 +307,40 @@ extern "C" int sb_penalize(float *logits, int vocab, const int32_t *item_row, co
   return sb::check_launch("sb_penalize");
 }
 
+// 64-bit words of scratch sb_top_candidates needs for rows of this length (0: none).  Rows of
+// more than two parts go through stage 1.
+extern "C" size_t sb_top_candidates_scratch(int n_rows, int vocab) {
+  if (n_rows <= 0 || vocab <= 2 * kPartElems) return 0;
+  return size_t(n_rows) * ((vocab + kPartElems - 1) / kPartElems) * kMaxCand;
+}
+// The longest row sb_top_candidates takes: what its second stage can hold of the parts' keys.
+extern "C" int sb_top_candidates_max_vocab(void) { return kRowKeys * kSelThreads / kMaxCand * kPartElems; }
+
+// cand_id int32 [n_rows, k], cand_z float [n_rows, k]: the k <= 256 best of every row by
+// z = logit / temperature, ordered (z descending, id ascending); entries past the row's length
+// hold id -1.  scratch: sb_top_candidates_scratch(n_rows, vocab) 64-bit words (may be NULL when 0).
 extern "C" int sb_top_candidates(int32_t *cand_id, float *cand_z, const float *logits, int n_rows,
-                                 int vocab, int k, float temperature, void *stream) {
+                                 int vocab, int k, float temperature, uint64_t *scratch, void *stream) {
   SB_REQUIRE(cand_id && cand_z && logits, "sb_top_candidates: null pointer");
   SB_REQUIRE(n_rows >= 0 && vocab > 0, "sb_top_candidates: bad sizes rows=%d vocab=%d", n_rows, vocab);
   SB_REQUIRE(temperature > 0.0f, "sb_top_candidates: temperature must be positive");
   SB_SUPPORT(k >= 1 && k <= kMaxCand, "sb_top_candidates: %d candidates asked, at most %d", k, kMaxCand);
+  SB_SUPPORT(n_rows <= 65535, "sb_top_candidates: more than 65535 rows");
+  SB_SUPPORT(vocab <= sb_top_candidates_max_vocab(), "sb_top_candidates: a row of %d logits, at most %d", vocab,
+             sb_top_candidates_max_vocab());
   if (n_rows == 0) return SB_OK;
-  top_candidates_kernel<<<n_rows, kSelThreads, 0, (hipStream_t)stream>>>(cand_id, cand_z, logits, vocab,
-                                                                         k, temperature);
+  hipStream_t s = (hipStream_t)stream;
+  if (sb_top_candidates_scratch(n_rows, vocab) == 0) {
+    top_candidates_kernel<false><<<n_rows, kSelThreads, 0, s>>>(cand_id, cand_z, logits, nullptr, 0, vocab, k,
+                                                                temperature);
+    return sb::check_launch("sb_top_candidates");
+  }
+  SB_REQUIRE(scratch, "sb_top_candidates: no scratch for the parts' candidates");
+  const int parts = (vocab + kPartElems - 1) / kPartElems;
+  top_part_kernel<<<dim3(parts, n_rows), kSelThreads, 0, s>>>(scratch, logits, vocab, temperature);
+  int rc = sb::check_launch("sb_top_candidates (parts)");
+  if (rc != SB_OK) return rc;
+  top_candidates_kernel<true><<<n_rows, kSelThreads, 0, s>>>(cand_id, cand_z, logits, scratch, parts * kMaxCand,
+                                                             vocab, k, temperature);
   return sb::check_launch("sb_top_candidates");
 }

@@ -124,9 +124,42 @@ int sb_penalize(float *logits, int vocab, const int32_t *item_row, const int32_t
 /* The `k` (<= 256) candidates with the largest z = logit / temperature of every
  * row (ties toward the lower id), ordered by (z descending, id ascending).
  * cand_id int32 [n_rows,k], cand_z f32 [n_rows,k]; rows with vocab < k are
- * filled with id -1. */
+ * filled with id -1.  Long rows are cut into parts whose best go through
+ * `scratch`: sb_top_candidates_scratch(...) 64-bit words (NULL when that is 0). */
+size_t sb_top_candidates_scratch(int n_rows, int vocab);
 int sb_top_candidates(int32_t *cand_id, float *cand_z, const float *logits, int n_rows, int vocab,
-                      int k, float temperature, void *stream);
+                      int k, float temperature, uint64_t *scratch, void *stream);
+
+/* ---- bf16 products on the matrix cores ----------------------------------
+ * X bf16 [n_rows, n_in] row-major, n_in a multiple of 8, operands 16-byte
+ * aligned.  W bf16 [n_out, n_in] row-major, or (packed != 0, or always for the
+ * stream kernel) re-laid in 16 x 32 tiles of 1 KB in MFMA fragment order, rows
+ * padded to 16 and k to 32, tiles of a row block consecutive in k; gated: the two
+ * halves [gate; up] packed one after the other, Y = silu(X Wg^T) * (X Wu^T).
+ * Y f32 or bf16; bias [n_out] f32 or bf16 or NULL; resid f32 [n_rows, n_out] or
+ * NULL (may be Y itself).  The *_partial_* forms write the raw product in K
+ * slices, f32 [slices][n_rows][n_out], slices as the matching *_slices says. */
+int sb_gemm_skinny_max_rows(void);                       /* up to 64 rows, waves split K */
+size_t sb_gemm_skinny_scratch(int n_rows, int n_out, int n_in, int gated);
+int sb_gemm_skinny_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,
+                        int bias_dtype, const float *resid, int n_rows, int n_out, int n_in, int gated,
+                        int packed, float *scratch, size_t scratch_floats, void *stream);
+int sb_gemm_skinny_slices(int n_rows, int n_out, int n_in);
+int sb_gemm_skinny_partial_bf16(float *partial, const void *x, const void *w, int n_rows, int n_out,
+                                int n_in, int packed, void *stream);
+int sb_gemm_stream_max_rows(void);                       /* up to 128 rows, waves split the features */
+int sb_gemm_stream_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,
+                        int bias_dtype, const float *resid, int n_rows, int n_out, int n_in, int gated,
+                        void *stream);
+int sb_gemm_stream_slices(int n_rows, int n_out, int n_in);     /* up to 64 rows */
+int sb_gemm_stream_partial_bf16(float *partial, const void *x, const void *w, int n_rows, int n_out,
+                                int n_in, void *stream);
+int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,   /* tiled */
+                      int bias_dtype, const float *resid, int n_rows, int n_out, int n_in, int gated,
+                      int packed, void *stream);
+int sb_gemm_mfma_slices(int n_rows, int n_out, int n_in);
+int sb_gemm_mfma_partial_bf16(float *partial, const void *x, const void *w, int n_rows, int n_out,
+                              int n_in, int packed, void *stream);
 
 #ifdef __cplusplus
 }

@@ -265,7 +265,9 @@ def top_candidates(logits: torch.Tensor, temperature: float, k: int = MAX_CANDID
     ids = torch.empty((n, k), dtype=torch.int32, device=logits.device)
     z = torch.empty((n, k), dtype=torch.float32, device=logits.device)
     lib = library.core()
-    check(lib.sb_top_candidates(_p(ids), _p(z), _p(logits), n, vocab, k, float(temperature), _stream()))
+    words = lib.sb_top_candidates_scratch(n, vocab)
+    scratch = torch.empty((words,), dtype=torch.int64, device=logits.device) if words else None
+    check(lib.sb_top_candidates(_p(ids), _p(z), _p(logits), n, vocab, k, float(temperature), _p(scratch), _stream()))
     return ids, z
 
 

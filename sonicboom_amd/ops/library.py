@@ -32,7 +32,7 @@ _CORE_SIGNATURES = {
     "sb_argmax": [_P, _P, _I, _I, _P, _P, _P],
     "sb_argmax_parts": [_I],
     "sb_penalize": [_P, _I, _P, _P, _P, _I, _F, _F, _F, _I, _P],
-    "sb_top_candidates": [_P, _P, _P, _I, _I, _I, _F, _P],
+    "sb_top_candidates": [_P, _P, _P, _I, _I, _I, _F, _P, _P],
 }
 # Entry points of later kernels; declared when the library has them.
 _OPTIONAL_SIGNATURES = {
@@ -95,6 +95,8 @@ def core():
                 _declare(lib, _OPTIONAL_SIGNATURES, optional=True)
                 lib.sb_gemm_skinny_scratch.argtypes = [_I, _I, _I, _I]
                 lib.sb_gemm_skinny_scratch.restype = c_size_t
+                lib.sb_top_candidates_scratch.argtypes = [_I, _I]
+                lib.sb_top_candidates_scratch.restype = c_size_t
                 lib._sb_path = path
                 _core = lib
     return _core

@@ -654,19 +654,23 @@ def test_argmax_first_maximum(vocab):
     assert got == want and got[:3] == [0, vocab - 1, 3]
 
 
-@pytest.mark.parametrize("vocab", [7, 256, 300, 5000, 152064])
+@pytest.mark.parametrize("vocab", [7, 256, 300, 5000, 8192, 8193, 12289, 152064])
 @pytest.mark.parametrize("temperature", [1.0, 0.7])
 def test_top_candidates(vocab, temperature):
+    """Rows short enough for one block, and rows cut into parts of 4,096 whose best are merged
+    (from 8,193 on; a last part of one element; a part that holds all of the best)."""
     from sonicboom_amd import ops
-    x = randn(4, vocab, scale=2.0)
+    x = randn(6, vocab, scale=2.0)
     x[1] = torch.round(x[1])                        # many ties: ordered by id
     x[2, :] = 1.25                                  # all equal
     x[3, ::3] = -0.0
     x[3, 1::3] = 0.0                                # signed zeros are one value
+    x[4, vocab // 3:] = -float("inf")               # fewer finite values than candidates, perhaps
+    x[5, -min(300, vocab):] += 50.0                 # all of the best at the row's end
     k = min(256, vocab)
     ids, z = ops.top_candidates(x.to(DEV), temperature, k)
     ids, z = ids.cpu().numpy(), z.cpu().numpy()
-    for r in range(4):
+    for r in range(6):
         want = sampling_plain.select_candidates(x[r].numpy(), temperature)
         assert [c[0] for c in want] == ids[r].tolist(), f"row {r}"
         assert np.array_equal(np.array([c[1] for c in want], dtype=np.float32), z[r]), f"row {r}"
