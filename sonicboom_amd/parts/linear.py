@@ -5,8 +5,8 @@ call this helper, which picks the kernel from the types and sizes at hand:
 
 * float32 weights (the 32-bit path, or a tensor the file stores in 32-bit):
   the plain kernel, true float32 throughout;
-* bfloat16 weights and activations: the matrix-core kernels (a weight-streaming
-  one for up to 64 rows, a tiled one for more).  For them the weight is
+* bfloat16 weights and activations: the matrix-core kernels (two that stream
+  the weights once for few rows, a tiled one for more).  For them the weight is
   re-laid once, when the projection is built, into the tile order the matrix
   cores read (:func:`sonicboom_amd.ops.pack_weight`) and the row-major copy is
   dropped.  An inner size that is not a multiple of 8 keeps the row-major
