@@ -184,6 +184,33 @@ def register_toys():
             view = qkv.view(qkv.shape[0], -1, head_dim)
             view[:, :heads_q + heads_kv, 0] += pos[:, None]
 
+    from sonicboom_amd.parts import Part
+
+    @register_part("ffn", "toy_routed")
+    class RoutedFFN(Part):
+        """Every row goes to the ``top`` experts whose router logits are largest, and gets their
+        outputs weighted by the softmax over those logits (float32).  The experts are nested
+        parts of the framework's own dense kind; the routing is torch on the host's terms."""
+        category = "ffn"
+
+        def __init__(self, spec, tensors, parts, rt):
+            super().__init__(spec, tensors, parts, rt)
+            self.top = int(spec.params["top"])
+            self.router = tensors["router"].float()
+            self.experts = [parts[f"expert{i}"] for i in range(int(spec.params["n_experts"]))]
+
+        def forward(self, h, x, ctx):
+            logits = h.float() @ self.router.T
+            best, which = torch.topk(logits, self.top, dim=-1)
+            share = torch.softmax(best, dim=-1)
+            for e, expert in enumerate(self.experts):
+                rows, slot = torch.nonzero(which == e, as_tuple=True)
+                if rows.numel() == 0:
+                    continue
+                out = torch.zeros((rows.numel(), x.shape[1]), dtype=torch.float32, device=x.device)
+                expert.forward(h[rows].contiguous(), out, ctx)
+                x[rows] += out * share[rows, slot][:, None]
+
     return ops, register_architecture
 
 
@@ -225,16 +252,24 @@ def toy_spec(cfg):
                 pos = rope_spec(layer["head_dim"], layer.get("base", 1e4))
             mixer = attention_spec(p + "attn.", w, layer["heads"], layer["kv_heads"], layer["head_dim"], pos,
                                    window=layer.get("window", 0), qkv_bias=layer.get("bias", True))
+        if "experts" in layer:
+            ffn = PartSpec("ffn", "toy_routed", {"top": layer["top"], "n_experts": layer["experts"]},
+                           {"router": TensorSpec(p + "router", (layer["experts"], w), init=(0.0, 1.0))},
+                           {f"expert{e}": gated_ffn_spec(p + f"e{e}.", w, layer["ff"]) for e in range(layer["experts"])})
+        else:
+            ffn = gated_ffn_spec(p + "mlp.", w, layer["ff"])
         blocks.append(prenorm_block_spec(rmsnorm_spec(p + "n1", w, d["eps"]), mixer,
-                                         rmsnorm_spec(p + "n2", w, d["eps"]), gated_ffn_spec(p + "mlp.", w, layer["ff"])))
+                                         rmsnorm_spec(p + "n2", w, d["eps"]), ffn))
     for e in d["order"]:
         order.append(OrderEntry(e["block"], e.get("cache"), e.get("writes", True)))
     return ModelSpec("ToyForCausalLM", w, v, embedding_spec("emb", v, w), blocks, order,
                      rmsnorm_spec("norm", w, d["eps"]), head_spec("head", v, w))
 
 
-def plain_toy(cfg, w, tokens):
-    """The toy architecture written out with the plain parts: whole sequence, no cache."""
+def plain_toy(cfg, w, tokens, margins=None):
+    """The toy architecture written out with the plain parts: whole sequence, no cache.
+    ``margins``: a list that receives, per routed layer, every row's gap between the last chosen
+    and the first rejected router logit."""
     d = cfg.d
     n = len(tokens)
     pos = np.arange(n)
@@ -271,8 +306,26 @@ def plain_toy(cfg, w, tokens):
             out = P.linear(a, w[p + "attn.o_proj.weight"])
         x = (out + x).astype(np.float32)
         f = P.rms_norm(x, w[p + "n2"], d["eps"])
-        x = (P.swiglu(f, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"]) + x
-             ).astype(np.float32)
+        if "experts" in layer:
+            logits = P.linear(f, w[p + "router"]).astype(np.float64)
+            order_ = np.argsort(-logits, axis=1, kind="stable")
+            top = layer["top"]
+            if margins is not None:
+                rows = np.arange(n)
+                margins.append(logits[rows, order_[:, top - 1]] - logits[rows, order_[:, top]])
+            y = np.zeros_like(x, dtype=np.float64)
+            for t in range(n):
+                chosen = order_[t, :top]
+                z = np.exp(logits[t, chosen] - logits[t, chosen].max())
+                z /= z.sum()
+                for share, e in zip(z, chosen):
+                    q = p + f"e{e}."
+                    y[t] += share * P.swiglu(f[t:t + 1], w[q + "gate_proj.weight"], w[q + "up_proj.weight"],
+                                             w[q + "down_proj.weight"])[0]
+            x = (y + x).astype(np.float32)
+        else:
+            x = (P.swiglu(f, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
+                          w[p + "mlp.down_proj.weight"]) + x).astype(np.float32)
     return P.linear(P.rms_norm(x, w["norm"], d["eps"]), w["head"])
 
 
@@ -293,6 +346,16 @@ TOY_WINDOWS = {
     # the two windowed layers have different needs, so three cache groups exist
     "order": [{"block": 0, "cache": 0}, {"block": 0, "cache": 0, "writes": False}, {"block": 1, "cache": 1},
               {"block": 2, "cache": 2}, {"block": 0, "cache": 3}],
+}
+
+
+TOY_ROUTED = {
+    "architectures": ["ToyForCausalLM"], "vocab_size": 130, "width": 56, "eps": 1e-5,
+    "layers": [{"mixer": "attention", "heads": 2, "kv_heads": 2, "head_dim": 16, "ff": 72},
+               # routing sits in the last layer: a row that another rounding would route elsewhere
+               # then changes its own logits only, and the test can leave such rows out
+               {"mixer": "attention", "heads": 4, "kv_heads": 1, "head_dim": 16, "ff": 24, "experts": 5, "top": 2}],
+    "order": [{"block": 0, "cache": 0}, {"block": 1, "cache": 1}],
 }
 
 
@@ -363,3 +426,39 @@ def test_windows_shared_cache_and_a_layer_that_runs_twice(dtype):
     assert held[0] == 5 and held[50] <= 2 and held[70] <= 3
     eng.free_slot(s)
     assert all(eng.cache.held_pages(i) == 0 for i in range(3))
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_toy_feed_forward_with_routing(dtype):
+    """A feed-forward that routes every row to two of five experts, defined above in this file
+    from a router tensor and five nested parts of the framework's dense kind: registered, built
+    from its spec, loaded by tensor name and stepped (whole, cut, and two sequences at once)
+    without a change to the framework."""
+    from sonicboom_amd.engine import StepEntry
+    cfg, ref, model, eng = build_toy(TOY_ROUTED, dtype)
+    assert not eng.decode_loop().use_graph              # the toy routes with host control flow
+    rng = np.random.default_rng(4)
+    a, b = ([int(t) for t in rng.integers(0, 130, size=n)] for n in (90, 41))
+    gaps_a, gaps_b = [], []
+    want_a, want_b = plain_toy(cfg, ref, a, gaps_a), plain_toy(cfg, ref, b, gaps_b)
+    # rows whose routing hangs on less than the rounding of the path are left out
+    least = 1e-4 if dtype == F32 else 0.05
+    ok_a, ok_b = gaps_a[0] > least, gaps_b[0] > least
+    assert ok_a.sum() > 60 and ok_b.sum() > 25
+    s = eng.alloc_slot()
+    got = eng.step([StepEntry(s, a, range(len(a)))])
+    close(got[ok_a], want_a[ok_a], dtype, "routed, whole")
+    eng.free_slot(s)
+    sa, sb = eng.alloc_slot(), eng.alloc_slot()
+    out = eng.step([StepEntry(sa, a[:50], range(50)), StepEntry(sb, b[:20], range(20))])
+    close(out[:50][ok_a[:50]], want_a[:50][ok_a[:50]], dtype, "routed, a's prompt")
+    close(out[50:][ok_b[:20]], want_b[:20][ok_b[:20]], dtype, "routed, b's prompt")
+    for i in range(21):
+        out = eng.step([StepEntry(sa, [a[50 + i]], [0]), StepEntry(sb, [b[20 + i]], [0])])
+        if ok_a[50 + i]:
+            close(out[:1], want_a[50 + i:51 + i], dtype, f"routed, a token {i}")
+        if ok_b[20 + i]:
+            close(out[1:], want_b[20 + i:21 + i], dtype, f"routed, b token {i}")
+    eng.free_slot(sa)
+    eng.free_slot(sb)
+    assert eng.cache.held_pages() == 0
