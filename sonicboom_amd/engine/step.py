@@ -11,7 +11,7 @@ rows that were asked for, in the order of the entries and of their ``want``.
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence
+from typing import Optional, Sequence
 
 import numpy as np
 import torch

@@ -17,7 +17,6 @@ the query rows of that matrix alone.
 """
 from __future__ import annotations
 
-import math
 from typing import Optional
 
 import numpy as np

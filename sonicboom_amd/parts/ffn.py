@@ -11,7 +11,6 @@ from __future__ import annotations
 
 import torch
 
-from .. import ops
 from .base import Part, register_part
 from .linear import Linear
 from .spec import PartSpec, TensorSpec

@@ -4,7 +4,6 @@ Tests build their models in temporary folders; nothing is read from or written
 to the repository.  GPU tests carry the ``gpu`` marker and are skipped by
 ``-m "not gpu"``.
 """
-import json
 import os
 import sys
 

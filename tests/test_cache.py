@@ -4,7 +4,7 @@ import random
 import numpy as np
 import pytest
 
-from sonicboom_amd.cache import PAGE, CacheError, GroupSpec, PagedCache, PagePool, group_entries, pages_for
+from sonicboom_amd.cache import CacheError, GroupSpec, PagedCache, PagePool, group_entries, pages_for
 
 
 def make(max_tokens=64 * 8, window=0, max_slots=None):

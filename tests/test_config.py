@@ -1,5 +1,4 @@
 """Configuration and registry (CPU)."""
-import copy
 import json
 
 import pytest

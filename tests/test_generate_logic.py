@@ -4,7 +4,7 @@ given back and used again, positions of the draws."""
 import numpy as np
 import pytest
 
-from sonicboom_amd.cache import PAGE, CacheError, GroupSpec, PagedCache
+from sonicboom_amd.cache import GroupSpec, PagedCache
 from sonicboom_amd.engine.generate import generate, plan_batches
 from sonicboom_amd.sampling import SamplingParams
 

@@ -1,6 +1,5 @@
 """Sampling on the host: the plain sampler against the reference's test vectors, and the
 product's host stages (filters, Philox, Gumbel draw) against the plain sampler."""
-import math
 
 import numpy as np
 import pytest
