@@ -136,6 +136,36 @@ def test_graph_replay_gives_the_same_tokens(model_folders):
     assert s == without.generate(prompts, temperature=0.7, seed=3, max_tokens=40, stop_tokens=())
 
 
+def test_graph_replay_when_the_page_table_grows(tmp_path):
+    """Decoding across 1,024 tokens: the decode loop's buffers are keyed by the page table's
+    width (steps of 16 pages), so the step is recorded a second time there; tokens with and
+    without graphs agree, and the logits on both sides of the edge are the plain ones."""
+    from sonicboom_amd.api import Model
+    from sonicboom_amd.engine import StepEntry
+    from sonicboom_amd.weights import write_random_model
+    cfg = dict(TINY["A"], max_position_embeddings=2048)
+    folder = str(tmp_path / "long_a")
+    write_random_model(folder, cfg, seed=77, dtype="bfloat16")
+    model = Model.load(folder, dtype="bfloat16")
+    rng = np.random.default_rng(12)
+    prompts = [random_prompt(rng, cfg["vocab_size"], n) for n in (1000, 30)]
+    with_graph = model.session(max_tokens=64 * 24)
+    without = model.session(max_tokens=64 * 24)
+    without.engine.use_graphs = False
+    a = with_graph.generate(prompts, max_tokens=60, stop_tokens=())
+    b = without.generate(prompts, max_tokens=60, stop_tokens=())
+    assert a == b and all(len(o) == 60 for o in a)
+    widths = sorted(k[1] for k in with_graph.engine.decode_loop()._graphs)
+    assert widths == [16, 32], f"graphs recorded for table widths {widths}"
+    # the produced tokens, fed back whole: logits around position 1,024 against the plain model
+    whole = prompts[0] + a[0]
+    eng = without.engine
+    s = eng.alloc_slot()
+    got = eng.step([StepEntry(s, whole, range(1000, len(whole)))]).cpu().numpy()
+    eng.free_slot(s)
+    assert_logits_close(got, plain_logits(folder, whole)[1000:], "bfloat16", "around the edge of the table")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_token_by_token_from_the_first_token(model_folders, dtype):
     """A sequence fed one token at a time from its very first token, over several pages,
