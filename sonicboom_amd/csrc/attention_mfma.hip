@@ -890,15 +890,25 @@ extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache
   hipStream_t s = (hipStream_t)stream;
   SB_SUPPORT(heads_kv * head_tiles <= 65535, "sb_attn_decode_bf16: too many heads");
   // A wave takes one page and asks for all of it at once (one round trip to memory), or, when
-  // that still leaves a block for every CU, 2, 4 or 8 pages in a row with half a page in flight
+  // that still leaves a block for every CU, several pages in a row with half a page in flight
   // while the half before it is multiplied (measured on cold caches, Qwen2.5-7B heads: 64
-  // sequences of 2,060 keys 65 us with eight pages per wave against 82 with one; 8 sequences of
-  // 16,400 keys 57 against 79; one sequence of 32,780 keys 33 against 43).
+  // sequences of 2,060 keys 53 us in one chunk, 65 with eight pages per wave and two chunks, 82
+  // with one page per wave; 8 sequences of 16,400 keys 57 with eight pages per wave against 79
+  // with one; one sequence of 32,780 keys 33 against 43).
   const long long per_chunk = (long long)heads_kv * head_tiles * n_seqs;
   int ppw = 1;
-  if (HD <= 128)
-    for (int c = 8; c >= 2 && ppw == 1; c /= 2)
-      if ((long long)((max_pages + 4 * c - 1) / (4 * c)) * per_chunk >= 256) ppw = c;
+  if (HD <= 128) {
+    if (per_chunk >= 256) {
+      // a block per CU without cutting the rows at all: one chunk, a quarter of the table's width
+      // per wave, no partial results and no second kernel (dealing each row's own pages evenly
+      // to the four waves instead measured the same at 64 sequences and 10 % slower at 128)
+      ppw = (max_pages + kPagesPerChunk - 1) / kPagesPerChunk;
+      if (ppw < 2) ppw = 2;
+    } else {
+      for (int c = 8; c >= 2 && ppw == 1; c /= 2)
+        if ((long long)((max_pages + 4 * c - 1) / (4 * c)) * per_chunk >= 256) ppw = c;
+    }
+  }
   if (g_force_ppw > 0 && (g_force_ppw == 1 || HD <= 128)) ppw = g_force_ppw;
   const int pages_per_chunk = kPagesPerChunk * ppw;
   const int n_chunks = (max_pages + pages_per_chunk - 1) / pages_per_chunk;
@@ -926,8 +936,8 @@ extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache
   return sb::check_launch("sb_attn_decode_bf16 (merge)");
 }
 
-// Measurement hook: pages per wave of the decode kernel (1, 2, 4, 8; 0: chosen from the sizes).
-extern "C" void sb_attn_decode_force(int ppw) { g_force_ppw = (ppw == 1 || ppw == 2 || ppw == 4 || ppw == 8) ? ppw : 0; }
+// Measurement hook: pages per wave of the decode kernel (0: chosen from the sizes).
+extern "C" void sb_attn_decode_force(int ppw) { g_force_ppw = ppw > 0 ? ppw : 0; }
 
 // Measurement hook: heads per wave and waves per block in prefill (0: chosen from the group size).
 extern "C" void sb_attn_prefill_force(int nc, int waves) { g_force_nc = nc; g_force_waves = waves; }

@@ -488,15 +488,20 @@ def test_attention_decode_matrix_cores(hq, hkv, hd, window):
         assert torch.equal(got, again)
 
 
-def test_attention_decode_matrix_cores_many_sequences():
-    """Two hundred sequences: enough blocks for the kernel whose waves take several pages."""
+@pytest.mark.parametrize("window", [0, 100])
+@pytest.mark.parametrize("longest", [300, 900])
+def test_attention_decode_matrix_cores_many_sequences(window, longest):
+    """Two hundred sequences: a block for every CU without cutting the rows, so each block takes
+    its row whole (one chunk, a quarter of the table's width per wave, no merge kernel); lengths
+    from one key to many pages, with and without a window."""
     from sonicboom_amd import ops
     hq, hkv, hd = 8, 4, 32
     rng = np.random.default_rng(5)
-    lens = [int(n) for n in rng.integers(1, 300, size=200)]
-    q, kc, vc, table, rows, scale, want = attention_case(hq, hkv, hd, lens, [[n - 1] for n in lens], 0, seed=9)
+    lens = [int(n) for n in rng.integers(1, longest, size=200)]
+    lens[:4] = [1, 64, 65, longest]
+    q, kc, vc, table, rows, scale, want = attention_case(hq, hkv, hd, lens, [[n - 1] for n in lens], window, seed=9)
     pos = torch.tensor([p for _, p in rows], dtype=torch.int32)
-    got = ops.attention_decode_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), hq, hkv, hd, scale, 0)
+    got = ops.attention_decode_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), hq, hkv, hd, scale, window)
     close(got, want, atol=1.5e-2, rtol=1e-2, what="decode, 200 sequences")
 
 
