@@ -890,23 +890,37 @@ extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache
   hipStream_t s = (hipStream_t)stream;
   SB_SUPPORT(heads_kv * head_tiles <= 65535, "sb_attn_decode_bf16: too many heads");
   // A wave takes one page and asks for all of it at once (one round trip to memory), or, when
-  // that still leaves a block for every CU, several pages in a row with half a page in flight
-  // while the half before it is multiplied (measured on cold caches, Qwen2.5-7B heads: 64
+  // two pages per wave still leave a block for every CU, several pages in a row with half a page
+  // in flight while the half before it is multiplied (measured on cold caches, Qwen2.5-7B heads: 64
   // sequences of 2,060 keys 53 us in one chunk, 65 with eight pages per wave and two chunks, 82
   // with one page per wave; 8 sequences of 16,400 keys 57 with eight pages per wave against 79
   // with one; one sequence of 32,780 keys 33 against 43).
   const long long per_chunk = (long long)heads_kv * head_tiles * n_seqs;
   int ppw = 1;
-  if (HD <= 128) {
-    if (per_chunk >= 256) {
-      // a block per CU without cutting the rows at all: one chunk, a quarter of the table's width
-      // per wave, no partial results and no second kernel (dealing each row's own pages evenly
-      // to the four waves instead measured the same at 64 sequences and 10 % slower at 128)
-      ppw = (max_pages + kPagesPerChunk - 1) / kPagesPerChunk;
-      if (ppw < 2) ppw = 2;
-    } else {
-      for (int c = 8; c >= 2 && ppw == 1; c /= 2)
-        if ((long long)((max_pages + 4 * c - 1) / (4 * c)) * per_chunk >= 256) ppw = c;
+  if (HD <= 128 && (long long)((max_pages + 7) / 8) * per_chunk >= 256) {
+    // How many pages in a row: the count with the least estimated time, in microseconds, from
+    // what was measured (MI355X, cold caches).  A wave gets through a page in about 3.3 us
+    // whatever the head size (two round trips to memory); a CU streams about 27 GB/s, all of
+    // them together 5.3 TB/s; a block costs about 4 us besides; more than one chunk costs the
+    // partial results and the second kernel, about 8 us.  The table's width is taken for the rows' length less half of the 16
+    // pages it is rounded up by.  One chunk (a quarter of the width per wave) is among the
+    // candidates: it wins when sequences x kv heads alone fill most of the GPU.
+    const double page_bytes = 2.0 * SB_PAGE * HD * 2;
+    const int pages = max_pages > 8 ? max_pages - 8 : 1;
+    const int whole = (max_pages + kPagesPerChunk - 1) / kPagesPerChunk;
+    const int candidates[5] = {2, 4, 8, 16, whole < 2 ? 2 : whole};
+    double best = -1.0;
+    for (int c : candidates) {
+      const int chunks = (max_pages + 4 * c - 1) / (4 * c);
+      const int full = pages / (4 * c) > 1 ? pages / (4 * c) : 1;
+      const double busy = double(per_chunk) * full < 256.0 ? double(per_chunk) * full : 256.0;
+      const double rate = busy * 27e3 < 5.3e6 ? busy * 27e3 : 5.3e6;            // bytes per us
+      const int run = c < pages ? c : pages;
+      // a block spends about 4 us on what is not streaming (look-ups, queries, the merge)
+      const double stream = double(per_chunk) * pages * page_bytes / rate * (1.0 + 4.0 / (run * 3.3));
+      const double in_a_row = run * 3.3 + 4.0;
+      const double t = (stream > in_a_row ? stream : in_a_row) + (chunks > 1 ? 8.0 : 0.0);
+      if (best < 0.0 || t < best) best = t, ppw = c;
     }
   }
   if (g_force_ppw > 0 && (g_force_ppw == 1 || HD <= 128)) ppw = g_force_ppw;
