@@ -505,6 +505,23 @@ def test_attention_decode_matrix_cores_many_sequences(window, longest):
     close(got, want, atol=1.5e-2, rtol=1e-2, what="decode, 200 sequences")
 
 
+@pytest.mark.parametrize("window", [0, 300])
+@pytest.mark.parametrize("n_seqs, longest", [(30, 2000), (12, 5000), (3, 9000)])
+def test_attention_decode_matrix_cores_long_rows_of_unequal_length(window, n_seqs, longest):
+    """Rows long enough for the launcher to deal several pages to a wave and cut the rows into
+    chunks of its own choosing; lengths from one key to thousands in one batch, so that chunks
+    are full, partly filled and empty side by side."""
+    from sonicboom_amd import ops
+    hq, hkv, hd = 8, 4, 64
+    rng = np.random.default_rng(n_seqs)
+    lens = [int(n) for n in rng.integers(1, longest, size=n_seqs)]
+    lens[0], lens[-1] = longest, 1
+    q, kc, vc, table, rows, scale, want = attention_case(hq, hkv, hd, lens, [[n - 1] for n in lens], window, seed=21)
+    pos = torch.tensor([p for _, p in rows], dtype=torch.int32)
+    got = ops.attention_decode_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), hq, hkv, hd, scale, window)
+    close(got, want, atol=1.5e-2, rtol=1e-2, what=f"decode, {n_seqs} rows up to {longest} keys")
+
+
 @pytest.mark.parametrize("hq, hkv, hd", [(4, 2, 16), (5, 5, 48), (6, 2, 80), (28, 4, 128), (40, 2, 64)])
 @pytest.mark.parametrize("window", [0, 70, 1000])
 @pytest.mark.parametrize("pages", [1, 2, 4, 8])
