@@ -78,7 +78,7 @@ typedef struct boom_llm_step_entry {
 } boom_llm_step_entry;
 
 /* Called for every produced token of prompt `prompt`; a non-zero return ends that prompt's
- * sequence (the token is still part of the output). */
+ * sequence before that token: it is not reported. */
 typedef int (*boom_llm_batch_token_cb)(void *user, uint32_t prompt, boom_token token);
 
 /* --- model ------------------------------------------------------------------------------- */

@@ -75,8 +75,9 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = 
     HIP graph replay, greedy choice on the device).  ``stop_tokens``
     defaults to the model's own (its configuration's eos ids).  ``callback(i,
     token)`` is called for every produced token of request i in order; a true
-    return value ends that request, and the token it was called with is still
-    part of the output.  ``sampler`` has ``pick(logits, positions, histories)``
+    return value ends that request before that token, which is not part of the
+    output (/root/reference/capi/src/capi.cpp:2892-2898: an abort at a token
+    returns the tokens before it).  ``sampler`` has ``pick(logits, positions, histories)``
     and defaults to the device sampler for ``params``.
     """
     params = params.validated()
@@ -105,11 +106,12 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = 
                 flags = []
                 for s, t in zip(live, tokens):
                     t = int(t)
-                    s.out.append(t)
-                    s.history.append(t)
-                    ended = t in stop or len(s.out) >= params.max_tokens
                     if callback is not None and callback(s.index, t):
-                        ended = True
+                        ended = True                     # aborted at this token: it is not reported
+                    else:
+                        s.out.append(t)
+                        s.history.append(t)
+                        ended = t in stop or len(s.out) >= params.max_tokens
                     if ended:
                         outputs[s.index] = s.out
                         engine.free_slot(s.slot)

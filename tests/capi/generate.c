@@ -1,6 +1,7 @@
 /* Walks the C interface on a model folder (argv[1], dtype argv[2]): queries, one step, a batch
- * generation with a callback that cuts one prompt short.  Prints what it got, one item a line,
- * for the Python test to compare with the package's own results. */
+ * generation with a callback that cuts one prompt short (the refused token is not reported).
+ * Prints what it got, one item a line, for the Python test to compare with the package's own
+ * results. */
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -15,7 +16,7 @@
     }                                                                     \
   } while (0)
 
-static int stop_second_prompt_after_three(void *user, uint32_t prompt, boom_token token) {
+static int stop_second_prompt_at_its_third_token(void *user, uint32_t prompt, boom_token token) {
   int *seen = (int *)user;
   (void)token;
   if (prompt == 1) return ++*seen >= 3;
@@ -72,7 +73,7 @@ int main(int argc, char **argv) {
   MUST(boom_llm_slot_free(session, s1, &err));
   if (boom_llm_slot_free(session, s1, &err) == BOOM_OK) return 6;      /* freed twice: refused */
 
-  /* generation: three prompts, greedy, the callback ends the second one after three tokens */
+  /* generation: three prompts, greedy, the callback refuses the second one's third token */
   const boom_token p0[] = {1, 2, 3}, p1[] = {4, 5, 6, 7, 8, 9, 10}, p2[] = {11};
   const boom_token *prompts[3] = {p0, p1, p2};
   const size_t lens[3] = {3, 7, 1};
@@ -84,7 +85,7 @@ int main(int argc, char **argv) {
   boom_token out[18];
   uint32_t counts[3];
   int seen = 0;
-  MUST(boom_llm_generate(session, prompts, lens, 3, &sp, no_stop, 0, stop_second_prompt_after_three, &seen, out, counts,
+  MUST(boom_llm_generate(session, prompts, lens, 3, &sp, no_stop, 0, stop_second_prompt_at_its_third_token, &seen, out, counts,
                          &err));
   for (int i = 0; i < 3; ++i) {
     printf("greedy %d:", i);

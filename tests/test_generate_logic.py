@@ -108,10 +108,12 @@ def test_callback_and_max_tokens():
 
     def cb(i, t):
         seen.append((i, t))
-        return i == 0 and len([1 for j, _ in seen if j == 0]) == 2    # end request 0 after its second token
+        return i == 0 and len([1 for j, _ in seen if j == 0]) == 3    # end request 0 at its third token
 
     outs = generate(eng, [[1, 2], [3]], SamplingParams(max_tokens=4), stop_tokens=(), callback=cb, sampler=HostSampler())
+    # the token the callback refused is not reported (the reference's rule); it was shown to the callback
     assert outs == [expected([1, 2], 2), expected([3], 4)]
+    assert [t for i, t in seen if i == 0] == expected([1, 2], 3)
     assert [t for i, t in seen if i == 1] == outs[1]
     assert generate(eng, [[1]], SamplingParams(max_tokens=0), sampler=HostSampler()) == [[]]
     assert generate(eng, [], SamplingParams(), sampler=HostSampler()) == []
