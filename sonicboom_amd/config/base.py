@@ -62,6 +62,30 @@ def read_config_json(folder: str) -> dict:
     return d
 
 
+def merge_generation_config(folder: str, d: dict) -> dict:
+    """config.json's dict with the stop ids of the folder's generation_config.json (when there is
+    one) added to ``eos_token_id``: model folders keep the ids that end a turn there, often more
+    than config.json names.  Ids of config.json come first; nothing else is taken from the file."""
+    path = os.path.join(folder, "generation_config.json")
+    if not os.path.isfile(path):
+        return d
+    try:
+        with open(path) as f:
+            g = json.load(f)
+    except json.JSONDecodeError as e:
+        raise ConfigError(f"{path}: not valid JSON ({e})") from None
+    if not isinstance(g, dict):
+        raise ConfigError(f"{path}: the top level must be an object")
+    more = token_id_list(g.get("eos_token_id"), "eos_token_id (generation_config.json)")
+    if not more:
+        return d
+    have = token_id_list(d.get("eos_token_id"), "eos_token_id")
+    merged = list(have) + [t for t in more if t not in have]
+    out = dict(d)
+    out["eos_token_id"] = merged[0] if len(merged) == 1 else merged
+    return out
+
+
 def token_id_list(v, key: str) -> tuple:
     """``eos_token_id`` style values: null, one id, or a list of ids."""
     if v is None:

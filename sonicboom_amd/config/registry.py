@@ -12,7 +12,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Callable, Dict, Mapping
 
-from .base import ConfigError, read_config_json
+from .base import ConfigError, merge_generation_config, read_config_json
 
 
 @dataclass(frozen=True)
@@ -52,6 +52,6 @@ def architecture_of(config: Mapping) -> Architecture:
 
 def load_config(folder: str):
     """(architecture, typed configuration) of a model folder."""
-    d = read_config_json(folder)
+    d = merge_generation_config(folder, read_config_json(folder))
     arch = architecture_of(d)
     return arch, arch.config_class.from_dict(d)

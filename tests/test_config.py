@@ -83,6 +83,22 @@ def test_registry(tiny_configs, tmp_path):
         load_config(str(tmp_path / "nowhere"))
 
 
+def test_stop_ids_of_generation_config_are_added(tiny_configs, tmp_path):
+    """B's config.json names eos 7; the folder's generation_config.json adds 9 and repeats 7."""
+    (tmp_path / "config.json").write_text(json.dumps(tiny_configs["B"]))
+    (tmp_path / "generation_config.json").write_text(json.dumps({"eos_token_id": [9, 7], "temperature": 0.7}))
+    _, cfg = load_config(str(tmp_path))
+    assert cfg.eos_token_ids == (7, 9) and build_spec(cfg).stop_tokens == (7, 9)
+    (tmp_path / "generation_config.json").write_text(json.dumps({"eos_token_id": 7}))
+    assert load_config(str(tmp_path))[1].eos_token_ids == (7,)
+    (tmp_path / "generation_config.json").write_text(json.dumps({"eos_token_id": 100000}))
+    with pytest.raises(ConfigError, match="eos_token_id"):
+        load_config(str(tmp_path))                       # outside the vocabulary
+    (tmp_path / "generation_config.json").write_text("{not json")
+    with pytest.raises(ConfigError, match="generation_config.json"):
+        load_config(str(tmp_path))
+
+
 def test_spec_carries_the_configuration(tiny_configs):
     a = build_spec(Qwen2Config.from_dict(tiny_configs["A"]))
     b = build_spec(Qwen2Config.from_dict(tiny_configs["B"]))
