@@ -9,6 +9,8 @@
 // ascending) (:257-285).  The filters and the Gumbel draw run on the host.
 #include "common.cuh"
 
+#include <mutex>
+
 namespace {
 
 constexpr int kSelThreads = 1024;
@@ -293,6 +295,73 @@ extern "C" int sb_argmax(int32_t *ids, const float *logits, int n_rows, int voca
   if (rc != SB_OK) return rc;
   argmax_kernel<<<dim3(1, n_rows), kArgThreads, 0, s>>>(ids, nullptr, nullptr, part_val, part_idx, parts, parts);
   return sb::check_launch("sb_argmax (second stage)");
+}
+
+// ---- the greedy choice for callers that cannot allocate ------------------------
+// The first stage's partial results go to a file-scope device array instead of
+// buffers the caller brings.  In host code the array's name is only a stand-in
+// for the symbol: its device address is asked for once per device and kept.
+namespace {
+
+constexpr int kNoAllocEntries = 64 * 1024;     // rows * parts of one call, at most
+constexpr int kNoAllocDevices = 64;
+
+// [0, 4 * kNoAllocEntries): float values; [4 * kNoAllocEntries, 8 * kNoAllocEntries): int32 indices
+static __device__ __align__(256) unsigned char scratch[size_t(kNoAllocEntries) * 8];
+
+std::mutex g_scratch_lock;
+void *g_scratch_ptr[kNoAllocDevices] = {nullptr};
+
+// Device address of this device's copy of the array (every GPU holds its own).
+int scratch_of_current_device(void **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return sb::fail(SB_ERR_LAUNCH, "sb_argmax_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kNoAllocDevices)
+    return sb::fail(SB_ERR_UNSUPPORTED, "sb_argmax_noalloc: device %d, at most %d devices", dev, kNoAllocDevices);
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return sb::fail(SB_ERR_LAUNCH, "sb_argmax_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return SB_OK;
+}
+
+}  // namespace
+
+extern "C" int sb_argmax_noalloc_max_entries(void) { return kNoAllocEntries; }
+
+extern "C" int sb_argmax_noalloc(int32_t *ids, const float *logits, int n_rows, int vocab, void *stream) {
+  SB_REQUIRE(ids && logits, "sb_argmax_noalloc: null pointer");
+  SB_REQUIRE(n_rows >= 0 && vocab > 0, "sb_argmax_noalloc: bad sizes rows=%d vocab=%d", n_rows, vocab);
+  SB_SUPPORT(n_rows <= 65535, "sb_argmax_noalloc: more than 65535 rows");
+  const int parts = sb_argmax_parts(vocab);
+  SB_SUPPORT(parts == 1 || size_t(n_rows) * parts <= size_t(kNoAllocEntries),
+             "sb_argmax_noalloc: %d rows of %d parts need %zu partial results, the fixed buffer holds %d", n_rows,
+             parts, size_t(n_rows) * parts, kNoAllocEntries);
+  if (n_rows == 0) return SB_OK;
+  hipStream_t s = (hipStream_t)stream;
+  if (parts == 1) {
+    argmax_kernel<<<dim3(1, n_rows), kArgThreads, 0, s>>>(ids, nullptr, nullptr, logits, nullptr, vocab, vocab);
+    return sb::check_launch("sb_argmax_noalloc");
+  }
+  void *base = nullptr;
+  int rc = scratch_of_current_device(&base);
+  if (rc != SB_OK) return rc;
+  // Stage 1 writes every partial result that stage 2 reads, so nothing has to be cleared.
+  float *part_val = (float *)base;
+  int32_t *part_idx = (int32_t *)((unsigned char *)base + size_t(kNoAllocEntries) * 4);
+  const int span = (vocab + parts - 1) / parts;
+  argmax_kernel<<<dim3(parts, n_rows), kArgThreads, 0, s>>>(nullptr, part_val, part_idx, logits, nullptr, vocab,
+                                                            span);
+  rc = sb::check_launch("sb_argmax_noalloc");
+  if (rc != SB_OK) return rc;
+  argmax_kernel<<<dim3(1, n_rows), kArgThreads, 0, s>>>(ids, nullptr, nullptr, part_val, part_idx, parts, parts);
+  return sb::check_launch("sb_argmax_noalloc (second stage)");
 }
 
 extern "C" int sb_penalize(float *logits, int vocab, const int32_t *item_row, const int32_t *item_token,

@@ -114,6 +114,20 @@ int sb_argmax_parts(int vocab);
 int sb_argmax(int32_t *ids, const float *logits, int n_rows, int vocab, float *part_val,
               int32_t *part_idx, void *stream);
 
+/* sb_argmax for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no
+ * counterpart in the reference.  The caller passes the logits and the output
+ * only; the first stage's partial results go to a fixed device array of
+ * 512 KB that every GPU the library runs on holds until the process ends, so
+ * n_rows * sb_argmax_parts(vocab) may be at most sb_argmax_noalloc_max_entries()
+ * (65,536; e.g. 1,724 rows of 152,064 logits); more is refused with
+ * SB_ERR_UNSUPPORTED.  The call allocates and frees nothing.  Every call on a
+ * GPU shares that GPU's array: the first stage overwrites every entry the second
+ * stage reads, so nothing is cleared, and two calls that overlap on one GPU
+ * (different streams, or threads) race.  Same results as sb_argmax. */
+int sb_argmax_noalloc_max_entries(void);
+int sb_argmax_noalloc(int32_t *ids, const float *logits, int n_rows, int vocab, void *stream);
+
 /* Sampling penalties on the logits in place, for `n_items` (row, token, count)
  * triples: v = v>0 ? v/rp : v*rp (when rp != 1), then v -= freq*count + presence.
  * exact != 0 uses the single-rounding fma form of the sampled path. */
