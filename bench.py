@@ -1,17 +1,23 @@
-"""Decode and prefill throughput of the Qwen2.5-7B layer sizes with random bf16 weights
-on one MI355X.
+"""Decode and prefill throughput of the Qwen2.5 layer sizes with random bf16 weights on one
+MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
-                    [--sizes 7b|14b|72b] [--prompt T] [--context C]
+                    [--sizes 7b|14b|72b] [--prompt T] [--context C] [--workload steady|mixed]
 
-A "step" is one decode step: every sequence of the batch goes on by one token
-(step function, greedy choice on the device, the token fed back).  The default
-run has the sizes of the benchmark configuration (28 layers, width 3584, 28
-heads, 4 kv heads, head size 128, inner width 18944, vocabulary 152064), a
-batch of 8 and a cache for 4096 tokens per sequence, each holding a
-2,048-token prompt of seeded random ids.  One JSON line is printed:
-decoded tokens a second, the prefill of one 2,048-token prompt, the decode
-step against the HBM roofline, and decode at batch 1 and 64.
+A "step" is one decode step: every sequence of the batch goes on by one token (step function,
+greedy choice on the device, the token fed back).
+
+``--workload steady`` (the default) has the sizes of the benchmark configuration (28 layers,
+width 3584, 28 heads, 4 kv heads, head size 128, inner width 18944, vocabulary 152064), a batch
+of 8 and a cache for 4096 tokens per sequence, each holding a 2,048-token prompt of seeded random
+ids.  One JSON line is printed: decoded tokens a second (from the median step), the prefill of one
+2,048-token prompt, the decode step against the HBM roofline with the rates of its kernels, and
+decode at batch 1 and 64.
+
+``--workload mixed`` runs what the baseline names for the larger sizes through the generation
+loop itself: ``--sizes 14b``: 16 prompts of seeded lengths uniform in [256, 4096] in a cache of
+8192 tokens a sequence, prompts in one step, then 256 greedy steps; ``--sizes 72b``: 8 prompts of
+512 to 2048 tokens, 128 steps, 4096 tokens a sequence.  Prefill and decode are timed apart.
 """
 import argparse
 import json
@@ -35,6 +41,8 @@ CONFIG_14B = dict(CONFIG_7B, num_hidden_layers=48, hidden_size=5120, num_attenti
 CONFIG_72B = dict(CONFIG_7B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
                   num_key_value_heads=8, intermediate_size=29568)
 SIZES = {"7b": ("Qwen2.5-7B", CONFIG_7B), "14b": ("Qwen2.5-14B", CONFIG_14B), "72b": ("Qwen2.5-72B", CONFIG_72B)}
+# the mixed workloads: prompts, shortest, longest, greedy steps, cache tokens a sequence
+MIXED = {"14b": (16, 256, 4096, 256, 8192), "72b": (8, 512, 2048, 128, 4096), "7b": (16, 256, 4096, 256, 8192)}
 CONTEXT = 4096
 PROMPT = 2048
 
@@ -49,10 +57,12 @@ def model_numbers(cfg, n_layers):
                 layers=n_layers)
 
 
-def prefill_flops(m, t):
+def prefill_flops(m, lengths):
+    """Flops of a prompt step of sequences of these lengths whose last rows go through the head."""
+    t = sum(lengths)
     per_layer = 2 * t * (m["d"] * (m["qw"] + 2 * m["kvw"]) + m["qw"] * m["d"] + 3 * m["d"] * m["ff"])
-    attn = 4 * (t * (t + 1) // 2) * m["hq"] * m["hd"]          # scores and mix over the causal pairs
-    return m["layers"] * (per_layer + attn) + 2 * m["v"] * m["d"]   # the head runs for the last row only
+    attn = sum(4 * (n * (n + 1) // 2) * m["hq"] * m["hd"] for n in lengths)   # scores and mix, causal pairs
+    return m["layers"] * (per_layer + attn) + len(lengths) * 2 * m["v"] * m["d"]
 
 
 def decode_bytes(m, batch, lengths):
@@ -61,6 +71,90 @@ def decode_bytes(m, batch, lengths):
     weights = m["layers"] * m["layer_params"] * 2 + (m["v"] * m["d"] + m["d"]) * 2 + batch * m["d"] * 2
     kv = sum(lengths) * 2 * m["kvw"] * 2 * m["layers"]
     return weights + kv
+
+
+class OpTimer:
+    """Times the kernel calls of one step that runs kernel by kernel: every function of
+    ``sonicboom_amd.ops`` that launches is wrapped between two events on the stream, and the
+    times are summed by (function, what it worked on)."""
+
+    NAMES = ("embed", "rmsnorm", "gemm_bf16", "gemm_bf16_partial", "reduce_resid_norm", "rope_kv_store",
+             "attention", "argmax", "gemm_plain", "silu_mul", "add_into", "cast")
+
+    def __init__(self, m):
+        self.m, self.records, self._saved = m, [], {}
+
+    def _label(self, name, args, kw):
+        m = self.m
+        if name in ("gemm_bf16", "gemm_bf16_partial"):
+            n, k = kw.get("packed_shape") or (args[1].shape[0], args[1].shape[-1])
+            if kw.get("gated"):
+                return "gate_up"
+            return {(m["qw"] + 2 * m["kvw"], m["d"]): "qkv", (m["d"], m["qw"]): "out", (m["d"], m["ff"]): "down",
+                    (m["v"], m["d"]): "head"}.get((n, k), f"product_{n}x{k}")
+        return {"reduce_resid_norm": "add_slices_norm", "rope_kv_store": "rotate_store"}.get(name, name)
+
+    def __enter__(self):
+        import torch
+        from sonicboom_amd import ops
+        for name in self.NAMES:
+            fn = getattr(ops, name)
+            self._saved[name] = fn
+
+            def timed(*args, _fn=fn, _name=name, **kw):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                out = _fn(*args, **kw)
+                e1.record()
+                self.records.append((self._label(_name, args, kw), e0, e1))
+                return out
+            setattr(ops, name, timed)
+        return self
+
+    def __exit__(self, *exc):
+        from sonicboom_amd import ops
+        for name, fn in self._saved.items():
+            setattr(ops, name, fn)
+
+    def totals(self):
+        """label -> (microseconds, calls)"""
+        import torch
+        torch.cuda.synchronize()
+        out = {}
+        for label, e0, e1 in self.records:
+            us, n = out.get(label, (0.0, 0))
+            out[label] = (us + e0.elapsed_time(e1) * 1e3, n + 1)
+        return out
+
+
+def kernel_rates(m, totals, rows, kv_tokens, prefill_lengths=None):
+    """Achieved rates of the step's kernels from an OpTimer's totals: GB/s of the bytes each must
+    read for a decode step, TFLOP/s for a prompt step."""
+    L = m["layers"]
+    weights = {"qkv": m["d"] * (m["qw"] + 2 * m["kvw"]), "out": m["qw"] * m["d"], "gate_up": 2 * m["d"] * m["ff"],
+               "down": m["d"] * m["ff"]}
+    out = {}
+    for label, (us, calls) in sorted(totals.items()):
+        item = {"us": round(us, 1), "calls": calls}
+        if prefill_lengths is None:
+            if label in weights:
+                item["GB/s"] = round(weights[label] * 2 * calls / us / 1e3, 1)
+            elif label == "head":
+                item["GB/s"] = round(m["v"] * m["d"] * 2 * calls / us / 1e3, 1)
+            elif label == "attention":
+                item["GB/s"] = round(kv_tokens * 2 * m["kvw"] * 2 * calls / us / 1e3, 1)
+            if "GB/s" in item:
+                item["frac"] = round(item["GB/s"] / PEAK_HBM_GBS, 3)
+        else:
+            if label in weights:
+                item["TFLOP/s"] = round(2 * rows * weights[label] * calls / us / 1e6, 1)
+            elif label == "attention":
+                flops = sum(4 * (n * (n + 1) // 2) * m["hq"] * m["hd"] for n in prefill_lengths)
+                item["TFLOP/s"] = round(flops * calls / us / 1e6, 1)
+            if "TFLOP/s" in item:
+                item["frac"] = round(item["TFLOP/s"] * 1e12 / PEAK_FLOPS["bf16"], 3)
+        out[label] = item
+    return out
 
 
 def main() -> int:
@@ -74,8 +168,10 @@ def main() -> int:
     ap.add_argument("--sizes", choices=sorted(SIZES), default="7b", help="layer sizes (default: the benchmark's)")
     ap.add_argument("--prompt", type=int, default=PROMPT, help="cached prompt tokens per sequence")
     ap.add_argument("--context", type=int, default=CONTEXT, help="cache size per sequence")
+    ap.add_argument("--workload", choices=("steady", "mixed"), default="steady")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--no-graph", action="store_true", help="launch decode steps kernel by kernel")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel rates")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported")
@@ -84,8 +180,10 @@ def main() -> int:
     import numpy as np
     import torch
 
-    from sonicboom_amd.engine import DecoderModel, Engine, StepEntry
+    from sonicboom_amd import ops
+    from sonicboom_amd.engine import DecoderModel, Engine, StepEntry, generate
     from sonicboom_amd.engine.decode import DecodeLoop
+    from sonicboom_amd.sampling import SamplingParams
 
     PROMPT, CONTEXT = a.prompt, max(a.context, a.prompt + a.steps + a.warmup + 64)
     model_name, base_cfg = SIZES[a.sizes]
@@ -97,12 +195,25 @@ def main() -> int:
     t0 = time.time()
     model = DecoderModel.from_random(cfg, seed=0, dtype="bfloat16", device="cuda:0")
     torch.cuda.synchronize()
-    print(f"[bench] model of {cfg['num_hidden_layers']} layers ready in {time.time() - t0:.1f} s",
+    print(f"[bench] model of {cfg['num_hidden_layers']} layers ready in {time.time() - t0:.1f} s, "
+          f"{torch.cuda.max_memory_allocated() / 2**30:.1f} GiB at most on the device",
           file=sys.stderr, flush=True)
     rng = np.random.default_rng(0)
+    peak_measured = None if a.no_kernels else round(ops.read_bandwidth() / 1e9, 1)
 
-    def prompts(n):
-        return [[int(t) for t in rng.integers(0, cfg["vocab_size"], size=PROMPT)] for _ in range(n)]
+    def config(**more):
+        c = {
+            "model": f"{model_name} sizes, random bf16 weights", "layers": cfg["num_hidden_layers"],
+            "layers_of_configuration": full_layers, "hidden_size": m["d"], "num_attention_heads": m["hq"],
+            "num_key_value_heads": m["hkv"], "head_dim": m["hd"], "intermediate_size": m["ff"],
+            "vocab_size": m["v"], "rope_theta": cfg["rope_theta"], "rms_norm_eps": cfg["rms_norm_eps"],
+            "tie_word_embeddings": False, "parallelism": "single GPU", "decode_graph": not a.no_graph,
+        }
+        c.update(more)
+        return c
+
+    def random_prompts(lengths):
+        return [[int(t) for t in rng.integers(0, cfg["vocab_size"], size=n)] for n in lengths]
 
     def sync_time(fn):
         torch.cuda.synchronize()
@@ -111,74 +222,140 @@ def main() -> int:
         torch.cuda.synchronize()
         return time.perf_counter() - t
 
+    # ------------------------------------------------------------------------------------------
+    if a.workload == "mixed":
+        n_prompts, shortest, longest, n_steps, per_seq = MIXED[a.sizes]
+        lengths = [int(n) for n in rng.integers(shortest, longest + 1, size=n_prompts)]
+        prompts = random_prompts(lengths)
+        engine = Engine(model, max_tokens=per_seq * n_prompts)
+        engine.use_graphs = not a.no_graph
+        params = SamplingParams(max_tokens=n_steps)
+        marks = []
+
+        def run():
+            marks.clear()
+            t_start = time.perf_counter()
+
+            def first_token(i, t):
+                if not marks:
+                    marks.append(time.perf_counter())      # the prompt step and the first choice are done
+                return False
+            outs = generate(engine, prompts, params, stop_tokens=(), max_batch=n_prompts, callback=first_token)
+            torch.cuda.synchronize()
+            t_end = time.perf_counter()
+            assert all(len(o) == n_steps for o in outs)
+            return marks[0] - t_start, t_end - marks[0]
+
+        warm = generate(engine, [p[:64] for p in prompts], SamplingParams(max_tokens=4), stop_tokens=(),
+                        max_batch=n_prompts)          # compiles nothing, but pages in the kernels
+        del warm
+        runs = [run() for _ in range(3)]
+        prefill_s = statistics.median(r[0] for r in runs)
+        decode_s = statistics.median(r[1] for r in runs)
+        decoded = n_prompts * (n_steps - 1)           # the first token of each comes from the prompt step
+        step_s = decode_s / (n_steps - 1)
+        mean_lengths = [n + n_steps / 2 for n in lengths]
+        nbytes = decode_bytes(m, n_prompts, mean_lengths)
+        pf = prefill_flops(m, lengths)
+        line = {
+            "metric": f"decode tokens/s, {model_name} sizes, {n_prompts} prompts of {shortest}-{longest} tokens "
+                      f"in one batch, {n_steps} greedy steps through the generation loop",
+            "value": round(decoded / decode_s, 1), "unit": "tokens/s", "n_gpus": 1, "steps": n_steps - 1,
+            "warmup": 1, "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": config(global_batch=n_prompts, seq_len=per_seq, prompt_tokens=sum(lengths),
+                             shortest_prompt=min(lengths), longest_prompt=max(lengths)),
+            "prefill": {"value": round(sum(lengths) / prefill_s, 1), "tokens": sum(lengths),
+                        "ms": round(prefill_s * 1e3, 3), "frac": round(pf / prefill_s / PEAK_FLOPS["bf16"], 4)},
+            "roofline": {"bound": "hbm", "achieved": round(nbytes / step_s / 1e9, 1), "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": round(nbytes / step_s / 1e9 / PEAK_HBM_GBS, 4),
+                         "peak_measured": peak_measured, "bytes_per_step": int(nbytes)},
+            "runs": [{"prefill_ms": round(p * 1e3, 2), "decode_ms": round(d * 1e3, 2)} for p, d in runs],
+        }
+        print(json.dumps(line), flush=True)
+        return 0
+
     # ---- prefill of one prompt (2,048 tokens unless --prompt says otherwise) ----------------
     engine = Engine(model, max_tokens=CONTEXT)
     times = []
     for i in range(5):
-        p = prompts(1)[0]
+        p = random_prompts([PROMPT])[0]
         slot = engine.alloc_slot()
         times.append(sync_time(lambda: engine.step([StepEntry(slot, p, (PROMPT - 1,))])))
         engine.free_slot(slot)
     prefill_s = statistics.median(times[1:])
-    pf = prefill_flops(m, PROMPT)
+    pf = prefill_flops(m, [PROMPT])
     prefill = {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT, "ms": round(prefill_s * 1e3, 3),
                "frac": round(pf / prefill_s / PEAK_FLOPS["bf16"], 4)}
+    if not a.no_kernels:
+        slot = engine.alloc_slot()
+        with OpTimer(m) as timer:
+            engine.step([StepEntry(slot, random_prompts([PROMPT])[0], (PROMPT - 1,))])
+        engine.free_slot(slot)
+        prefill["kernels"] = kernel_rates(m, timer.totals(), PROMPT, 0, prefill_lengths=[PROMPT])
     print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
     del engine
 
     # ---- decode -----------------------------------------------------------------------------
-    def decode_run(batch, steps, warmup):
+    def decode_run(batch, steps, warmup, kernels=False):
         eng = Engine(model, max_tokens=CONTEXT * batch)
         loop = DecodeLoop(eng, use_graph=not a.no_graph)
         slots = [eng.alloc_slot() for _ in range(batch)]
-        ps = prompts(batch)
-        first = []
-        for i in range(0, batch, 8):            # prompts in steps of 8 sequences
-            logits = eng.step([StepEntry(s, p, (PROMPT - 1,)) for s, p in zip(slots[i:i + 8], ps[i:i + 8])])
-            first += torch.argmax(logits, dim=-1).tolist()
+        ps = random_prompts([PROMPT] * batch)
+        # the prompts in one step; the engine runs it in portions of its row limit
+        logits = eng.step([StepEntry(s, p, (PROMPT - 1,)) for s, p in zip(slots, ps)])
+        first = torch.argmax(logits, dim=-1).tolist()
         loop.start(slots, first)
         for _ in range(warmup):
             loop.step()
         torch.cuda.synchronize()
-        t = time.perf_counter()
+        per_step = []
+        t_all = time.perf_counter()
         for _ in range(steps):
-            loop.step()
+            t = time.perf_counter()
+            loop.step()                         # ends with the chosen tokens on the host
+            per_step.append(time.perf_counter() - t)
         torch.cuda.synchronize()
-        dt = (time.perf_counter() - t) / steps
+        mean = (time.perf_counter() - t_all) / steps
         lengths = [eng.length(s) for s in slots]
+        rates = None
+        if kernels:
+            plain = DecodeLoop(eng, use_graph=False)
+            plain.start(slots, loop.pending)
+            plain.step()
+            with OpTimer(m) as timer:
+                plain.step()
+            rates = kernel_rates(m, timer.totals(), batch, sum(lengths) + batch, None)
         loop.close()
         for s in slots:
             eng.free_slot(s)
         del eng
-        return dt, lengths
+        return statistics.median(per_step), mean, lengths, rates
 
-    step_s, lengths = decode_run(a.batch, a.steps, a.warmup)
+    step_s, mean_s, lengths, rates = decode_run(a.batch, a.steps, a.warmup, kernels=not a.no_kernels)
     value = a.batch / step_s
     nbytes = decode_bytes(m, a.batch, lengths)
     roofline = {"bound": "hbm", "achieved": round(nbytes / step_s / 1e9, 1), "peak": PEAK_HBM_GBS,
-                "unit": "GB/s", "frac": round(nbytes / step_s / 1e9 / PEAK_HBM_GBS, 4)}
-    print(f"[bench] decode b{a.batch}: {value:.1f} tok/s, {step_s * 1e3:.3f} ms/step, {roofline}",
-          file=sys.stderr, flush=True)
+                "unit": "GB/s", "frac": round(nbytes / step_s / 1e9 / PEAK_HBM_GBS, 4),
+                "peak_measured": peak_measured, "bytes_per_step": int(nbytes)}
+    if rates is not None:
+        roofline["kernels"] = rates
+    print(f"[bench] decode b{a.batch}: {value:.1f} tok/s, median {step_s * 1e3:.3f} ms/step "
+          f"(mean {mean_s * 1e3:.3f}), {roofline}", file=sys.stderr, flush=True)
     points = {}
     if not a.no_points:
         for b in (1, 64):
-            dt, _ = decode_run(b, max(8, a.steps // 2), max(2, a.warmup // 2))
+            dt, _, _, _ = decode_run(b, max(8, a.steps // 2), max(2, a.warmup // 2))
             points[f"decode_b{b}"] = round(b / dt, 1)
             print(f"[bench] decode b{b}: {points[f'decode_b{b}']} tok/s", file=sys.stderr, flush=True)
 
     line = {
         "metric": f"decode tokens/s, {model_name} sizes, batch {a.batch}, {PROMPT}-token cached prompts",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
-        "ms_per_step": round(step_s * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "ms_per_step": round(step_s * 1e3, 4), "ms_per_step_mean": round(mean_s * 1e3, 4),
+        "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {
-            "model": f"{model_name} sizes, random bf16 weights", "layers": cfg["num_hidden_layers"],
-            "layers_of_configuration": full_layers, "hidden_size": m["d"], "num_attention_heads": m["hq"],
-            "num_key_value_heads": m["hkv"], "head_dim": m["hd"], "intermediate_size": m["ff"],
-            "vocab_size": m["v"], "rope_theta": cfg["rope_theta"], "rms_norm_eps": cfg["rms_norm_eps"],
-            "tie_word_embeddings": False, "global_batch": a.batch, "seq_len": CONTEXT,
-            "cached_prompt_tokens": PROMPT, "parallelism": "single GPU", "decode_graph": not a.no_graph,
-        },
+        "config": config(global_batch=a.batch, seq_len=CONTEXT, cached_prompt_tokens=PROMPT),
         "prefill": prefill, "roofline": roofline, "points": points,
     }
     print(json.dumps(line), flush=True)

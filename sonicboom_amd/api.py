@@ -47,15 +47,19 @@ class Model:
     def vocab_size(self) -> int:
         return self.decoder.vocab
 
-    def session(self, max_tokens: int, max_slots: Optional[int] = None) -> "Session":
-        """A cache for at most ``max_tokens`` live tokens (each sequence rounded up to 64)."""
-        return Session(self, max_tokens, max_slots)
+    def session(self, max_tokens: int, max_slots: Optional[int] = None,
+                max_positions: Optional[int] = None) -> "Session":
+        """A cache for at most ``max_tokens`` live tokens (each sequence rounded up to 64).
+        ``max_positions`` bounds a sequence's length: None takes the model's own maximum of
+        positions, 0 sets no bound."""
+        return Session(self, max_tokens, max_slots, max_positions)
 
 
 class Session:
-    def __init__(self, model: Model, max_tokens: int, max_slots: Optional[int] = None):
+    def __init__(self, model: Model, max_tokens: int, max_slots: Optional[int] = None,
+                 max_positions: Optional[int] = None):
         self.model = model
-        self.engine = Engine(model.decoder, max_tokens, max_slots)
+        self.engine = Engine(model.decoder, max_tokens, max_slots, max_positions=max_positions)
 
     def alloc_slot(self) -> int:
         return self.engine.alloc_slot()

@@ -105,6 +105,7 @@ _ENTRIES = {
     "model_eos": lambda m: [int(t) for t in m.eos],
     "model_vocab": lambda m: int(m.vocab_size),
     "session_new": _session_new,
+    "session_vocab": lambda s: int(s.model.vocab_size),
     "slot_alloc": lambda s: int(s.alloc_slot()),
     "slot_free": lambda s, slot: s.free_slot(int(slot)),
     "step": _step,

@@ -12,15 +12,35 @@
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <unordered_set>
 #include <vector>
 
 struct boom_error { std::string message; };
-struct boom_llm_model { PyObject *obj; uint32_t magic; };
-struct boom_llm_session { PyObject *obj; boom_llm_model *model; uint32_t magic; };
+struct boom_llm_model { PyObject *obj; };
+// A session's Python object holds its model: the session outlives boom_llm_model_free of the
+// handle it was made from (/root/reference/capi/src/capi.cpp:2320-2350 keeps the model alive
+// the same way).
+struct boom_llm_session { PyObject *obj; };
 
 namespace {
 
-constexpr uint32_t kModelMagic = 0x4d4f444cu, kSessionMagic = 0x53455353u;
+// The handles that are alive.  A handle is looked up here before it is touched, so a freed or
+// made-up pointer is refused without being read (/root/reference/capi/src/capi.cpp:198-208).
+std::mutex g_handles_lock;
+std::unordered_set<const void *> g_models, g_sessions;
+
+bool known(const std::unordered_set<const void *> &set, const void *h) {
+  std::lock_guard<std::mutex> hold(g_handles_lock);
+  return h && set.count(h) != 0;
+}
+void remember(std::unordered_set<const void *> &set, const void *h) {
+  std::lock_guard<std::mutex> hold(g_handles_lock);
+  set.insert(h);
+}
+bool forget(std::unordered_set<const void *> &set, const void *h) {
+  std::lock_guard<std::mutex> hold(g_handles_lock);
+  return h && set.erase(h) != 0;
+}
 
 boom_status fail(boom_error **slot, boom_status st, const std::string &msg) {
   if (slot) {
@@ -145,15 +165,16 @@ const char *dtype_of(const boom_llm_load_options *o) {
 int device_of(const boom_llm_load_options *o) {
   return (o && o->struct_size >= offsetof(boom_llm_load_options, device) + sizeof(o->device)) ? o->device : 0;
 }
-bool live(const boom_llm_model *m) { return m && m->magic == kModelMagic && m->obj; }
-bool live(const boom_llm_session *s) { return s && s->magic == kSessionMagic && s->obj; }
+bool live(const boom_llm_model *m) { return known(g_models, m); }
+bool live(const boom_llm_session *s) { return known(g_sessions, s); }
 
 boom_status wrap_model(PyObject *obj, boom_llm_model **out, boom_error **err) {
-  boom_llm_model *m = new (std::nothrow) boom_llm_model{obj, kModelMagic};
+  boom_llm_model *m = new (std::nothrow) boom_llm_model{obj};
   if (!m) {
     Py_DECREF(obj);
     return fail(err, BOOM_ERR_INTERNAL, "out of memory");
   }
+  remember(g_models, m);
   *out = m;
   return BOOM_OK;
 }
@@ -188,11 +209,9 @@ boom_status boom_llm_model_random(const char *config_json_path, uint64_t seed, c
 }
 
 void boom_llm_model_free(boom_llm_model *model) {
-  if (!live(model)) return;
+  if (!forget(g_models, model)) return;      // NULL, made up, or freed before
   Gil gil;
   Py_DECREF(model->obj);
-  model->obj = nullptr;
-  model->magic = 0;
   delete model;
 }
 
@@ -251,21 +270,20 @@ boom_status boom_llm_session_new(boom_llm_model *model, uint64_t max_tokens, boo
   const boom_status st =
       bridge("session_new", Py_BuildValue("(OK)", model->obj, (unsigned long long)max_tokens), &obj, err_out);
   if (st != BOOM_OK) return st;
-  boom_llm_session *s = new (std::nothrow) boom_llm_session{obj, model, kSessionMagic};
+  boom_llm_session *s = new (std::nothrow) boom_llm_session{obj};
   if (!s) {
     Py_DECREF(obj);
     return fail(err_out, BOOM_ERR_INTERNAL, "out of memory");
   }
+  remember(g_sessions, s);
   *session_out = s;
   return BOOM_OK;
 }
 
 void boom_llm_session_free(boom_llm_session *session) {
-  if (!live(session)) return;
+  if (!forget(g_sessions, session)) return;
   Gil gil;
   Py_DECREF(session->obj);
-  session->obj = nullptr;
-  session->magic = 0;
   delete session;
 }
 
@@ -294,7 +312,7 @@ boom_status boom_llm_step(boom_llm_session *session, const boom_llm_step_entry *
   uint32_t vocab = 0;
   {
     PyObject *res = nullptr;
-    const boom_status st = bridge("model_vocab", Py_BuildValue("(O)", session->model->obj), &res, err_out);
+    const boom_status st = bridge("session_vocab", Py_BuildValue("(O)", session->obj), &res, err_out);
     if (st != BOOM_OK) return st;
     vocab = (uint32_t)PyLong_AsUnsignedLong(res);
     Py_DECREF(res);
@@ -333,6 +351,10 @@ boom_status boom_llm_generate(boom_llm_session *session, const boom_token *const
   boom_llm_sampling sp;
   std::memset(&sp, 0, sizeof sp);
   std::memcpy(&sp, sampling, sampling->struct_size < sizeof sp ? sampling->struct_size : sizeof sp);
+  // A struct too short to hold repeat_last_n gets the default window of 64; a 0 the caller wrote
+  // is an empty window and switches every penalty off (/root/reference/capi/src/capi.cpp:2651-2653).
+  if (sampling->struct_size < offsetof(boom_llm_sampling, repeat_last_n) + sizeof(sp.repeat_last_n))
+    sp.repeat_last_n = 64;
   if (sampling->struct_size < offsetof(boom_llm_sampling, max_tokens) + sizeof(sp.max_tokens))
     return fail(err_out, BOOM_ERR_BINDING, "boom_llm_generate: sampling.struct_size does not reach max_tokens");
   if (sp.temperature < 0.f) return fail(err_out, BOOM_ERR_BINDING, "boom_llm_generate: temperature must be >= 0");
@@ -349,7 +371,7 @@ boom_status boom_llm_generate(boom_llm_session *session, const boom_token *const
       "{s:f,s:f,s:I,s:K,s:I,s:f,s:f,s:I,s:f,s:f}", "temperature", sp.temperature, "top_p",
       (sp.top_p == 0.f ? 1.f : sp.top_p), "top_k", sp.top_k, "seed", (unsigned long long)sp.seed, "max_tokens",
       sp.max_tokens, "min_p", sp.min_p, "repeat_penalty", (sp.repeat_penalty == 0.f ? 1.f : sp.repeat_penalty),
-      "repeat_last_n", (sp.repeat_last_n == 0 ? 64u : sp.repeat_last_n), "presence_penalty", sp.presence_penalty,
+      "repeat_last_n", sp.repeat_last_n, "presence_penalty", sp.presence_penalty,
       "frequency_penalty", sp.frequency_penalty);
   PyObject *stops;
   if (stop) {

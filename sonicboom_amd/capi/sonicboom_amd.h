@@ -62,7 +62,7 @@ typedef struct boom_llm_sampling {
   uint32_t max_tokens;     /* tokens to produce per prompt */
   float min_p;
   float repeat_penalty;
-  uint32_t repeat_last_n;  /* 0 reads as 64 */
+  uint32_t repeat_last_n;  /* window of the penalties; 0: empty, no penalty applies; 64 when struct_size ends before it */
   float presence_penalty;
   float frequency_penalty;
 } boom_llm_sampling;

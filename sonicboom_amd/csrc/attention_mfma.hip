@@ -26,7 +26,7 @@
 // ascending order.  It depends on positions only, not on the batch.
 #include <type_traits>
 
-#include "mfma.cuh"
+#include "mfma.h"
 
 #ifndef SB_HEAD_DIM
 #error "compile with -DSB_HEAD_DIM=<head size>"

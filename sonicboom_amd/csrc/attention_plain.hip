@@ -16,7 +16,7 @@
 // ascending key, so the arithmetic of a row is a function of its position and
 // window alone: it does not change with the batch, with the cut of the prompt
 // into steps or with the physical pages.
-#include "common.cuh"
+#include "common.h"
 
 namespace {
 

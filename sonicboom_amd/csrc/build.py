@@ -40,7 +40,7 @@ CORE_SOURCES = [
     "status.hip", "embed_norm.hip", "elementwise.hip", "gemm_plain.hip", "rope_kv.hip",
     "attention_plain.hip", "sampling.hip", "gemm_skinny.hip", "gemm_stream.hip", "gemm_mfma.hip",
 ]
-HEADERS = ["common.cuh", "sb_hip.h", "mfma.cuh"]
+HEADERS = ["common.h", "sb_hip.h", "mfma.h"]
 ATTN_SOURCES = ["attention_mfma.hip"]
 
 # Head sizes compiled ahead of time by build_all(): every size the kernels take.

@@ -3,7 +3,7 @@
 // silu(g) = g / (1 + expf(-g)) with the full-precision expf, then the product
 // with the up projection (/root/reference/core/src/nn/activation.cpp:41-50,
 // /root/reference/core/src/model/emit.cpp:364-374).
-#include "common.cuh"
+#include "common.h"
 
 namespace {
 

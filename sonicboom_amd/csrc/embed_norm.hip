@@ -4,7 +4,7 @@
 // scale), /root/reference/core/src/nn/norm.cpp:25-42 (eps inside the root,
 // product order (x*inv)*w).  The mean of squares is accumulated in double, as
 // the reference's default reduction does (/root/reference/core/src/nn/cpu_reduce.h:55-57).
-#include "common.cuh"
+#include "common.h"
 
 namespace {
 
@@ -61,8 +61,8 @@ __device__ __forceinline__ void write_normed(TO *yr, const float4 &v, int g, flo
 // unconditionally (from a clamped address) so that all are in flight together, and the groups
 // stay in registers for the second pass.  Rows wider than 4 * KEEP * THREADS, or not readable in
 // groups of four, go through the scalar tail loops.  Few rows: 1024 threads keeping two groups
-// each, to have the row's loads in flight at once; many rows: 256 threads keeping four, so
-// that eight rows share a CU.
+// each, to have the row's loads in flight at once; many rows of bfloat16 output: 256 threads
+// keeping four, so that eight rows share a CU.
 template <typename TO, int kNormThreads, int kNormKeep>
 __global__ void __launch_bounds__(kNormThreads)
 rmsnorm_kernel(TO *__restrict__ y, const float *__restrict__ x, const void *__restrict__ w,
@@ -231,10 +231,12 @@ extern "C" int sb_rmsnorm(void *y, int out_dtype, const float *x, const void *w,
   SB_REQUIRE(eps >= 0.0f, "sb_rmsnorm: eps must not be negative");
   if (n_rows == 0) return SB_OK;
   hipStream_t s = (hipStream_t)stream;
+  // The two block shapes sum a row's squares in different orders.  Float output is the true
+  // 32-bit path, whose rows must not change by a bit with the number of rows that share the
+  // launch: it keeps one shape.  bfloat16 output takes the faster shape for many rows.
   const bool many = n_rows >= 256;
   if (out_dtype == SB_F32) {
-    if (many) rmsnorm_kernel<float, 256, 4><<<n_rows, 256, 0, s>>>((float *)y, x, w, w_dtype, rows, width, eps);
-    else rmsnorm_kernel<float, 1024, 2><<<n_rows, 1024, 0, s>>>((float *)y, x, w, w_dtype, rows, width, eps);
+    rmsnorm_kernel<float, 1024, 2><<<n_rows, 1024, 0, s>>>((float *)y, x, w, w_dtype, rows, width, eps);
   } else {
     if (many) rmsnorm_kernel<bf16_t, 256, 4><<<n_rows, 256, 0, s>>>((bf16_t *)y, x, w, w_dtype, rows, width, eps);
     else rmsnorm_kernel<bf16_t, 1024, 2><<<n_rows, 1024, 0, s>>>((bf16_t *)y, x, w, w_dtype, rows, width, eps);

@@ -18,7 +18,7 @@
 // their X rows and neighbouring W rows.
 #include <type_traits>
 
-#include "mfma.cuh"
+#include "mfma.h"
 
 namespace {
 

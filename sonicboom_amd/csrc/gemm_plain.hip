@@ -9,7 +9,7 @@
 // projection weight (/root/reference/core/include/sonicboom/quant/quantized_matmul.h:74-77);
 // the bias is added after the product and the residual after the bias
 // (/root/reference/core/src/model/emit.cpp:260-261, :447).
-#include "common.cuh"
+#include "common.h"
 
 namespace {
 

@@ -13,7 +13,7 @@
 //
 // MFMA roles: A = 16 rows of W, B = 16 rows of X, D[n][t]; a lane then holds
 // four consecutive n of one t, a 16-byte store.
-#include "mfma.cuh"
+#include "mfma.h"
 
 namespace {
 

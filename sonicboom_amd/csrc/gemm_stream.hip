@@ -20,7 +20,7 @@
 //
 // MFMA roles: A = 16 rows of W, B = 16 rows of X, D[n][t]; a lane holds four
 // consecutive n of one t.
-#include "mfma.cuh"
+#include "mfma.h"
 
 namespace {
 

@@ -9,7 +9,7 @@
 // whatever that rule is; only the D layout shapes the epilogues.
 #pragma once
 
-#include "common.cuh"
+#include "common.h"
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));

@@ -8,7 +8,7 @@
 // rotation in float.  The bias has been added before
 // (/root/reference/core/src/model/emit.cpp:252-254); values are not rotated;
 // the key is cached after its rotation (emit.cpp:291-293).
-#include "common.cuh"
+#include "common.h"
 
 namespace {
 

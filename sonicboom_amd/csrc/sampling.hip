@@ -7,7 +7,7 @@
 // and the single-rounding fma form for the sampled path (:77-104); candidates
 // are z = l/T as one float division, the 256 largest by (z descending, id
 // ascending) (:257-285).  The filters and the Gumbel draw run on the host.
-#include "common.cuh"
+#include "common.h"
 
 #include <mutex>
 

@@ -1,5 +1,5 @@
 // The error slot and the build description of the kernel library.
-#include "common.cuh"
+#include "common.h"
 
 namespace sb {
 char *error_slot() {

@@ -130,6 +130,8 @@ class DecodeLoop:
             if not 0 <= t < vocab:
                 raise StepError(f"token id {t} is outside the vocabulary of {vocab}")
         ones = [1] * len(self.slots)
+        for slot in self.slots:
+            eng.check_positions(slot, 1)
         try:
             cache.reserve(self.slots, ones)
         except CacheError as e:

@@ -91,6 +91,12 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = 
     outputs: List[List[int]] = [[] for _ in prompts]
     if params.max_tokens == 0 or not prompts:
         return outputs
+    # a bound on positions (the model's own unless the engine was given another; 0 = none): a prompt
+    # beyond it is refused, a sequence that reaches it ends there
+    max_positions = int(getattr(engine, "max_positions", 0) or 0)
+    for i, p in enumerate(prompts):
+        if max_positions and len(p) > max_positions:
+            raise ValueError(f"request {i}: a prompt of {len(p)} tokens passes the model's {max_positions} positions")
     batches = plan_batches([len(p) for p in prompts], params.max_tokens, engine.cache.n_pages, max_batch,
                            engine.cache.max_slots)
     loop = engine.decode_loop() if hasattr(engine, "decode_loop") else None
@@ -111,7 +117,8 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = 
                     else:
                         s.out.append(t)
                         s.history.append(t)
-                        ended = t in stop or len(s.out) >= params.max_tokens
+                        ended = t in stop or len(s.out) >= params.max_tokens or \
+                            (max_positions > 0 and len(s.history) > max_positions)
                     if ended:
                         outputs[s.index] = s.out
                         engine.free_slot(s.slot)

@@ -9,7 +9,7 @@ import torch
 from ..cache.paged import GroupSpec, PagedCache, group_entries
 from ..config.registry import architecture_of, load_config
 from ..parts import ModelSpec, Runtime, build_part
-from ..weights import load_tensors, random_tensors
+from ..weights import open_tensors, random_source
 
 DTYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16}
 
@@ -82,8 +82,11 @@ class DecoderModel:
         arch, cfg = load_config(folder)          # configuration errors first: they need no GPU
         spec = arch.build_spec(cfg)
         dev = require_gpu(device)
-        tensors = load_tensors(folder, spec, dtype, dev)
-        return cls(spec, tensors, Runtime(dev, DTYPES[dtype], fast_kernels), cfg)
+        tensors = open_tensors(folder, spec, dtype, dev)      # read as the parts ask for them
+        try:
+            return cls(spec, tensors, Runtime(dev, DTYPES[dtype], fast_kernels), cfg)
+        finally:
+            tensors.close()
 
     @classmethod
     def from_random(cls, config, seed: int, dtype: str = "bfloat16", device=None, fast_kernels: bool = True):
@@ -93,7 +96,7 @@ class DecoderModel:
         cfg = arch.config_class.from_dict(d)
         spec = arch.build_spec(cfg)
         dev = require_gpu(device)
-        tensors = random_tensors(spec, seed, dtype, dev)
+        tensors = random_source(spec, seed, dtype, dev)       # drawn as the parts ask for them
         return cls(spec, tensors, Runtime(dev, DTYPES[dtype], fast_kernels), cfg)
 
     # ---- cache -----------------------------------------------------------------

@@ -21,6 +21,33 @@ from .model import DecoderModel
 
 
 ROW_TILE = 16      # rows of one sequence that the attention kernels take together
+# Rows that run as one batch.  More than this and a step runs in portions: the tiled products
+# are at their best rate from a few thousand rows on, and their operands (rows x inner width,
+# two bytes each) must stay below 4 GiB.
+MAX_STEP_ROWS = 16384
+
+
+def portion_rows(n_new: Sequence[int], limit: int):
+    """Cut a step of ``n_new[i]`` rows per sequence into portions of at most ``limit`` rows:
+    a list of portions, each a list of (sequence, first row, end row).  Sequences stay in
+    order and a sequence's rows ascend over the portions; a sequence is cut only where a
+    portion is full."""
+    if limit <= 0:
+        raise ValueError("the row limit of a step must be positive")
+    portions, cur, room = [], [], limit
+    for i, n in enumerate(n_new):
+        a = 0
+        while a < n:
+            b = min(n, a + room)
+            cur.append((i, a, b))
+            room -= b - a
+            a = b
+            if room == 0:
+                portions.append(cur)
+                cur, room = [], limit
+    if cur:
+        portions.append(cur)
+    return portions
 
 
 class StepError(ValueError):
@@ -97,8 +124,14 @@ class StepContext:
 class Engine:
     """A model with its cache: slots, the step function, and the device."""
 
-    def __init__(self, model: DecoderModel, max_tokens: int, max_slots: Optional[int] = None):
+    def __init__(self, model: DecoderModel, max_tokens: int, max_slots: Optional[int] = None,
+                 max_step_rows: int = MAX_STEP_ROWS, max_positions: Optional[int] = None):
+        """``max_positions``: the longest sequence a step accepts; None takes the model's own
+        bound (its configuration's maximum of positions), 0 sets none."""
         self.model = model
+        self.max_step_rows = int(max_step_rows)
+        own = int(getattr(model.spec, "max_positions", 0) or 0)
+        self.max_positions = own if max_positions is None else int(max_positions)
         self.device = model.rt.device
         self.cache = model.new_cache(max_tokens, max_slots)
         self.bindings = model.bindings(self.cache)
@@ -137,9 +170,25 @@ class Engine:
             for w in e.want:
                 if not 0 <= w < n:
                     raise StepError(f"slot {e.slot}: wanted row {w} is not among the {n} tokens of this step")
+            self.check_positions(e.slot, n)
+
+    def check_positions(self, slot: int, n_new: int) -> None:
+        """Refuse ``n_new`` more tokens of ``slot`` when they pass the bound on positions."""
+        if self.max_positions > 0:
+            try:
+                after = self.cache.length(slot) + n_new
+            except CacheError as e:
+                raise StepError(str(e)) from None
+            if after > self.max_positions:
+                raise StepError(f"slot {slot}: {after} tokens pass the model's {self.max_positions} positions")
 
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
-        """Run the entries' tokens; float32 logits [wanted rows, vocab] on the device."""
+        """Run the entries' tokens; float32 logits [wanted rows, vocab] on the device.
+
+        A step of more than ``max_step_rows`` rows runs in portions, one after the other from
+        the cache the earlier ones left: whole sequences while they fit, a sequence cut where
+        the portion is full.  The logits come back in the order of the entries and of their
+        ``want`` all the same."""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
         try:
             self._check(entries)
@@ -148,9 +197,27 @@ class Engine:
             self.cache.reserve(slots, n_new)
         except CacheError as e:
             raise StepError(str(e)) from None
-        ctx = StepContext(self.cache, entries, self.device)
-        logits = self.forward(ctx)
-        self.cache.advance(slots, n_new)
+        portions = portion_rows(n_new, self.max_step_rows)
+        if len(portions) == 1:
+            ctx = StepContext(self.cache, entries, self.device)
+            logits = self.forward(ctx)
+            self.cache.advance(slots, n_new)
+            return logits
+        pieces, place = [], []          # place[i] = (entry, index in its want) of output row i
+        for portion in portions:
+            sub = []
+            for i, a, b in portion:
+                e = entries[i]
+                picked = [(k, w - a) for k, w in enumerate(e.want) if a <= w < b]
+                sub.append(StepEntry(e.slot, e.tokens[a:b], [w for _, w in picked]))
+                place += [(i, k) for k, _ in picked]
+            ctx = StepContext(self.cache, sub, self.device)
+            pieces.append(self.forward(ctx))
+            self.cache.advance([e.slot for e in sub], [len(e.tokens) for e in sub])
+        logits = torch.cat(pieces, dim=0)
+        order = sorted(range(len(place)), key=place.__getitem__)
+        if order != list(range(len(place))):
+            logits = logits[torch.tensor(order, dtype=torch.long, device=logits.device)]
         return logits
 
     def forward(self, ctx) -> torch.Tensor:

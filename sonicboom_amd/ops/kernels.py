@@ -271,6 +271,25 @@ def top_candidates(logits: torch.Tensor, temperature: float, k: int = MAX_CANDID
     return ids, z
 
 
+def read_bandwidth(n_bytes: int = 1 << 30, blocks: int = 512, repeats: int = 5, device="cuda:0") -> float:
+    """Bytes a second that a plain streaming read of ``n_bytes`` reaches on this GPU (the best of
+    ``repeats`` passes over a buffer that the caches do not hold): what "achievable" means beside
+    the published peak in a bandwidth report."""
+    n_bytes = max(16, n_bytes // 16 * 16)
+    src = torch.zeros((n_bytes // 4,), dtype=torch.int32, device=device)
+    sink = torch.zeros((4,), dtype=torch.int32, device=device)
+    lib = library.core()
+    best = 0.0
+    for _ in range(repeats + 1):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        check(lib.sb_read_probe(_p(sink), _p(src), n_bytes, int(blocks), _stream()))
+        e1.record()
+        e1.synchronize()
+        best = max(best, n_bytes / (e0.elapsed_time(e1) * 1e-3))
+    return best
+
+
 # --------------------------------------------------------------------------
 # dispatch between the plain kernels and the MFMA kernels
 # --------------------------------------------------------------------------

@@ -97,6 +97,8 @@ def core():
                 lib.sb_gemm_skinny_scratch.restype = c_size_t
                 lib.sb_top_candidates_scratch.argtypes = [_I, _I]
                 lib.sb_top_candidates_scratch.restype = c_size_t
+                lib.sb_read_probe.argtypes = [_P, _P, _Z, _I, _P]
+                lib.sb_read_probe.restype = c_int
                 lib._sb_path = path
                 _core = lib
     return _core

@@ -101,25 +101,87 @@ def _to_torch(raw: np.ndarray, file_dtype: str, kind: str, mode: str) -> torch.T
     return t if mode == "float32" else t.to(torch.bfloat16)
 
 
-def load_tensors(folder: str, spec: ModelSpec, dtype: str, device) -> Dict[str, torch.Tensor]:
-    """All tensors ``spec`` names, on ``device``; raises :class:`WeightError`
-    listing every missing, unexpected and ill-shaped tensor."""
+class LazyTensors:
+    """name -> tensor, made when it is first asked for and kept until it is popped.
+
+    A model is built part by part; each part packs its tensors into the layout its kernels read
+    and the model pops the originals.  Making a tensor only when its part asks for it keeps one
+    part's worth of originals alive at a time, on the host and on the device, whatever the
+    model's size.  ``get``, ``pop``, ``in`` and ``keys`` are what the builders use of a dict."""
+
+    def __init__(self, names, make, close=None):
+        self._names = set(names)
+        self._make = make
+        self._close = close
+        self._kept: Dict[str, torch.Tensor] = {}
+
+    def get(self, name, default=None):
+        if name in self._kept:
+            return self._kept[name]
+        if name not in self._names:
+            return default
+        t = self._kept[name] = self._make(name)
+        return t
+
+    def __getitem__(self, name):
+        t = self.get(name)
+        if t is None:
+            raise KeyError(name)
+        return t
+
+    def __contains__(self, name):
+        return name in self._names
+
+    def pop(self, name, default=None):
+        self._names.discard(name)
+        return self._kept.pop(name, default)
+
+    def keys(self):
+        return sorted(self._names)
+
+    def materialize(self) -> Dict[str, torch.Tensor]:
+        return {name: self.get(name) for name in self.keys()}
+
+    def close(self) -> None:
+        if self._close is not None:
+            self._close()
+            self._close = None
+        self._names = set(self._kept)
+
+
+def open_tensors(folder: str, spec: ModelSpec, dtype: str, device) -> LazyTensors:
+    """The tensors ``spec`` names, read from the folder's files one by one as they are asked for
+    and put on ``device``.  Everything is checked first: raises :class:`WeightError` listing every
+    missing, unexpected, ill-shaped and ill-typed tensor.  ``close()`` the result when the model
+    is built."""
     if dtype not in ("float32", "bfloat16"):
         raise ValueError(f"dtype must be float32 or bfloat16, not {dtype}")
     owner = open_files(folder)
-    try:
-        wanted = spec.all_tensors()
-        found = {name: (sf.tensors[name].dtype, sf.tensors[name].shape) for name, sf in owner.items()}
-        problems = check_against_spec(found, wanted, spec.ignorable_tensors)
-        if problems:
-            raise WeightError(f"{folder}: {len(problems)} problem(s) with the weights\n" + "\n".join(problems))
-        out = {}
-        for t in wanted:
-            sf = owner.get(t.name)
-            if sf is None:
-                continue
-            out[t.name] = _to_torch(sf.raw(t.name), sf.tensors[t.name].dtype, t.kind, dtype).to(device)
-        return out
-    finally:
+
+    def close():
         for sf in set(owner.values()):
             sf.close()
+    try:
+        wanted = {t.name: t for t in spec.all_tensors()}
+        found = {name: (sf.tensors[name].dtype, sf.tensors[name].shape) for name, sf in owner.items()}
+        problems = check_against_spec(found, list(wanted.values()), spec.ignorable_tensors)
+        if problems:
+            raise WeightError(f"{folder}: {len(problems)} problem(s) with the weights\n" + "\n".join(problems))
+    except BaseException:
+        close()
+        raise
+
+    def make(name):
+        sf, t = owner[name], wanted[name]
+        return _to_torch(sf.raw(name), sf.tensors[name].dtype, t.kind, dtype).to(device)
+    return LazyTensors([n for n in wanted if n in owner], make, close)
+
+
+def load_tensors(folder: str, spec: ModelSpec, dtype: str, device) -> Dict[str, torch.Tensor]:
+    """All tensors ``spec`` names, on ``device``; raises :class:`WeightError`
+    listing every missing, unexpected and ill-shaped tensor."""
+    source = open_tensors(folder, spec, dtype, device)
+    try:
+        return source.materialize()
+    finally:
+        source.close()

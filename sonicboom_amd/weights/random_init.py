@@ -70,19 +70,29 @@ def write_random_model(folder: str, config, seed: int, dtype: str = "bfloat16",
     return spec
 
 
-def random_tensors(spec: ModelSpec, seed: int, dtype: str, device) -> Dict[str, torch.Tensor]:
-    """The spec's tensors drawn on ``device`` with torch's generator (a different
-    stream of numbers than the folder writer's, same distributions)."""
+def random_source(spec: ModelSpec, seed: int, dtype: str, device):
+    """The spec's tensors drawn on ``device`` as they are asked for (a model of 145 GB is then
+    built block by block without its row-major weights ever standing whole beside the packed
+    ones).  Tensor number i of the spec comes from torch's generator seeded by (seed, i): the
+    values do not depend on the order of asking.  Another stream of numbers than the folder
+    writer's, the same distributions."""
+    from .loader import LazyTensors
     tdt = torch.float32 if dtype == "float32" else torch.bfloat16
-    gen = torch.Generator(device=device)
-    gen.manual_seed(int(seed))
-    out = {}
-    for t in spec.all_tensors():
+    specs = {t.name: (i, t) for i, t in enumerate(spec.all_tensors())}
+
+    def make(name):
+        i, t = specs[name]
         if t.kind == "int":
-            out[t.name] = torch.zeros(t.shape, dtype=torch.int32, device=device)
-            continue
+            return torch.zeros(t.shape, dtype=torch.int32, device=device)
+        gen = torch.Generator(device=device)
+        gen.manual_seed((int(seed) * 1000003 + i) & (2**63 - 1))
         mean, std = t.init
         a = torch.empty(t.shape, dtype=torch.float32, device=device)
         a.normal_(mean, std, generator=gen)
-        out[t.name] = a.to(tdt)
-    return out
+        return a.to(tdt)
+    return LazyTensors(specs, make)
+
+
+def random_tensors(spec: ModelSpec, seed: int, dtype: str, device) -> Dict[str, torch.Tensor]:
+    """All of :func:`random_source` at once, as a dict."""
+    return random_source(spec, seed, dtype, device).materialize()

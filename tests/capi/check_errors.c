@@ -30,6 +30,15 @@ int main(void) {
   CHECK(boom_llm_model_arch(NULL, NULL, 0, &n, &err) == BOOM_ERR_INTERNAL);
   CHECK(boom_llm_session_new(NULL, 64, NULL, &err) == BOOM_ERR_INTERNAL);
   CHECK(boom_llm_step(NULL, NULL, 0, NULL, 0, &n, &err) == BOOM_ERR_INTERNAL);
+  /* pointers that were never handed out are refused without being read */
+  {
+    uint32_t vocab = 0;
+    int32_t slot = 0;
+    CHECK(boom_llm_model_vocab((const boom_llm_model *)(uintptr_t)0x10, &vocab, &err) == BOOM_ERR_INTERNAL);
+    CHECK(boom_llm_slot_alloc((boom_llm_session *)(uintptr_t)0x10, &slot, &err) == BOOM_ERR_INTERNAL);
+    boom_llm_model_free((boom_llm_model *)(uintptr_t)0x10);
+    boom_llm_session_free((boom_llm_session *)(uintptr_t)0x10);
+  }
   boom_llm_model_free(NULL);
   boom_llm_session_free(NULL);
   CHECK(strcmp(boom_error_message(NULL), "") == 0);

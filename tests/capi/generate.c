@@ -2,6 +2,7 @@
  * generation with a callback that cuts one prompt short (the refused token is not reported).
  * Prints what it got, one item a line, for the Python test to compare with the package's own
  * results. */
+#include <stddef.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -50,6 +51,10 @@ int main(int argc, char **argv) {
 
   boom_llm_session *session = NULL;
   MUST(boom_llm_session_new(model, 512, &session, &err));
+  /* the session keeps its model alive: the model handle is given back before any step */
+  boom_llm_model_free(model);
+  if (boom_llm_model_vocab(model, &vocab, &err) != BOOM_ERR_INTERNAL) return 7;   /* a freed handle is refused */
+  boom_llm_model_free(model);                                                      /* twice: ignored */
 
   /* one step: two sequences of unequal length, logits at three places */
   int32_t s0 = -1, s1 = -1;
@@ -92,6 +97,23 @@ int main(int argc, char **argv) {
     for (uint32_t j = 0; j < counts[i]; ++j) printf(" %d", out[i * 6 + j]);
     printf("\n");
   }
+  /* a penalty with an explicit empty window penalises nothing; a struct that ends before
+   * repeat_last_n gets the window of 64 and does */
+  sp.repeat_penalty = 5.0f;
+  sp.repeat_last_n = 0;
+  boom_token out2[18];
+  uint32_t counts2[3];
+  MUST(boom_llm_generate(session, prompts, lens, 3, &sp, no_stop, 0, NULL, NULL, out2, counts2, &err));
+  printf("empty window %s\n", (counts2[0] == 6 && memcmp(out2, out, 6 * sizeof(boom_token)) == 0) ? "same" : "differs");
+  sp.struct_size = offsetof(boom_llm_sampling, repeat_last_n);
+  sp.repeat_last_n = 12345;                     /* not read: beyond struct_size */
+  MUST(boom_llm_generate(session, prompts, lens, 3, &sp, no_stop, 0, NULL, NULL, out2, counts2, &err));
+  printf("short struct:");
+  for (uint32_t j = 0; j < counts2[0]; ++j) printf(" %d", out2[j]);
+  printf("\n");
+  sp.struct_size = sizeof sp;
+  sp.repeat_penalty = 0.0f;
+  sp.repeat_last_n = 0;
   /* sampled, seeded */
   sp.temperature = 0.8f;
   sp.seed = 7;
@@ -105,7 +127,8 @@ int main(int argc, char **argv) {
   free(logits);
   free(arch);
   boom_llm_session_free(session);
-  boom_llm_model_free(model);
+  if (boom_llm_slot_alloc(session, &s0, &err) != BOOM_ERR_INTERNAL) return 8;      /* a freed session is refused */
+  boom_llm_session_free(session);
   boom_error_free(err);
   printf("ok\n");
   return 0;

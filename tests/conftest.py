@@ -68,5 +68,45 @@ def model_folders(tmp_path_factory):
     return out
 
 
+# Random N(0, 0.02) weights give attention scores near 0.03: the softmax is almost uniform and a
+# wrong scale, rope base, bias or position moves the logits by less than bfloat16's rounding.
+# The "sharp" folders hold the same models with the query and key projections times SHARP_QK and
+# their biases times SHARP_QK_BIAS (a bias of N(0, 0.02) is an eighth of what the projection of a
+# normed row gives; the larger factor makes it a third), which spreads the scores over several
+# units so that such mistakes show (tests/test_plain.py::test_sharp_models_show_attention_mistakes
+# measures by how much).
+SHARP_QK = 10.0
+SHARP_QK_BIAS = 30.0
+
+
+def sharpen_model(src: str, dst: str, factor: float = SHARP_QK, bias_factor: float = SHARP_QK_BIAS) -> None:
+    """Copy the model folder ``src`` to ``dst`` with q_proj and k_proj (weights and biases) scaled."""
+    import shutil
+
+    import torch
+    from safetensors import safe_open
+    from safetensors.torch import save_file
+    os.makedirs(dst, exist_ok=True)
+    shutil.copy(os.path.join(src, "config.json"), os.path.join(dst, "config.json"))
+    tensors = {}
+    with safe_open(os.path.join(src, "model.safetensors"), framework="pt") as f:
+        for name in f.keys():
+            t = f.get_tensor(name)
+            if ".q_proj." in name or ".k_proj." in name:
+                t = (t.float() * (bias_factor if name.endswith(".bias") else factor)).to(t.dtype)
+            tensors[name] = t.contiguous()
+    save_file(tensors, os.path.join(dst, "model.safetensors"), metadata={"format": "pt"})
+
+
+@pytest.fixture(scope="session")
+def sharp_folders(model_folders, tmp_path_factory):
+    """name -> folder of the same tiny model with attention scores of several units."""
+    out = {}
+    for name in ("A", "B", "C"):
+        out[name] = str(tmp_path_factory.mktemp(f"sharp_{name}"))
+        sharpen_model(model_folders[name], out[name])
+    return out
+
+
 def random_prompt(rng: np.random.Generator, vocab: int, n: int):
     return [int(t) for t in rng.integers(0, vocab, size=n)]

@@ -12,9 +12,15 @@ _PLAIN_MODELS = {}
 _PLAIN_LOGITS = {}
 
 
-def plain_model(folder):
+def plain_model(folder, wide=False):
+    """The plain implementation's (configuration, weights) of a folder.  ``wide`` keeps the
+    matrices in float64 (the same values: every float32 is one), which spares the plain products
+    their conversion at every call; it pays for models of real layer sizes."""
     if folder not in _PLAIN_MODELS:
-        _PLAIN_MODELS[folder] = qwen2_plain.load_model(folder)
+        cfg, w = qwen2_plain.load_model(folder)
+        if wide:
+            w = {k: (v.astype(np.float64) if v.ndim == 2 else v) for k, v in w.items()}
+        _PLAIN_MODELS[folder] = (cfg, w)
     return _PLAIN_MODELS[folder]
 
 
@@ -27,20 +33,46 @@ def plain_logits(folder, tokens):
     return _PLAIN_LOGITS[key]
 
 
-# Tolerances, fixed: float32 differs from the plain implementation by the
-# rounding of float32 sums (the plain one sums in float64); bfloat16 by the
-# rounding of activations to 8 bits of mantissa at every part's boundary.
-TOL = {"float32": dict(atol=5e-5, rtol=5e-5), "bfloat16": dict(atol=3e-2, rtol=3e-2)}
+def forget_plain(folder):
+    """Drop what is cached for a folder (large models)."""
+    _PLAIN_MODELS.pop(folder, None)
+    for key in [k for k in _PLAIN_LOGITS if k[0] == folder]:
+        del _PLAIN_LOGITS[key]
 
 
-def assert_logits_close(got, want, dtype, what=""):
+# Tolerances, fixed.  float32 differs from the plain implementation by the rounding of float32
+# sums (the plain one sums in float64).  bfloat16 rounds activations to 8 bits of mantissa at
+# every part's boundary; what that does to a logit is measured against the spread of the logits
+# (their standard deviation), not against 1, and in two ways: no logit may be off by more than
+# a fraction of the spread plus a fraction of itself, and the root mean square of all differences,
+# which rounding keeps small and a systematic mistake does not, has a tighter bound of its own.
+# On the "sharp" models (conftest.SHARP_QK) scores of ten and more make the softmax amplify the
+# rounding of queries and keys: measured on the GPU the largest difference was 0.23 spreads and
+# the root mean square 0.021, against 0.018 and 0.004 on the models of plain random weights.
+F32_TOL = dict(atol=5e-5, rtol=5e-5)
+BF16_MAX = {False: 0.04, True: 0.5}       # largest difference, in spreads (plus BF16_REL * |logit|)
+BF16_RMS = {False: 0.01, True: 0.05}      # root mean square of the differences, in spreads
+BF16_REL = 0.02
+
+
+def bf16_limits(want, sharp=False):
+    """(bound on every |difference|, bound on their root mean square) for logits ``want``."""
+    want = np.asarray(want, dtype=np.float64)
+    spread = float(want.std())
+    return BF16_MAX[sharp] * spread + BF16_REL * np.abs(want), BF16_RMS[sharp] * spread
+
+
+def assert_logits_close(got, want, dtype, what="", sharp=False):
     got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
     assert got.shape == want.shape, f"{what}: shape {got.shape} vs {want.shape}"
     assert np.isfinite(got).all(), f"{what}: logits are not finite"
-    tol = TOL[dtype]
-    scale = max(1.0, float(np.abs(want).max()))
     err = np.abs(got - want)
-    bound = tol["atol"] * scale + tol["rtol"] * np.abs(want)
+    if dtype == "float32":
+        bound = F32_TOL["atol"] * max(1.0, float(np.abs(want).max())) + F32_TOL["rtol"] * np.abs(want)
+    else:
+        bound, rms_bound = bf16_limits(want, sharp)
+        rms = float(np.sqrt((err ** 2).mean())) if err.size else 0.0
+        assert rms <= rms_bound, f"{what}: root mean square difference {rms:.3g} > {rms_bound:.3g}"
     if not (err <= bound).all():
         i = np.unravel_index(np.argmax(err - bound), err.shape)
         raise AssertionError(f"{what}: logits differ at {i}: got {got[i]:.6g}, want {want[i]:.6g} "

@@ -42,6 +42,30 @@ def test_failures_are_statuses_with_messages(tmp_path):
     assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stdout + r.stderr
 
 
+def test_host_code_under_the_sanitizers(tmp_path):
+    """capi.cpp and the command line built with ASan and UBSan (host code only, no GPU): the
+    failure paths, made-up handles and the command line's argument errors run clean."""
+    from sonicboom_amd.capi import build
+    lib, cmd, san_env = build.build_sanitized()
+    exe = str(tmp_path / "check_errors_san")
+    r = subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-O1", "-g", "-fsanitize=address,undefined",
+                        os.path.join(HERE, "check_errors.c"), f"-I{CAPI}", f"-L{os.path.dirname(lib)}",
+                        "-lsonicboom_amd", f"-Wl,-rpath,{os.path.dirname(lib)}", "-o", exe],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    env = dict(os.environ, SONICBOOM_AMD_ROOT=ROOT, **san_env)
+    env.pop("LD_PRELOAD", None)           # ASan's runtime has to come first in the list of libraries
+    r = subprocess.run([exe], capture_output=True, text=True, env=env, timeout=600)
+    assert r.returncode == 0 and r.stdout.strip().endswith("ok"), r.stdout + r.stderr
+    assert "runtime error" not in r.stderr and "AddressSanitizer" not in r.stderr, r.stderr
+    tokens = tmp_path / "p.txt"
+    tokens.write_text("1 2 3\n")
+    r = subprocess.run([cmd, "-m", str(tmp_path / "nowhere"), "--tokens", str(tokens)], capture_output=True,
+                       text=True, env=env, timeout=600)
+    assert r.returncode == 1 and "config.json" in r.stderr
+    assert "runtime error" not in r.stderr and "AddressSanitizer" not in r.stderr, r.stderr
+
+
 def test_command_line_usage_and_errors(tmp_path):
     from sonicboom_amd.capi import build
     _, cmd = build.build()
@@ -89,6 +113,9 @@ def test_a_c_program_gets_what_the_package_gives(tmp_path, model_folders, dtype)
     outs = session.generate(prompts, max_tokens=6, stop_tokens=[], callback=cb)
     assert len(outs[1]) == 2          # the callback refused the third token: it is not reported
     want += [f"greedy {i}:" + "".join(f" {t}" for t in o) for i, o in enumerate(outs)]
+    want.append("empty window same")
+    pen = session.generate(prompts, max_tokens=6, stop_tokens=[], repeat_penalty=5.0, repeat_last_n=64)
+    want.append("short struct:" + "".join(f" {t}" for t in pen[0]))
     outs = session.generate(prompts, max_tokens=6, stop_tokens=[], temperature=0.8, seed=7, top_k=40)
     want += [f"sampled {i}:" + "".join(f" {t}" for t in o) for i, o in enumerate(outs)]
     want.append("ok")

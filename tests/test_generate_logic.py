@@ -139,3 +139,25 @@ def test_plan_batches():
         plan_batches([5, 300], 8, n_pages=4, max_batch=64)
     with pytest.raises(ValueError, match="empty prompt"):
         plan_batches([0], 8, n_pages=4, max_batch=64)
+
+
+def test_portions_of_a_long_step():
+    """A step above the row limit is cut into portions: sequences in order, a sequence cut only
+    where a portion is full, every row exactly once."""
+    from sonicboom_amd.engine.step import portion_rows
+    assert portion_rows([3, 4], 10) == [[(0, 0, 3), (1, 0, 4)]]
+    assert portion_rows([10], 10) == [[(0, 0, 10)]]
+    assert portion_rows([11], 10) == [[(0, 0, 10)], [(0, 10, 11)]]
+    # the second sequence starts in the first portion's last two rows and ends in the third
+    assert portion_rows([8, 14, 1], 10) == [[(0, 0, 8), (1, 0, 2)], [(1, 2, 12)], [(1, 12, 14), (2, 0, 1)]]
+    rng = np.random.default_rng(3)
+    for _ in range(200):
+        n_new = [int(n) for n in rng.integers(1, 40, size=rng.integers(1, 9))]
+        limit = int(rng.integers(1, 50))
+        portions = portion_rows(n_new, limit)
+        assert all(sum(b - a for _, a, b in p) <= limit for p in portions)
+        assert all(sum(b - a for _, a, b in p) == limit for p in portions[:-1])      # only the last is short
+        flat = [(i, r) for p in portions for i, a, b in p for r in range(a, b)]
+        assert flat == [(i, r) for i, n in enumerate(n_new) for r in range(n)]
+    with pytest.raises(ValueError):
+        portion_rows([3], 0)

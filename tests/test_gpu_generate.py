@@ -173,7 +173,8 @@ def test_long_decoding_token_by_token_from_the_first_token(model_folders, dtype)
     from sonicboom_amd.engine import StepEntry
     folder = model_folders["B"]
     a, b = prompts_for("B", [260, 200], seed=8)
-    eng = model_for(folder, dtype).session(max_tokens=64 * 10).engine
+    # 260 tokens: past tiny B's 256 positions on purpose
+    eng = model_for(folder, dtype).session(max_tokens=64 * 10, max_positions=0).engine
     sa, sb = eng.alloc_slot(), eng.alloc_slot()
     got_a, got_b = [], []
     out = eng.step([StepEntry(sa, a[:1], [0]), StepEntry(sb, b[:70], range(70))]).cpu().numpy()
@@ -206,10 +207,35 @@ def test_step_errors(model_folders):
     with pytest.raises(StepError, match="not in use"):
         eng.step([StepEntry(99, [1], [0])])
     with pytest.raises(StepError, match="out of cache pages"):
-        eng.step([StepEntry(s, [1] * 200, [0])])
+        eng.step([StepEntry(s, [1] * 70, [0]), StepEntry(eng.alloc_slot(), [1] * 70, [0])])
     assert eng.step([StepEntry(s, [1, 2, 3], [])]).shape == (0, 256)     # nothing wanted
     assert eng.length(s) == 3
     eng.free_slot(s)
+    # the model's own bound on positions (tiny A: 128), unless the session lifts it
+    eng = model_for(model_folders["A"], "float32").session(max_tokens=64 * 4).engine
+    s = eng.alloc_slot()
+    eng.step([StepEntry(s, [1] * 127, [])])
+    eng.step([StepEntry(s, [1], [])])
+    with pytest.raises(StepError, match="128 positions"):
+        eng.step([StepEntry(s, [1], [0])])
+    loop = eng.decode_loop()
+    loop.start([s], [1])
+    with pytest.raises(StepError, match="128 positions"):
+        loop.step()
+    assert eng.length(s) == 128
+    eng.free_slot(s)
+
+
+def test_generation_ends_at_the_bound_on_positions(model_folders):
+    session = model_for(model_folders["A"], "float32").session(max_tokens=64 * 4)
+    prompts = prompts_for("A", [120, 10], seed=4)
+    out = session.generate(prompts, max_tokens=20, stop_tokens=())
+    assert [len(o) for o in out] == [9, 20]          # 120 + 9 = 129 tokens: the last one is never fed
+    free = model_for(model_folders["A"], "float32").session(max_tokens=64 * 4, max_positions=0)
+    longer = free.generate(prompts, max_tokens=20, stop_tokens=())
+    assert longer[0][:9] == out[0] and len(longer[0]) == 20
+    with pytest.raises(ValueError, match="128 positions"):
+        session.generate([[1] * 129], max_tokens=2)
 
 
 def test_command_line(model_folders, tmp_path):

@@ -221,6 +221,128 @@ def test_bias_precedes_rotation(models):
     assert abs(s[4, 2] - s[4, 3]) > 1e-7                                         # another distance differs
 
 
+def _zero_qk_bias(w, prefix):
+    w = dict(w)
+    for r in ("q_proj", "k_proj", "v_proj"):
+        w[prefix + r + ".bias"] = np.zeros_like(w[prefix + r + ".bias"])
+    return w
+
+
+def test_self_attention_default_scale_is_the_library_routines(models):
+    """P.self_attention itself (not a scale passed in by the test) against torch's
+    scaled_dot_product_attention with its default scale, 1/sqrt(head size): biases zero, and the
+    rotation frozen by a linear position scaling of 1e30 (every angle is 0), so what is left is
+    projections, causal grouped attention and the output projection.  A scale of 1, of
+    1/head size or of 1/sqrt(width) fails this."""
+    for name in ("A", "B"):
+        cfg, w = models[name]
+        cfg = dict(cfg, rope_scaling={"type": "linear", "factor": 1e30})
+        hq, hkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["_head_dim"]
+        p = "model.layers.1.self_attn."
+        w = _zero_qk_bias(w, p)
+        n = 11
+        # activations large enough for scores of a few units: a wrong scale then matters
+        h = (rng(12).standard_normal((n, cfg["hidden_size"])) * 12.0).astype(F32)
+        got = P.self_attention(h, np.arange(n), w, p, cfg)
+        hh = torch.from_numpy(h).double()
+        q, k, v = (hh @ torch.from_numpy(w[p + r + ".weight"]).double().T for r in ("q_proj", "k_proj", "v_proj"))
+        q = q.view(n, hq, hd).transpose(0, 1)
+        k = k.view(n, hkv, hd).transpose(0, 1).repeat_interleave(hq // hkv, dim=0)
+        v = v.view(n, hkv, hd).transpose(0, 1).repeat_interleave(hq // hkv, dim=0)
+        a = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True)
+        want = a.transpose(0, 1).reshape(n, hq * hd) @ torch.from_numpy(w[p + "o_proj.weight"]).double().T
+        assert np.allclose(got, want.numpy(), atol=2e-5), name
+        wrong = torch.nn.functional.scaled_dot_product_attention(q, k, v, is_causal=True, scale=1.0)
+        wrong = wrong.transpose(0, 1).reshape(n, hq * hd) @ torch.from_numpy(w[p + "o_proj.weight"]).double().T
+        assert np.abs(wrong.numpy() - want.numpy()).max() > 1e-2, "the case cannot tell the scales apart"
+
+
+def test_self_attention_rotates_after_the_bias(models):
+    """Through P.self_attention, with zero q and k matrices: queries and keys are rotated
+    biases, so the score of (row m, key n) is scale * sum over pairs of
+    (qa ka + qb kb) cos(t (m - n)) + (qa kb - qb ka) sin(t (m - n)) with the biases' halves a, b:
+    a function of the distance.  Biases added after the rotation would give every pair of rows
+    the same score, and the output would be the causal running mean of the values."""
+    cfg, w = models["A"]
+    hq, hkv, hd = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["_head_dim"]
+    half, group = hd // 2, hq // hkv
+    p = "model.layers.0.self_attn."
+    w = dict(w)
+    w[p + "q_proj.weight"] = np.zeros_like(w[p + "q_proj.weight"])
+    w[p + "k_proj.weight"] = np.zeros_like(w[p + "k_proj.weight"])
+    r = rng(13)
+    w[p + "q_proj.bias"] = r.standard_normal(hq * hd).astype(F32) * F32(1.5)
+    w[p + "k_proj.bias"] = r.standard_normal(hkv * hd).astype(F32) * F32(1.5)
+    n = 9
+    h = r.standard_normal((n, cfg["hidden_size"])).astype(F32) * F32(5.0)
+    got = P.self_attention(h, np.arange(n), w, p, cfg)
+    # the closed form, in float64
+    theta = float(cfg["rope_theta"]) ** (-2.0 * np.arange(half) / hd)
+    bq = w[p + "q_proj.bias"].astype(np.float64).reshape(hq, hd)
+    bk = w[p + "k_proj.bias"].astype(np.float64).reshape(hkv, hd)
+    v = (h.astype(np.float64) @ w[p + "v_proj.weight"].astype(np.float64).T + w[p + "v_proj.bias"]).reshape(n, hkv, hd)
+    out = np.zeros((n, hq, hd))
+    for hh in range(hq):
+        g = hh // group
+        qa, qb, ka, kb = bq[hh, :half], bq[hh, half:], bk[g, :half], bk[g, half:]
+        for m in range(n):
+            d = m - np.arange(m + 1)
+            s = ((qa * ka + qb * kb)[None, :] * np.cos(d[:, None] * theta[None, :])
+                 + (qa * kb - qb * ka)[None, :] * np.sin(d[:, None] * theta[None, :])).sum(-1) / math.sqrt(hd)
+            e = np.exp(s - s.max())
+            out[m, hh] = (e / e.sum()) @ v[: m + 1, g]
+    want = out.reshape(n, hq * hd) @ w[p + "o_proj.weight"].astype(np.float64).T
+    assert np.allclose(got, want, atol=2e-5)
+    mean = np.cumsum(v, axis=0) / np.arange(1, n + 1)[:, None, None]
+    mean = np.repeat(mean, group, axis=1).reshape(n, hq * hd) @ w[p + "o_proj.weight"].astype(np.float64).T
+    assert np.abs(mean - want).max() > 1e-2, "the case cannot tell the orders apart"
+    # only distances count: all positions shifted, same output
+    assert np.allclose(P.self_attention(h, np.arange(n) + 37, w, p, cfg), got, atol=1e-5)
+
+
+def test_sharp_models_show_attention_mistakes(models, sharp_folders):
+    """What the engine's bfloat16 comparisons can see.  A wrong attention scale (1 for
+    1/sqrt(head size) and the like: times 4), a rope base ten times too big, a dropped query bias
+    and positions that slip by one each move the plain logits of the "sharp" models by several
+    times what the bfloat16 comparisons allow there, in the largest difference and in the root
+    mean square; on the models of plain N(0, 0.02) weights most of them hide below the bounds."""
+    from helpers import bf16_limits
+    mistakes = ("scale", "base", "bias", "position")
+
+    def moved(c, ww, tokens, what, sharp):
+        base = P.forward(c, ww, tokens)
+        c2, w2 = dict(c), dict(ww)
+        att, rope = P.attention, P.rope_neox
+        try:
+            if what == "scale":
+                P.attention = lambda q, k, v, qp, kp, a, b, hd, scale, **kw: att(q, k, v, qp, kp, a, b, hd,
+                                                                                 scale * 4.0, **kw)
+            elif what == "base":
+                c2["rope_theta"] = c["rope_theta"] * 10.0
+            elif what == "bias":
+                for key in w2:
+                    if key.endswith("q_proj.bias"):
+                        w2[key] = np.zeros_like(w2[key])
+            elif what == "position":
+                P.rope_neox = lambda x, pos, *a, **kw: rope(x, [q + (1 if q % 7 == 3 else 0) for q in pos], *a, **kw)
+            diff = np.abs(P.forward(c2, w2, tokens) - base)
+        finally:
+            P.attention, P.rope_neox = att, rope
+        bound, rms_bound = bf16_limits(base, sharp)
+        return float((diff / bound).max()), float(np.sqrt((diff ** 2).mean())) / rms_bound
+
+    for name in ("A", "B"):
+        cfg, w = P.load_model(sharp_folders[name])
+        tokens = [int(t) for t in rng(14).integers(0, cfg["vocab_size"], size=65)]
+        for what in mistakes:
+            by_max, by_rms = moved(cfg, w, tokens, what, True)
+            assert by_max > 2.0 and by_rms > 3.0, \
+                f"sharp {name}: a wrong {what} is {by_max:.2f} bounds at its largest, {by_rms:.2f} in the mean"
+        soft_cfg, soft_w = models[name]
+        hidden = [what for what in mistakes if max(moved(soft_cfg, soft_w, tokens, what, False)) < 1.0]
+        assert hidden, "the models of plain random weights were expected to hide some of these mistakes"
+
+
 def test_head_choice_and_causality(models):
     cfg_a, w_a = models["A"]                    # tied: the head is the embedding
     cfg_b, w_b = models["B"]                    # untied

@@ -190,3 +190,31 @@ def test_command_writes_a_model_folder(tmp_path, tiny_configs):
     cfg_path.write_text(json.dumps(bad))
     r = subprocess.run(cmd + [str(cfg_path), str(tmp_path / "c")], capture_output=True, text=True)
     assert r.returncode == 1 and "hidden_size" in r.stderr
+
+
+def test_tensors_are_read_as_they_are_asked_for(model_folders, tiny_configs):
+    """open_tensors checks everything first, then reads a tensor when a part asks for it and
+    forgets it when the model pops it; the values are load_tensors' own."""
+    from sonicboom_amd.weights import open_tensors, random_source
+    folder = model_folders["B"]
+    spec = build_spec(Qwen2Config.from_dict(tiny_configs["B"]))
+    whole = load_tensors(folder, spec, "bfloat16", "cpu")
+    src = open_tensors(folder, spec, "bfloat16", "cpu")
+    assert src.keys() == sorted(whole) and not src._kept
+    name = "model.layers.1.mlp.down_proj.weight"
+    assert name in src and "no.such.tensor" not in src and src.get("no.such.tensor") is None
+    t = src.get(name)
+    assert torch.equal(t, whole[name]) and src.get(name) is t and list(src._kept) == [name]
+    assert src.pop(name) is t and name not in src and src.pop(name, None) is None
+    with pytest.raises(KeyError):
+        src["model.layers.9.mlp.down_proj.weight"]
+    src.close()
+    # drawn on demand: any order of asking gives the same values
+    a, b = random_source(spec, 3, "float32", "cpu"), random_source(spec, 3, "float32", "cpu")
+    names = a.keys()
+    for n in names:
+        a.get(n)
+    for n in reversed(names):
+        b.get(n)
+    assert all(torch.equal(a.get(n), b.get(n)) for n in names)
+    assert not torch.equal(a.get(names[0]), random_source(spec, 4, "float32", "cpu").get(names[0]))
