@@ -836,8 +836,6 @@ attn_decode_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ par
                 first, last, seq, heads_q, kvh, ht, group);
 }
 
-int g_force_nc = 0, g_force_waves = 0, g_force_ppw = 0;
-
 int check_common(const void *out, const void *q, const void *k, const void *v, const void *pt,
                  const void *row_pos, int max_pages, int n_pages_total, int heads_q, int heads_kv,
                  int window, const char *who) {
@@ -876,7 +874,8 @@ extern "C" size_t sb_attn_decode_part_ml(int n_seqs, int heads_q, int heads_kv, 
 extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
                                    const int32_t *page_table, int max_pages, int n_pages_total,
                                    const int32_t *row_pos, float *part_o, float *part_ml, int n_seqs,
-                                   int heads_q, int heads_kv, float scale, int window, void *stream) {
+                                   int heads_q, int heads_kv, float scale, int window, int pages_per_wave,
+                                   void *stream) {
   int rc = check_common(out, q, k_cache, v_cache, page_table, row_pos, max_pages, n_pages_total, heads_q,
                         heads_kv, window, "sb_attn_decode_bf16");
   if (rc != SB_OK) return rc;
@@ -891,10 +890,7 @@ extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache
   SB_SUPPORT(heads_kv * head_tiles <= 65535, "sb_attn_decode_bf16: too many heads");
   // A wave takes one page and asks for all of it at once (one round trip to memory), or, when
   // two pages per wave still leave a block for every CU, several pages in a row with half a page
-  // in flight while the half before it is multiplied (measured on cold caches, Qwen2.5-7B heads: 64
-  // sequences of 2,060 keys 53 us in one chunk, 65 with eight pages per wave and two chunks, 82
-  // with one page per wave; 8 sequences of 16,400 keys 57 with eight pages per wave against 79
-  // with one; one sequence of 32,780 keys 33 against 43).
+  // in flight while the half before it is multiplied.
   const long long per_chunk = (long long)heads_kv * head_tiles * n_seqs;
   int ppw = 1;
   if (HD <= 128 && (long long)((max_pages + 7) / 8) * per_chunk >= 256) {
@@ -923,7 +919,8 @@ extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache
       if (best < 0.0 || t < best) best = t, ppw = c;
     }
   }
-  if (g_force_ppw > 0 && (g_force_ppw == 1 || HD <= 128)) ppw = g_force_ppw;
+  // a test's or a measurement's choice (0: the launcher's own)
+  if (pages_per_wave > 0 && (pages_per_wave == 1 || HD <= 128)) ppw = pages_per_wave;
   const int pages_per_chunk = kPagesPerChunk * ppw;
   const int n_chunks = (max_pages + pages_per_chunk - 1) / pages_per_chunk;
   SB_SUPPORT((long long)n_chunks * per_chunk <= 0x7fffffffLL, "sb_attn_decode_bf16: too many blocks");
@@ -950,12 +947,6 @@ extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache
   return sb::check_launch("sb_attn_decode_bf16 (merge)");
 }
 
-// Measurement hook: pages per wave of the decode kernel (0: chosen from the sizes).
-extern "C" void sb_attn_decode_force(int ppw) { g_force_ppw = ppw > 0 ? ppw : 0; }
-
-// Measurement hook: heads per wave and waves per block in prefill (0: chosen from the group size).
-extern "C" void sb_attn_prefill_force(int nc, int waves) { g_force_nc = nc; g_force_waves = waves; }
-
 // q, out: bf16 [n_rows, heads_q * HD]; tiles int32 [n_tiles][4] = (first row, rows <= 16, sequence, 0),
 // every tile inside one sequence and its rows at consecutive positions.
 extern "C" int sb_attn_prefill_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
@@ -973,11 +964,9 @@ extern "C" int sb_attn_prefill_bf16(void *out, const void *q, const void *k_cach
   // waves cover the group, eight of them (two per SIMD) when the group is big enough to use them,
   // as far as the accumulators fit the registers.
   int waves = (group >= 5 && group <= 8 && HD <= 128) ? 8 : 4;
-  if (g_force_waves == 4) waves = 4;
   int nc = (group + waves - 1) / waves;
   const int nc_max = waves == 8 ? 1 : (DT <= 4 ? 4 : (DT <= 12 ? 2 : 1));
   if (nc > nc_max) nc = nc_max;
-  if (g_force_nc > 0 && g_force_nc <= nc_max) nc = g_force_nc;
   const int head_tiles = (group + nc - 1) / nc;
   const int y_per_kv = (head_tiles + waves - 1) / waves;
   SB_SUPPORT((long long)n_tiles * heads_kv * y_per_kv <= 0x7fffffffLL, "sb_attn_prefill_bf16: too many blocks");

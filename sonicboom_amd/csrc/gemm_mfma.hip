@@ -316,7 +316,6 @@ gemm_mfma_kernel(Args a) {
 }
 
 constexpr int kCus = 256;
-int g_force_variant = -1;
 
 template <int MT, int NW, int BK, int DEPTH, int GATED, bool PACKED, bool EVEN_K>
 int launch_one(const Args &a, long long blocks, hipStream_t s) {
@@ -385,7 +384,7 @@ int pick_shape(int n_rows, int n_out, int gated) {
 // in the packed tile layout.
 extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,
                                  int bias_dtype, const float *resid, int n_rows, int n_out, int n_in,
-                                 int gated, int packed, void *stream) {
+                                 int gated, int packed, int tile_shape, void *stream) {
   SB_REQUIRE(y && x && w, "sb_gemm_mfma_bf16: null pointer");
   SB_REQUIRE(n_rows >= 0 && n_out > 0 && n_in > 0, "sb_gemm_mfma_bf16: bad sizes rows=%d out=%d in=%d",
              n_rows, n_out, n_in);
@@ -402,7 +401,7 @@ extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void
   a.n_rows = n_rows; a.n_out = n_out; a.n_in = n_in; a.gated = gated ? 1 : 0;
   a.partial = nullptr; a.stages_per_slice = 0;
   int variant = pick_shape(n_rows, n_out, a.gated);
-  if (g_force_variant >= 0 && g_force_variant < 3) variant = g_force_variant;
+  if (tile_shape >= 0 && tile_shape < 3) variant = tile_shape;      // a test's or a measurement's choice
   if (!packed) variant = 0;       // the bigger tiles are built for packed weights only
   const int bm = kShapes[variant].bm, bn = gated ? kShapes[variant].bn / 2 : kShapes[variant].bn;
   a.tiles_m = (n_rows + bm - 1) / bm;
@@ -480,6 +479,3 @@ extern "C" int sb_gemm_mfma_partial_bf16(float *partial, const void *x, const vo
   return sb::check_launch("sb_gemm_mfma_partial_bf16");
 }
 
-// Measurement hook: -1 lets the launcher choose; 0, 1, 2 force the 128 x 128, 256 x 128 and
-// 256 x 256 tiles.
-extern "C" void sb_gemm_mfma_force(int variant) { g_force_variant = variant; }

@@ -224,7 +224,6 @@ namespace {
 struct Plan {
   int R, TT, n_slices, steps_per_slice;
 };
-int g_force_r = 0, g_force_slices = 0;   // measurement hooks, see sb_gemm_skinny_force
 Plan plan_for(int n_rows, int n_out, int n_in, int gated) {
   Plan p;
   p.TT = n_rows <= 16 ? 1 : (n_rows <= 32 ? 2 : 4);
@@ -242,7 +241,6 @@ Plan plan_for(int n_rows, int n_out, int n_in, int gated) {
     p.R = gated ? 2 : 4;
     want_blocks = 224;
   }
-  if (g_force_r) p.R = g_force_r;
   const int blocks = (tiles + p.R - 1) / p.R;
   int slices = 1;
   if (blocks < want_blocks) {
@@ -252,19 +250,11 @@ Plan plan_for(int n_rows, int n_out, int n_in, int gated) {
     if (slices > 8) slices = 8;     // what the kernels that add the slices take
     if (slices < 1) slices = 1;
   }
-  if (g_force_slices) slices = g_force_slices;
   p.steps_per_slice = (n_steps + slices - 1) / slices;
   p.n_slices = (n_steps + p.steps_per_slice - 1) / p.steps_per_slice;
   return p;
 }
 }  // namespace
-
-// For measurements: fix the rows-tiles per block (1, 2, 4; 0 = choose) and the number of K
-// slices over the grid (0 = choose) of every later call.
-extern "C" void sb_gemm_skinny_force(int r, int slices) {
-  g_force_r = r;
-  g_force_slices = slices;
-}
 
 extern "C" size_t sb_gemm_skinny_scratch(int n_rows, int n_out, int n_in, int gated) {
   if (n_rows <= 0 || n_out <= 0 || n_in <= 0) return 0;

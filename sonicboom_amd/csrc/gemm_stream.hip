@@ -200,11 +200,14 @@ void launch_w(const bf16_t *x, const bf16_t *w, const StreamArgs &a, hipStream_t
   kern<<<dim3((tiles + per_block - 1) / per_block, slices), 64 * W, lds, s>>>(x, w, a);
 }
 
-int g_force_waves = 0;   // measurement hook, see sb_gemm_stream_force
+// A call's hint (for tests and measurements; 0 = the launcher chooses): bits 0..7 the waves per
+// block (4..8), bits 8..15 the K slices the partial form aims at (1..8).
+inline int hint_waves(int hint) { return hint & 0xff; }
+inline int hint_slices(int hint) { return (hint >> 8) & 0xff; }
 
 // Waves per block: the count whose blocks fill whole rounds over the CUs best; more waves on a tie.
-int waves_for(int tiles, int r) {
-  if (g_force_waves >= 4 && g_force_waves <= 8) return g_force_waves;
+int waves_for(int tiles, int r, int force_waves) {
+  if (force_waves >= 4 && force_waves <= 8) return force_waves;
   constexpr int n_cu = 256;   // MI355X
   int best = 4;
   long long best_cost = -1;
@@ -225,17 +228,17 @@ struct Cut {
   int waves, slices, steps_per_slice;
 };
 inline int row_tiles(int n_rows) { return n_rows <= 16 ? 1 : (n_rows <= 32 ? 2 : (n_rows <= 64 ? 4 : 8)); }
-int g_force_slices = 0;
-Cut cut_for(int tiles, int n_steps, int tt) {
+Cut cut_for(int tiles, int n_steps, int tt, int hint) {
+  const int force_waves = hint_waves(hint), force_slices = hint_slices(hint);
   constexpr int n_cu = 256;   // MI355X
   Cut best{4, 1, (n_steps + kAhead - 1) / kAhead * kAhead};
   long long best_cost = -1;
   for (int want = 1; want <= 8; ++want) {
-    if (g_force_slices && want != g_force_slices) continue;
+    if (force_slices && want != force_slices) continue;
     const int sps = ((n_steps + want - 1) / want + kAhead - 1) / kAhead * kAhead;
     const int slices = (n_steps + sps - 1) / sps;
     for (int w = 4; w <= 8; ++w) {
-      if (g_force_waves >= 4 && g_force_waves <= 8 && w != g_force_waves) continue;
+      if (force_waves >= 4 && force_waves <= 8 && w != force_waves) continue;
       const long long blocks = (long long)((tiles + w - 1) / w) * slices;
       const long long cost = (blocks + n_cu - 1) / n_cu * (sps + 24) * (2 * w + tt) + 12LL * slices;
       if (best_cost < 0 || cost < best_cost) best = Cut{w, slices, sps}, best_cost = cost;
@@ -256,8 +259,8 @@ void launch_cut(const bf16_t *x, const bf16_t *w, const StreamArgs &a, int waves
 }
 
 template <int TT, int G, int R>
-void launch(const bf16_t *x, const bf16_t *w, const StreamArgs &a, hipStream_t s) {
-  switch (waves_for((a.n_out + 15) / 16, R)) {
+void launch(const bf16_t *x, const bf16_t *w, const StreamArgs &a, int hint, hipStream_t s) {
+  switch (waves_for((a.n_out + 15) / 16, R, hint_waves(hint))) {
     case 4: return launch_w<TT, G, R, 4>(x, w, a, s);
     case 5: return launch_w<TT, G, R, 5>(x, w, a, s);
     case 6: return launch_w<TT, G, R, 6>(x, w, a, s);
@@ -268,11 +271,6 @@ void launch(const bf16_t *x, const bf16_t *w, const StreamArgs &a, hipStream_t s
 
 }  // namespace
 
-// For measurements: waves per block of every later call (4..8; 0 = choose).
-extern "C" void sb_gemm_stream_force(int waves) { g_force_waves = waves; }
-// ... and the K slices sb_gemm_stream_partial_bf16 aims at (1..8; 0 = choose).
-extern "C" void sb_gemm_stream_force_slices(int slices) { g_force_slices = slices; }
-
 // Rows of X this kernel takes.
 extern "C" int sb_gemm_stream_max_rows(void) { return 128; }
 
@@ -281,7 +279,7 @@ extern "C" int sb_gemm_stream_max_rows(void) { return 128; }
 // tile layout (16 x 32 tiles of 1 KB in fragment order, tiles of a row block consecutive in k).
 extern "C" int sb_gemm_stream_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,
                                    int bias_dtype, const float *resid, int n_rows, int n_out, int n_in,
-                                   int gated, void *stream) {
+                                   int gated, int hint, void *stream) {
   SB_REQUIRE(y && x && w, "sb_gemm_stream_bf16: null pointer");
   SB_REQUIRE(n_rows >= 0 && n_out > 0 && n_in > 0, "sb_gemm_stream_bf16: bad sizes rows=%d out=%d in=%d",
              n_rows, n_out, n_in);
@@ -301,29 +299,29 @@ extern "C" int sb_gemm_stream_bf16(void *y, int y_dtype, const void *x, const vo
   const bf16_t *xb = (const bf16_t *)x, *wb = (const bf16_t *)w;
   const int tt = row_tiles(n_rows);
   if (gated) {
-    if (tt == 1) launch<1, 2, 1>(xb, wb, a, s);
-    else if (tt == 2) launch<2, 2, 1>(xb, wb, a, s);
-    else if (tt == 4) launch<4, 2, 1>(xb, wb, a, s);
-    else launch<8, 2, 1>(xb, wb, a, s);
+    if (tt == 1) launch<1, 2, 1>(xb, wb, a, hint, s);
+    else if (tt == 2) launch<2, 2, 1>(xb, wb, a, hint, s);
+    else if (tt == 4) launch<4, 2, 1>(xb, wb, a, hint, s);
+    else launch<8, 2, 1>(xb, wb, a, hint, s);
   } else {
-    if (tt == 1) launch<1, 1, 2>(xb, wb, a, s);
-    else if (tt == 2) launch<2, 1, 2>(xb, wb, a, s);
-    else if (tt == 4) launch<4, 1, 2>(xb, wb, a, s);
-    else launch<8, 1, 2>(xb, wb, a, s);
+    if (tt == 1) launch<1, 1, 2>(xb, wb, a, hint, s);
+    else if (tt == 2) launch<2, 1, 2>(xb, wb, a, hint, s);
+    else if (tt == 4) launch<4, 1, 2>(xb, wb, a, hint, s);
+    else launch<8, 1, 2>(xb, wb, a, hint, s);
   }
   return sb::check_launch("sb_gemm_stream_bf16");
 }
 
 // K slices sb_gemm_stream_partial_bf16 will produce for these sizes.
-extern "C" int sb_gemm_stream_slices(int n_rows, int n_out, int n_in) {
+extern "C" int sb_gemm_stream_slices(int n_rows, int n_out, int n_in, int hint) {
   if (n_rows <= 0 || n_out <= 0 || n_in <= 0) return 1;
-  return cut_for((n_out + 15) / 16, (n_in + kStepK - 1) / kStepK, row_tiles(n_rows)).slices;
+  return cut_for((n_out + 15) / 16, (n_in + kStepK - 1) / kStepK, row_tiles(n_rows), hint).slices;
 }
 
 // The raw product in K slices, for a consumer that adds them (and bias, residual, ...) itself:
 // partial float [slices][n_rows][n_out], slices = sb_gemm_stream_slices(...).  Operands as above.
 extern "C" int sb_gemm_stream_partial_bf16(float *partial, const void *x, const void *w, int n_rows, int n_out,
-                                           int n_in, void *stream) {
+                                           int n_in, int hint, void *stream) {
   SB_REQUIRE(partial && x && w, "sb_gemm_stream_partial_bf16: null pointer");
   SB_REQUIRE(n_rows >= 0 && n_out > 0 && n_in > 0, "sb_gemm_stream_partial_bf16: bad sizes");
   SB_SUPPORT(n_rows <= 64, "sb_gemm_stream_partial_bf16: %d rows, at most 64", n_rows);
@@ -333,7 +331,7 @@ extern "C" int sb_gemm_stream_partial_bf16(float *partial, const void *x, const 
   SB_SUPPORT((unsigned long long)(n_rows + 1) * n_in * 2 < (1ull << 31) && (unsigned long long)n_in * 32 < (1ull << 31),
              "sb_gemm_stream_partial_bf16: inner size %d is too large", n_in);
   if (n_rows == 0) return SB_OK;
-  const Cut c = cut_for((n_out + 15) / 16, (n_in + kStepK - 1) / kStepK, row_tiles(n_rows));
+  const Cut c = cut_for((n_out + 15) / 16, (n_in + kStepK - 1) / kStepK, row_tiles(n_rows), hint);
   const StreamArgs a{nullptr, SB_F32, nullptr, 0, nullptr, n_rows, n_out, n_in, partial, c.steps_per_slice};
   const bf16_t *xb = (const bf16_t *)x, *wb = (const bf16_t *)w;
   hipStream_t s = (hipStream_t)stream;

@@ -162,15 +162,18 @@ int sb_gemm_skinny_slices(int n_rows, int n_out, int n_in);
 int sb_gemm_skinny_partial_bf16(float *partial, const void *x, const void *w, int n_rows, int n_out,
                                 int n_in, int packed, void *stream);
 int sb_gemm_stream_max_rows(void);                       /* up to 128 rows, waves split the features */
+/* `hint` (0: the launcher chooses; for tests and measurements): bits 0..7 waves per block (4..8),
+ * bits 8..15 the K slices the partial form aims at (1..8).  `tile_shape`: -1 the launcher
+ * chooses, 0 / 1 / 2 tiles of 128 x 128, 256 x 128, 256 x 256 outputs. */
 int sb_gemm_stream_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,
                         int bias_dtype, const float *resid, int n_rows, int n_out, int n_in, int gated,
-                        void *stream);
-int sb_gemm_stream_slices(int n_rows, int n_out, int n_in);     /* up to 64 rows */
+                        int hint, void *stream);
+int sb_gemm_stream_slices(int n_rows, int n_out, int n_in, int hint);     /* up to 64 rows */
 int sb_gemm_stream_partial_bf16(float *partial, const void *x, const void *w, int n_rows, int n_out,
-                                int n_in, void *stream);
+                                int n_in, int hint, void *stream);
 int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,   /* tiled */
                       int bias_dtype, const float *resid, int n_rows, int n_out, int n_in, int gated,
-                      int packed, void *stream);
+                      int packed, int tile_shape, void *stream);
 int sb_gemm_mfma_slices(int n_rows, int n_out, int n_in);
 int sb_gemm_mfma_partial_bf16(float *partial, const void *x, const void *w, int n_rows, int n_out,
                               int n_in, int packed, void *stream);

@@ -27,6 +27,23 @@ from .step import StepError
 
 WIDTH_STEP = 16      # page-table widths are rounded up to this many pages (1024 tokens)
 CAPTURE_AFTER = 2    # kernel-by-kernel steps of a shape before its graph is captured
+MAX_GRAPHS = 24      # recorded shapes kept; the one unused for longest goes first
+EXACT_BATCHES = 8    # batches up to this size run as they are; larger ones are padded to a bucket
+
+
+def batch_bucket(n: int) -> int:
+    """The batch size a step of ``n`` sequences runs at: ``n`` itself up to 8, then the next of
+    12, 16, 24, 32, 48, 64, ... (twice and three times the powers of two).  A batch whose
+    sequences end one by one then passes through a handful of recorded shapes instead of one per
+    size; the rows added are sequences without pages, which store nothing and see no key."""
+    if n <= EXACT_BATCHES:
+        return n
+    p = 8
+    while True:
+        for b in (p + p // 2, 2 * p):
+            if n <= b:
+                return b
+        p *= 2
 
 
 class _StaticContext:
@@ -37,6 +54,7 @@ class _StaticContext:
         self.batch, self.width = batch, width
         self.n_groups = len(cache.groups)
         self.n_rows = self.n_seqs = self.n_wanted = batch
+        self.trace = None
         self.is_decode = True
         self.max_new = 1
         sizes = [batch, batch, batch, batch + 1, batch, batch, batch, 4 * batch] + [batch * width] * self.n_groups
@@ -68,22 +86,30 @@ class _StaticContext:
         return self._tables[group]
 
     def refresh(self, cache, slots: Sequence[int], tokens: Sequence[int]) -> None:
-        """This step's ids, positions and page tables, in one copy to the device."""
+        """This step's ids, positions and page tables, in one copy to the device.  Fewer
+        sequences than the buffers' batch: the rest are rows of token 0 at position 0 with no
+        page at all (they store nothing and attend to nothing; their logits are not read)."""
         host = self._hosts[self._turn]
         self._turn ^= 1
         n, o = host.numpy(), self._off
-        lengths = np.asarray([cache.length(s) for s in slots], dtype=np.int32)
-        n[o[0]:o[1]] = np.asarray(tokens, dtype=np.int32)
+        live = len(slots)
+        lengths = np.zeros(self.batch, dtype=np.int32)
+        lengths[:live] = [cache.length(s) for s in slots]
+        n[o[0]:o[0] + live] = np.asarray(tokens, dtype=np.int32)
+        n[o[0] + live:o[1]] = 0
         n[o[1]:o[2]] = lengths
         n[o[4]:o[5]] = lengths
-        n[o[5]:o[6]] = np.asarray(slots, dtype=np.int32)
+        n[o[5]:o[5] + live] = np.asarray(slots, dtype=np.int32)
+        n[o[5] + live:o[6]] = slots[0]
         for g in range(self.n_groups):
-            n[o[8 + g]:o[9 + g]] = cache.page_table(g, slots, min_width=self.width).reshape(-1)
+            table = n[o[8 + g]:o[9 + g]].reshape(self.batch, self.width)
+            table[:live] = cache.page_table(g, slots, min_width=self.width)
+            table[live:] = -1
         self.max_len_after = int(lengths.max()) + 1
         # the host's view of the step, as StepContext has it
-        self.slot_list = list(slots)
+        self.slot_list = list(slots) + [slots[0]] * (self.batch - live)
         self.lengths_before = lengths.tolist()
-        self.n_new = [1] * len(slots)
+        self.n_new = [1] * self.batch
         self.host_row_pos = lengths
         self.dev.copy_(host, non_blocking=True)
 
@@ -98,6 +124,8 @@ class DecodeLoop:
         # sequences) cannot be replayed from a recording; parts say so with graph_safe
         parts = [p for b in engine.model.blocks for p in (getattr(b, "mixer", None), getattr(b, "ffn", None))]
         self.use_graph = use_graph and all(getattr(p, "graph_safe", False) for p in parts if p is not None)
+        # added rows would run a mixer's per-sequence state of some live slot: no padding then
+        self.pad_batches = not engine.cache.state
         self._ctx: Dict[Tuple[int, int], _StaticContext] = {}
         self._graphs: Dict[Tuple[int, int, bool], Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
         self._uses: Dict[Tuple[int, int, bool], int] = {}
@@ -118,7 +146,8 @@ class DecodeLoop:
     def _key(self) -> Tuple[int, int]:
         cache = self.engine.cache
         need = max((cache.length(s) + 1 + 63) // 64 for s in self.slots)
-        return len(self.slots), ((need + WIDTH_STEP - 1) // WIDTH_STEP) * WIDTH_STEP
+        batch = batch_bucket(len(self.slots)) if self.pad_batches else len(self.slots)
+        return batch, ((need + WIDTH_STEP - 1) // WIDTH_STEP) * WIDTH_STEP
 
     def _run(self, tokens: Sequence[int], choose: bool):
         """One step of the live sequences feeding ``tokens``: the logits [B, vocab] and the
@@ -142,8 +171,9 @@ class DecodeLoop:
             ctx = self._ctx[key] = _StaticContext(eng, *key)
         ctx.refresh(cache, self.slots, tokens)
         gkey = (*key, choose)
-        entry = self._graphs.get(gkey)
+        entry = self._graphs.pop(gkey, None)
         if entry is not None:
+            self._graphs[gkey] = entry          # most recently used last
             entry[0].replay()
             logits = entry[1]
         else:
@@ -154,7 +184,8 @@ class DecodeLoop:
             if self.use_graph and n >= CAPTURE_AFTER:
                 self._capture(gkey, ctx, choose)
         cache.advance(self.slots, ones)
-        return logits, ctx.next_ids
+        live = len(self.slots)
+        return logits[:live], ctx.next_ids[:live]
 
     def _capture(self, gkey, ctx, choose: bool) -> None:
         """Record the launches of a step of this shape.  Capture runs nothing; replays read the
@@ -165,6 +196,10 @@ class DecodeLoop:
             logits = self.engine.forward(ctx)
             if choose:
                 ops.argmax(logits, out=ctx.next_ids)
+        while len(self._graphs) >= MAX_GRAPHS:
+            oldest = next(iter(self._graphs))
+            del self._graphs[oldest]            # its memory pool goes with it
+            self._uses.pop(oldest, None)
         self._graphs[gkey] = (graph, logits)
 
     def step(self) -> List[int]:

@@ -116,6 +116,7 @@ class StepContext:
         self.tiles = flat_tiles.view(-1, 4)
         self._tables = [v.view(t.shape) for v, t in zip(views[8:], tables)]
         self.host_row_pos = row_pos
+        self.trace = None            # set by the engine while a tracer listens
 
     def page_table(self, group: int) -> torch.Tensor:
         return self._tables[group]
@@ -137,6 +138,9 @@ class Engine:
         self.bindings = model.bindings(self.cache)
         self.use_graphs = True
         self._loop = None
+        # set to a callable (name, tensor) to receive a step's named intermediates, in the order of
+        # the computation: "embedding", "entry<i>.after_mixer", "entry<i>.after_ffn", "logits"
+        self.tracer = None
 
     def decode_loop(self):
         """The engine's loop for single-token steps (one per engine: it keeps the captured graphs)."""
@@ -224,13 +228,22 @@ class Engine:
         """The device work of a step whose bookkeeping ``ctx`` holds: embedding, the blocks in
         their run order, and for the wanted rows the final norm and the head."""
         model = self.model
+        tracer = self.tracer
         x = model.embedding.forward(ctx.ids)
+        if tracer is not None:
+            tracer("embedding", x)
         h = None
         for i, e in enumerate(model.order):
             nxt = model.order[i + 1].block if i + 1 < len(model.order) else None
-            next_norm = getattr(model.blocks[nxt], "mixer_norm", None) if nxt is not None else None
+            next_norm = getattr(model.blocks[nxt], "first_norm", None) if nxt is not None else None
+            # a block reports what it has computed through ctx.trace, if it cares to
+            ctx.trace = (lambda what, t, _i=i: tracer(f"entry{_i}.{what}", t)) if tracer is not None else None
             h = model.blocks[e.block].forward(x, ctx, self.bindings[i], h=h, next_norm=next_norm)
+        ctx.trace = None
         if ctx.n_wanted == 0:
             return torch.empty((0, model.vocab), dtype=torch.float32, device=self.device)
         h = model.final_norm.forward(x, model.rt.act_dtype, rows=ctx.want_rows)
-        return model.head.forward(h)
+        logits = model.head.forward(h)
+        if tracer is not None:
+            tracer("logits", logits)
+        return logits

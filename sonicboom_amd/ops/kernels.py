@@ -11,6 +11,7 @@ from __future__ import annotations
 
 import contextlib
 import math
+import threading
 
 from typing import Optional
 
@@ -18,6 +19,18 @@ import torch
 
 from . import library
 from .library import KernelLibraryError, check
+
+class _Hints(threading.local):
+    """Choices a test or a measurement imposes on the launchers, for the calls of its own thread
+    inside a ``with`` block; every kernel call passes them as arguments (the library keeps no
+    such state)."""
+    few_rows_kernel = None      # "stream", "skinny", "tiled" or None
+    stream = 0                  # waves | slices << 8 of the weight-streaming product
+    tile_shape = -1             # of the tiled product
+    decode_pages = 0            # pages per wave of decode attention
+
+
+_hints = _Hints()
 
 PAGE = 64          # tokens per cache page; SB_PAGE of csrc/sb_hip.h
 MAX_CANDIDATES = 256
@@ -300,12 +313,10 @@ def gemm_bf16_partial(x: torch.Tensor, w: torch.Tensor, packed_shape=None) -> Op
     """The raw product x w^T of bfloat16 rows in K slices, float32 [slices, rows, out], for a
     consumer that adds the slices itself (:func:`reduce_resid_norm`, :func:`rope_kv_store`).
     Packed weights, up to 64 rows: the kernel whose waves split the output features and share
-    the rows through LDS, with K cut over the grid so that the blocks fill the GPU (measured
-    with the kernel that adds the slices, Qwen2.5-7B down product: 31 us at 8 rows, 38 at 64).
+    the rows through LDS, with K cut over the grid so that the blocks fill the GPU.
     Packed weights, more rows: the tiled kernel with K cut over the grid, as long as the cut gives
     more than one slice (a narrow matrix and up to a few hundred rows; one slice would leave most
-    of the GPU without a tile: at 128 rows the output product takes 18 against 49 us, down 36
-    against 146).  Row-major weights, up to 64 rows: the kernel whose waves split K.  None when
+    of the GPU without a tile).  Row-major weights, up to 64 rows: the kernel whose waves split K.  None when
     none applies: the caller then takes the whole product."""
     _dev(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or x.dim() != 2:
@@ -317,11 +328,11 @@ def gemm_bf16_partial(x: torch.Tensor, w: torch.Tensor, packed_shape=None) -> Op
     if t == 0 or k % 8 or x.data_ptr() % 16 or w.data_ptr() % 16:
         return None
     lib = library.core()
-    which = _few_rows_kernel[0]
+    which = _hints.few_rows_kernel
     if packed_shape is not None and t <= SKINNY_MAX_ROWS and which in (None, "stream"):
-        slices = lib.sb_gemm_stream_slices(t, n, k)
+        slices = lib.sb_gemm_stream_slices(t, n, k, _hints.stream)
         partial = torch.empty((slices, t, n), dtype=torch.float32, device=x.device)
-        check(lib.sb_gemm_stream_partial_bf16(_p(partial), _p(x), _p(w), t, n, k, _stream()))
+        check(lib.sb_gemm_stream_partial_bf16(_p(partial), _p(x), _p(w), t, n, k, _hints.stream, _stream()))
         return partial
     if packed_shape is not None and (t > SKINNY_MAX_ROWS or which == "tiled"):
         slices = lib.sb_gemm_mfma_slices(t, n, k)
@@ -421,23 +432,20 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], re
     # A wide packed matrix (enough 16-row tiles, or gate/up pairs of them, for STREAM_MIN_BLOCKS
     # blocks of four waves) and up to 128 rows: the kernel whose waves split the output features
     # and share the rows through LDS.  Other products of up to 64 rows: the kernel whose waves
-    # split K and which can cut K over the grid as well.  The rest: the tiled kernel.  Measured at Qwen2.5-7B sizes: gate/up at 64
-    # rows 53 us (tiled kernel 74, few-row kernel 85), at 8 rows 48 (few-row kernel 50); the
-    # head at 16 rows 196 (few-row kernel 259).
-    which = _few_rows_kernel[0]
+    # split K and which can cut K over the grid as well.  The rest: the tiled kernel.
+    which = _hints.few_rows_kernel
     if which is None:
         wave_units = -(-n // 16) if gated else -(-n // 32)
         which = "stream" if packed and wave_units >= 4 * STREAM_MIN_BLOCKS else "skinny"
         if t > SKINNY_MAX_ROWS and which == "stream":
             # 65 to 128 rows: the tiled kernel's 128 x 128 tiles do as well or better unless their
-            # count leaves the last round over the 256 CUs nearly empty (Qwen2.5-7B gate/up: 296
-            # tiles, 85 us at 128 rows against 70 here; 216, 462 or 1,188 tiles: the tiled kernel)
+            # count leaves the last round over the 256 CUs nearly empty
             rounds = -(-n // (64 if gated else 128)) / 256.0
             if math.ceil(rounds) / rounds < 1.4:
                 which = "tiled"
     if t <= STREAM_MAX_ROWS and which == "stream" and packed:
         check(lib.sb_gemm_stream_bf16(_p(out), _dt(out), _p(x), _p(w), _p(bias), bdt, _p(resid), t, n, k,
-                                      1 if gated else 0, _stream()))
+                                      1 if gated else 0, _hints.stream, _stream()))
     elif t <= SKINNY_MAX_ROWS and which != "tiled":
         need = lib.sb_gemm_skinny_scratch(t, n, k, 1 if gated else 0)
         scratch = torch.empty((need,), dtype=torch.float32, device=x.device) if need else None
@@ -445,44 +453,40 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], re
                                       1 if gated else 0, packed, _p(scratch), need, _stream()))
     else:
         check(lib.sb_gemm_mfma_bf16(_p(out), _dt(out), _p(x), _p(w), _p(bias), bdt, _p(resid), t, n, k,
-                                    1 if gated else 0, packed, _stream()))
+                                    1 if gated else 0, packed, _hints.tile_shape, _stream()))
     return out
 
 
 @contextlib.contextmanager
 def gemm_tile_shape(shape: Optional[int]):
-    """For tests and measurements: inside the block the tiled product uses tile shape ``shape``
-    (0: 128 x 128, 1: 256 x 128, 2: 256 x 256 outputs per block) instead of choosing one."""
-    lib = library.core()
-    lib.sb_gemm_mfma_force(-1 if shape is None else int(shape))
+    """For tests and measurements: inside the block the tiled products of this thread use tile
+    shape ``shape`` (0: 128 x 128, 1: 256 x 128, 2: 256 x 256 outputs per block) instead of
+    choosing one."""
+    before = _hints.tile_shape
+    _hints.tile_shape = -1 if shape is None else int(shape)
     try:
         yield
     finally:
-        lib.sb_gemm_mfma_force(-1)
+        _hints.tile_shape = before
 
 
 @contextlib.contextmanager
 def gemm_few_rows_kernel(which: Optional[str], waves: int = 0, slices: int = 0):
-    """For tests and measurements: inside the block products of up to 64 rows, whole or in K
-    slices, go to the kernel ``which`` ("stream", "skinny" or "tiled"; "stream" needs packed
-    weights) whatever the sizes, and the stream kernel uses ``waves`` waves per block (4 to 8)
-    and aims at ``slices`` K slices (1 to 8); 0: its own choice."""
+    """For tests and measurements: inside the block this thread's products of up to 64 rows,
+    whole or in K slices, go to the kernel ``which`` ("stream", "skinny" or "tiled"; "stream"
+    needs packed weights) whatever the sizes, and the stream kernel uses ``waves`` waves per block
+    (4 to 8) and aims at ``slices`` K slices (1 to 8); 0: its own choice."""
     if which not in (None, "stream", "skinny", "tiled"):
         raise ValueError(f"unknown kernel {which!r}")
-    lib = library.core()
-    before = _few_rows_kernel[0]
-    _few_rows_kernel[0] = which
-    lib.sb_gemm_stream_force(int(waves))
-    lib.sb_gemm_stream_force_slices(int(slices))
+    before = (_hints.few_rows_kernel, _hints.stream)
+    _hints.few_rows_kernel = which
+    _hints.stream = (int(waves) & 0xff) | ((int(slices) & 0xff) << 8)
     try:
         yield
     finally:
-        _few_rows_kernel[0] = before
-        lib.sb_gemm_stream_force(0)
-        lib.sb_gemm_stream_force_slices(0)
+        _hints.few_rows_kernel, _hints.stream = before
 
 
-_few_rows_kernel = [None]
 MFMA_MAX_HEAD_DIM = 256
 STREAM_MIN_BLOCKS = 192
 STREAM_MAX_ROWS = 128
@@ -517,22 +521,22 @@ def attention_decode_mfma(q, k_cache, v_cache, page_table, seq_pos, heads_q, hea
                               device=q.device)
     check(lib.sb_attn_decode_bf16(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(page_table), max_pages,
                                   k_cache.shape[0], _p(seq_pos), _p(part_o), _p(part_ml), n, heads_q,
-                                  heads_kv, float(scale), int(window), _stream()), lib, "sb_attn_last_error")
+                                  heads_kv, float(scale), int(window), _hints.decode_pages, _stream()),
+          lib, "sb_attn_last_error")
     return out
 
 
 @contextlib.contextmanager
 def attention_decode_pages_per_wave(head_dim: int, pages: int):
-    """For tests and measurements: inside the block the decode attention kernel of this head size
-    gives every wave ``pages`` pages (1, 2, 4 or 8; more than one only up to head size 128)
-    instead of choosing from the sizes."""
-    lib = library.attention_library(head_dim)
-    lib.sb_attn_decode_force.restype = None
-    lib.sb_attn_decode_force(int(pages))
+    """For tests and measurements: inside the block this thread's decode attention gives every
+    wave ``pages`` pages (1, 2, 4 or 8; more than one only up to head size 128) instead of
+    choosing from the sizes; 0: the launcher's choice."""
+    before = _hints.decode_pages
+    _hints.decode_pages = int(pages)
     try:
         yield
     finally:
-        lib.sb_attn_decode_force(0)
+        _hints.decode_pages = before
 
 
 def attention_prefill_mfma(q, k_cache, v_cache, page_table, row_pos, tiles, heads_q, heads_kv, head_dim, scale,

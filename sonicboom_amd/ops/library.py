@@ -39,25 +39,21 @@ _OPTIONAL_SIGNATURES = {
     "sb_gemm_skinny_partial_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
     "sb_gemm_skinny_slices": [_I, _I, _I],
     "sb_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _P, _Z, _P],
-    "sb_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _P],
-    "sb_gemm_stream_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P],
-    "sb_gemm_stream_force": [_I],
-    "sb_gemm_stream_force_slices": [_I],
-    "sb_gemm_stream_slices": [_I, _I, _I],
-    "sb_gemm_stream_partial_bf16": [_P, _P, _P, _I, _I, _I, _P],
-    "sb_gemm_mfma_force": [_I],
+    "sb_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
+    "sb_gemm_stream_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _P],
+    "sb_gemm_stream_slices": [_I, _I, _I, _I],
+    "sb_gemm_stream_partial_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
     "sb_gemm_mfma_slices": [_I, _I, _I],
     "sb_gemm_mfma_partial_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
 }
 _ATTN_SIGNATURES = {
     # out, q, k_cache, v_cache, page_table, max_pages, n_pages, row_pos, part_o, part_ml, n_seqs,
-    # heads_q, heads_kv, scale, window, stream
-    "sb_attn_decode_bf16": [_P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _F, _I, _P],
+    # heads_q, heads_kv, scale, window, pages per wave (0: chosen), stream
+    "sb_attn_decode_bf16": [_P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _I, _F, _I, _I, _P],
     # out, q, k_cache, v_cache, page_table, max_pages, n_pages, row_pos, tiles, n_tiles, heads_q,
     # heads_kv, scale, window, stream
     "sb_attn_prefill_bf16": [_P, _P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _F, _I, _P],
     "sb_attn_decode_chunks": [_I],
-    "sb_attn_decode_force": [_I],
     "sb_attn_head_dim": [],
 }
 

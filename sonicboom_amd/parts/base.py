@@ -21,7 +21,10 @@ copy in the activation type, ``ctx`` the step's
                 takes ``then_norm=`` and may return the normed stream) and ``graph_safe``
                 (their launches depend on device buffers only, so a decode step may be
                 recorded once and replayed).
-* **block**     ``mixer`` attribute and ``forward(x, ctx, binding)``.
+* **block**     ``mixer`` attribute and ``forward(x, ctx, binding, h=None, next_norm=None)``;
+                optionally ``first_norm``, the norm the block starts with (the block before
+                may then hand over ``h`` = first_norm(x) from its last pass), and calls of
+                ``ctx.trace(name, x)`` after its mixer and feed-forward when that is set.
 * **embedding** ``forward(ids) -> x``
 * **head**      ``forward(h) -> float32 logits [rows, vocab]``
 """

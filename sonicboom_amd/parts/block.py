@@ -23,6 +23,7 @@ class PreNormBlock(Part):
     def __init__(self, spec, tensors, parts, rt):
         super().__init__(spec, tensors, parts, rt)
         self.mixer_norm = parts["mixer_norm"]
+        self.first_norm = self.mixer_norm      # what the block before may apply in its last pass
         self.mixer = parts["mixer"]
         self.ffn_norm = parts["ffn_norm"]
         self.ffn = parts["ffn"]
@@ -41,9 +42,16 @@ class PreNormBlock(Part):
             f = self.mixer.forward(h, x, ctx, binding, then_norm=self.ffn_norm)
         else:
             self.mixer.forward(h, x, ctx, binding)
+        trace = getattr(ctx, "trace", None)
+        if trace is not None:
+            trace("after_mixer", x)
         if f is None:
             f = self.ffn_norm.forward(x, act)
+        out = None
         if getattr(self.ffn, "fuses_norm", False):
-            return self.ffn.forward(f, x, ctx, then_norm=next_norm)
-        self.ffn.forward(f, x, ctx)
-        return None
+            out = self.ffn.forward(f, x, ctx, then_norm=next_norm)
+        else:
+            self.ffn.forward(f, x, ctx)
+        if trace is not None:
+            trace("after_ffn", x)
+        return out

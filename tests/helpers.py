@@ -48,18 +48,24 @@ def forget_plain(folder):
 # which rounding keeps small and a systematic mistake does not, has a tighter bound of its own.
 # On the "sharp" models (conftest.SHARP_QK) scores of ten and more make the softmax amplify the
 # rounding of queries and keys: measured on the GPU the largest difference was 0.23 spreads and
-# the root mean square 0.021, against 0.018 and 0.004 on the models of plain random weights.
+# the root mean square 0.022, against 0.018 and 0.004 on the tiny models of plain random weights.
+# "wide" is for models of real layer sizes, where a row of 3,584 and a sum over 18,944 products
+# round more often: measured 0.058 and 0.0095 there, where the smallest of the mistakes that
+# tests/test_plain.py::test_sharp_models_show_attention_mistakes plants, a dropped query bias,
+# moves the plain logits by 0.20 and 0.031 (a wrong scale by 4.6 and 0.88).
 F32_TOL = dict(atol=5e-5, rtol=5e-5)
-BF16_MAX = {False: 0.04, True: 0.5}       # largest difference, in spreads (plus BF16_REL * |logit|)
-BF16_RMS = {False: 0.01, True: 0.05}      # root mean square of the differences, in spreads
+BF16_MAX = {"tiny": 0.04, "wide": 0.16, "sharp": 0.5}     # largest difference, in spreads (plus BF16_REL * |logit|)
+BF16_RMS = {"tiny": 0.01, "wide": 0.02, "sharp": 0.05}    # root mean square of the differences, in spreads
 BF16_REL = 0.02
 
 
 def bf16_limits(want, sharp=False):
-    """(bound on every |difference|, bound on their root mean square) for logits ``want``."""
+    """(bound on every |difference|, bound on their root mean square) for logits ``want``;
+    ``sharp``: False / "tiny", True / "sharp", or "wide"."""
+    kind = {False: "tiny", True: "sharp"}.get(sharp, sharp)
     want = np.asarray(want, dtype=np.float64)
     spread = float(want.std())
-    return BF16_MAX[sharp] * spread + BF16_REL * np.abs(want), BF16_RMS[sharp] * spread
+    return BF16_MAX[kind] * spread + BF16_REL * np.abs(want), BF16_RMS[kind] * spread
 
 
 def assert_logits_close(got, want, dtype, what="", sharp=False):

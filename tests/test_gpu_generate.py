@@ -136,6 +136,42 @@ def test_graph_replay_gives_the_same_tokens(model_folders):
     assert s == without.generate(prompts, temperature=0.7, seed=3, max_tokens=40, stop_tokens=())
 
 
+def test_batches_run_in_buckets_with_rows_that_do_nothing(model_folders):
+    """The decode loop runs a batch of more than eight sequences at the next bucket's size (12,
+    16, 24, ...): the rows it adds have no pages, store nothing and see no key.  A batch of 21
+    whose sequences end one by one must give every sequence the tokens it gets alone, pass
+    through a handful of recorded shapes, not one per size, and leave the cache empty."""
+    from sonicboom_amd.engine.decode import batch_bucket
+    assert [batch_bucket(n) for n in (1, 7, 8, 9, 12, 13, 17, 24, 25, 33, 64, 65, 100)] == \
+        [1, 7, 8, 12, 12, 16, 24, 24, 32, 48, 64, 96, 128]
+    folder = model_folders["B"]
+    model = model_for(folder, "float32")
+    prompts = prompts_for("B", [3 + (7 * i) % 40 for i in range(21)], seed=31)
+    session = model.session(max_tokens=64 * 64)
+    lone = model.session(max_tokens=64 * 4)
+    lone.engine.use_graphs = False
+    # every sequence stops at its own length: the batch shrinks by one again and again
+    counts = [4 + i for i in range(21)]
+    want = [lone.generate([p], max_tokens=n, stop_tokens=())[0] for p, n in zip(prompts, counts)]
+    ends = {}
+
+    def cut(i, t):
+        ends[i] = ends.get(i, 0) + 1
+        return ends[i] > counts[i]
+    got = session.generate(prompts, max_tokens=40, stop_tokens=(), callback=cut)
+    assert got == want
+    shapes = sorted({k[0] for k in session.engine.decode_loop()._graphs})
+    assert shapes and set(shapes) <= {1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 24}, shapes
+    assert not session.engine.cache.live_slots and session.engine.cache.held_pages() == 0
+    # sampled, in bfloat16, graph against kernel by kernel: the same tokens with added rows in the batch
+    model16 = model_for(folder, "bfloat16")
+    a, b = model16.session(max_tokens=64 * 64), model16.session(max_tokens=64 * 64)
+    b.engine.use_graphs = False
+    ta = a.generate(prompts[:11], temperature=0.9, seed=5, max_tokens=12, stop_tokens=())
+    tb = b.generate(prompts[:11], temperature=0.9, seed=5, max_tokens=12, stop_tokens=())
+    assert ta == tb
+
+
 def test_graph_replay_when_the_page_table_grows(tmp_path):
     """Decoding across 1,024 tokens: the decode loop's buffers are keyed by the page table's
     width (steps of 16 pages), so the step is recorded a second time there; tokens with and

@@ -661,6 +661,110 @@ def test_attention_matrix_cores_when_the_maximum_moves(hq, hkv, hd, shape):
         close(got[-1:], v_far.numpy(), atol=2e-2, rtol=1e-2, what="far key's value")
 
 
+def _looking_along_zero(n, hq, hkv, hd, n_rows, seed):
+    """Small random keys and queries whose coordinate 0 is large in the queries: a key whose
+    coordinate 0 is raised takes all of a row's weight.  Returns keys, values, queries, the raise
+    that puts one score 56 above the rest, and the scale."""
+    scale = 1.0 / math.sqrt(hd)
+    keys = randn(n, hkv, hd, scale=0.05, seed=seed)
+    vals = randn(n, hkv, hd, seed=seed + 1)
+    q = randn(n_rows, hq * hd, scale=0.05, seed=seed + 2)
+    q.view(n_rows, hq, hd)[:, :, 0] = 8.0
+    return keys.to(BF16).float(), vals.to(BF16).float(), q.to(BF16), 56.0 / (8.0 * scale), scale
+
+
+@pytest.mark.parametrize("pages", [0, 1, 2, 4, 8])
+def test_attention_decode_one_dominant_key_in_each_chunk(pages):
+    """A row of 6,500 keys is cut into chunks of 4 x ``pages`` pages whose partial results a
+    second kernel merges.  One key at a time is made to dominate: the first key of all, the first
+    and last key of a wave's run of pages in a middle chunk, the first key of the second and of
+    the last chunk, the row's own key and the one before it.  The output must be that key's
+    value: a chunk or a wave's run that is dropped, merged twice or weighted wrongly shows at
+    once, where random keys would move the output by less than the tolerance."""
+    from sonicboom_amd import ops
+    hq, hkv, hd, n = 8, 2, 64, 6500
+    keys, vals, q, rise, scale = _looking_along_zero(n, hq, hkv, hd, 1, seed=31)
+    width = (n + 63) // 64
+    table = torch.randperm(width + 5, generator=torch.Generator().manual_seed(3))[:width].to(torch.int32)[None, :]
+    kc, vc = fill_cache_from([keys], [vals], table, BF16)
+    pos = torch.tensor([n - 1], dtype=torch.int32, device=DEV)
+    run = max(pages, 1)                    # pages of a wave's run; a chunk is four runs
+    last_chunk = ((n - 1) // 64 // (4 * run)) * 4 * run * 64
+    spots = sorted({0, 4 * run * 64, (4 * run + 2 * run) * 64, (4 * run + 2 * run) * 64 - 1,
+                    (4 * run + run) * 64 - 1, last_chunk, last_chunk - 1, n - 2, n - 1})
+    group = hq // hkv
+    with ops.attention_decode_pages_per_wave(hd, pages):
+        for far in spots:
+            page, slot = int(table[0, far // 64]), far % 64
+            before = kc[page, :, slot, 0].clone()
+            kc[page, :, slot, 0] = rise
+            got = ops.attention_decode_mfma(q.to(DEV), kc, vc, table.to(DEV), pos, hq, hkv, hd, scale, 0)
+            kc[page, :, slot, 0] = before
+            want = vals[far].repeat_interleave(group, dim=0).reshape(1, -1)
+            close(got, want.numpy(), atol=2e-2, rtol=1e-2, what=f"dominant key at {far}, {pages} pages per wave")
+
+
+@pytest.mark.parametrize("window", [70, 200, 1000])
+@pytest.mark.parametrize("pages", [0, 1, 2, 8])
+def test_attention_decode_window_edge(window, pages):
+    """The lower edge of the window, to the key: a dominant key at position - window is out of
+    the window and must count for nothing; at position - window + 1 it is the window's first key
+    and must take all the weight.  On random data the keys before the edge are valid cache
+    contents, and one key too many moves the output by less than the tolerance."""
+    from sonicboom_amd import ops
+    hq, hkv, hd, n = 6, 2, 64, 1500
+    keys, vals, q, rise, scale = _looking_along_zero(n, hq, hkv, hd, 1, seed=41)
+    table = torch.arange((n + 63) // 64, dtype=torch.int32).flip(0)[None, :].contiguous()
+    group = hq // hkv
+    for p in (n - 1, 1030, 1024 + window - 1):          # the edge inside a page, and on a page's first key
+        p = min(p, n - 1)
+        for inside in (False, True):
+            k = keys.clone()
+            edge = p - window + (1 if inside else 0)
+            k[edge, :, 0] = rise
+            kc, vc = fill_cache_from([k], [vals], table, BF16)
+            pos = torch.tensor([p], dtype=torch.int32, device=DEV)
+            with ops.attention_decode_pages_per_wave(hd, pages):
+                got = ops.attention_decode_mfma(q.to(DEV), kc, vc, table.to(DEV), pos, hq, hkv, hd, scale, window)
+            if inside:
+                want = vals[edge].repeat_interleave(group, dim=0).reshape(1, -1).numpy()
+            else:
+                want = plain.attention(q.float().numpy(), k.reshape(n, -1).numpy(), vals.reshape(n, -1).numpy(), [p],
+                                       np.arange(n), hq, hkv, hd, scale, causal=True, window=window)
+                assert np.abs(want - vals[edge].repeat_interleave(group, dim=0).reshape(1, -1).numpy()).max() > 0.5
+            close(got, want, atol=2e-2, rtol=1e-2, what=f"position {p}, window {window}, key {edge}")
+
+
+@pytest.mark.parametrize("hq, hkv, hd", [(6, 2, 64), (28, 4, 128), (3, 1, 32)])
+@pytest.mark.parametrize("window", [70, 300])
+def test_attention_prefill_window_edge(hq, hkv, hd, window):
+    """Prompt rows over a window: one dominant key at position d.  Rows up to d + window - 1
+    have it as a key of their window (the last of them as its very first key) and must return
+    its value; from row d + window on it has left the window and must count for nothing."""
+    from sonicboom_amd import ops
+    n = 700
+    rows_pos = list(range(n - 80, n))
+    keys, vals, q, rise, scale = _looking_along_zero(n, hq, hkv, hd, len(rows_pos), seed=51)
+    group = hq // hkv
+    table = torch.tensor([[7, 2, 9, 4, 0, 5, 1, 8, 3, 6, 10]], dtype=torch.int32)
+    pos = torch.tensor(rows_pos, dtype=torch.int32)
+    tiles = torch.tensor([(r0, min(16, len(rows_pos) - r0), 0, 0) for r0 in range(0, len(rows_pos), 16)],
+                         dtype=torch.int32)
+    for last_seeing in (rows_pos[0] + 20, rows_pos[0] + 47, rows_pos[0] + 48):     # inside a tile of 16, at its end, at its start
+        d = last_seeing - window + 1
+        k = keys.clone()
+        k[d, :, 0] = rise
+        kc, vc = fill_cache_from([k], [vals], table, BF16)
+        got = ops.attention_prefill_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), tiles.to(DEV), hq, hkv, hd,
+                                         scale, window)
+        want = plain.attention(q.float().numpy(), k.reshape(n, -1).numpy(), vals.reshape(n, -1).numpy(), rows_pos,
+                               np.arange(n), hq, hkv, hd, scale, causal=True, window=window)
+        v_d = vals[d].repeat_interleave(group, dim=0).reshape(1, -1).numpy()
+        r = last_seeing - rows_pos[0]
+        assert np.abs(want[r] - v_d).max() < 2e-2 and np.abs(want[r + 1] - v_d).max() > 0.5     # the case is sharp
+        close(got, want, atol=2e-2, rtol=1e-2, what=f"window {window}, dominant key {d}")
+
+
 @pytest.mark.parametrize("vocab", [5, 256, 1000, 152064])
 def test_argmax_first_maximum(vocab):
     from sonicboom_amd import ops

@@ -85,6 +85,75 @@ def test_replay_three_ways(model_folders, tmp_path, name, dtype):
         assert_logits_close(got, want, dtype, f"{name} step {s}")
 
 
+def plain_dump(folder, tokens, path, want):
+    """The plain implementation's intermediates for one whole request, in the dump format."""
+    from plain import qwen2_plain as P
+    cfg, w = P.load_model(folder)
+    pos = np.arange(len(tokens))
+    lines = ["# plain implementation"]
+
+    def emit(name, a):
+        a = np.asarray(a, np.float32).reshape(-1)
+        lines.append(f"@ {name} f32 {a.size} 1 1 1")
+        lines.extend("%.9g" % v for v in a.tolist())
+    x = P.embedding(w["model.embed_tokens.weight"], tokens)
+    emit("embedding", x)
+    for layer in range(cfg["num_hidden_layers"]):
+        p = f"model.layers.{layer}."
+        h = P.rms_norm(x, w[p + "input_layernorm.weight"], cfg["rms_norm_eps"])
+        x1 = (P.self_attention(h, pos, w, p + "self_attn.", cfg) + x).astype(np.float32)
+        emit(f"entry{layer}.after_mixer", x1)
+        x = P.block(x, pos, w, layer, cfg)
+        emit(f"entry{layer}.after_ffn", x)
+    emit("logits", P.lm_head(x, w, cfg)[want])
+    with open(path, "w") as f:
+        f.write("\n".join(lines) + "\n")
+
+
+def test_dumps_of_intermediates_and_their_comparison(model_folders, tmp_path):
+    """--trace writes every step's residual stream after each mixer and feed-forward; the
+    comparison tool finds them equal to the plain implementation's in 32-bit, and names the first
+    entry that differs when one layer's weights do."""
+    import shutil
+
+    import torch
+    from safetensors import safe_open
+    from safetensors.torch import save_file
+    folder, vocab = model_folders["B"], TINY["B"]["vocab_size"]
+    tokens = random_prompt(np.random.default_rng(3), vocab, 21)
+    want = [0, 20]
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": tokens, "want": want}], "end": ["a"]}]
+    cmd = lambda model, out: [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", model,  # noqa: E731
+                              "--dtype", "float32", "--out", str(out), "--max-tokens", "64", "--trace", str(out)]
+    text = "".join(json.dumps(s) + "\n" for s in steps)
+    p = subprocess.run(cmd(folder, tmp_path / "good"), input=text, capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    plain_dump(folder, tokens, tmp_path / "plain.dump", want)
+    compare = [sys.executable, os.path.join(ROOT, "bin", "compare_dumps")]
+    r = subprocess.run(compare + [str(tmp_path / "plain.dump"), str(tmp_path / "good" / "0.dump"), "1e-4"],
+                       capture_output=True, text=True)
+    assert r.returncode == 0 and "dumps agree" in r.stdout, r.stdout + r.stderr
+    names = [line.split()[0] for line in r.stdout.splitlines() if line.startswith(("embedding", "entry", "logits"))]
+    assert names == ["embedding"] + [f"entry{i}.after_{w}" for i in range(3) for w in ("mixer", "ffn")] + ["logits"]
+    # the same model with layer 1's down projection changed: the first difference is after that feed-forward
+    bad = tmp_path / "bad_model"
+    os.makedirs(bad)
+    shutil.copy(os.path.join(folder, "config.json"), bad / "config.json")
+    tensors = {}
+    with safe_open(os.path.join(folder, "model.safetensors"), framework="pt") as f:
+        for name in f.keys():
+            t = f.get_tensor(name)
+            tensors[name] = (t * 1.5).to(t.dtype) if name == "model.layers.1.mlp.down_proj.weight" else t
+    save_file(tensors, str(bad / "model.safetensors"), metadata={"format": "pt"})
+    p = subprocess.run(cmd(str(bad), tmp_path / "bad"), input=text, capture_output=True, text=True, timeout=600)
+    assert p.returncode == 0, p.stderr[-2000:]
+    r = subprocess.run(compare + [str(tmp_path / "plain.dump"), str(tmp_path / "bad" / "0.dump")],
+                       capture_output=True, text=True)
+    assert r.returncode == 1 and "first tensor out of tolerance: entry1.after_ffn" in r.stdout, r.stdout
+    assert subprocess.run(compare, capture_output=True, text=True).returncode == 2
+    del torch
+
+
 def test_trace_run_reports_bad_input(model_folders, tmp_path):
     cmd = [sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", str(tmp_path), "--dtype", "float32",
            "--out", str(tmp_path / "o"), "--max-tokens", "64"]
