@@ -180,9 +180,40 @@ def ensure_attention(head_dim: int, force: bool = False) -> str:
     return _ensure(f"libsbattn_hd{head_dim}.so", ATTN_SOURCES, [f"SB_HEAD_DIM={head_dim}"], force)
 
 
+def ensure_plain_host(force: bool = False) -> str:
+    """Path of ``libsbplain.so``: the kernels' plain C++ twins on host memory (plain_host.cpp),
+    compiled with the host compiler.  The tests compare the kernels with them."""
+    out_dir = build_dir()
+    lib, stamp = os.path.join(out_dir, "libsbplain.so"), os.path.join(out_dir, "libsbplain.so.stamp")
+    src, header = os.path.join(HERE, "plain_host.cpp"), os.path.join(HERE, "plain_host.h")
+    h = hashlib.sha256()
+    for path in (src, header):
+        with open(path, "rb") as f:
+            h.update(f.read())
+    want = h.hexdigest()
+    if not force and os.path.exists(lib) and os.path.exists(stamp):
+        with open(stamp) as f:
+            if f.read().strip() == want:
+                return lib
+    cxx = shutil.which("g++") or shutil.which("c++") or shutil.which("amdclang++")
+    if not cxx:
+        raise BuildError("no host C++ compiler (g++) for the plain twins")
+    tmp = lib + f".tmp{os.getpid()}"
+    # no contraction into fused multiply-adds: the arithmetic is what the source says
+    _run([cxx, "-O2", "-std=c++17", "-shared", "-fPIC", "-ffp-contract=off", "-Wall", src, "-o", tmp],
+         "compiling plain_host.cpp")
+    os.replace(tmp, lib)
+    with open(stamp, "w") as f:
+        f.write(want)
+    _log(f"built {lib}")
+    return lib
+
+
 def build_all(force: bool = True) -> None:
-    """Compile the core library and the attention libraries of the usual head sizes."""
+    """Compile the core library, the plain host twins and the attention libraries of the usual
+    head sizes."""
     ensure_core(force=force)
+    ensure_plain_host(force=force)
     if _existing(ATTN_SOURCES):
         with ThreadPoolExecutor(max_workers=_jobs()) as ex:
             list(ex.map(lambda hd: ensure_attention(hd, force=force), PREBUILT_HEAD_DIMS))

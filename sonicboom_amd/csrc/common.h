@@ -27,6 +27,16 @@ __device__ __forceinline__ float ld_f(const bf16_t *p, size_t i) { return bf16_t
 __device__ __forceinline__ void st_f(float *p, size_t i, float v) { p[i] = v; }
 __device__ __forceinline__ void st_f(bf16_t *p, size_t i, float v) { p[i] = f32_to_bf16(v); }
 
+// The gate's activation of a gated feed-forward, by the value of the products' `gated` argument:
+// SB_GATE_SILU g / (1 + exp(-g)) with the full-precision expf
+// (/root/reference/core/src/nn/activation.cpp:41-50); SB_GATE_GELU_TANH the tanh form of GELU,
+// 0.5 g (1 + tanh(sqrt(2/pi) g (1 + 0.044715 g^2))), constants and order of :27-36.
+__device__ __forceinline__ float gate_act(float g, int kind) {
+  if (kind == SB_GATE_GELU_TANH)
+    return 0.5f * g * (1.0f + tanhf(0.79788456080286535587989211986876f * g * (1.0f + 0.044715f * g * g)));
+  return g / (1.0f + expf(-g));
+}
+
 // Value of element i of a buffer whose type is only known at run time.
 __device__ __forceinline__ float ld_dyn(const void *p, int dtype, size_t i) {
   return dtype == SB_F32 ? ((const float *)p)[i] : bf16_to_f32(((const bf16_t *)p)[i]);

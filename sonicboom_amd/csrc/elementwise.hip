@@ -1,15 +1,15 @@
-// SiLU-gated product, residual add, type conversion.
+// Gated product, residual add, type conversion.
 //
-// silu(g) = g / (1 + expf(-g)) with the full-precision expf, then the product
-// with the up projection (/root/reference/core/src/nn/activation.cpp:41-50,
-// /root/reference/core/src/model/emit.cpp:364-374).
+// act(g) * u with the gate's activation (SiLU with the full-precision expf, or the tanh form
+// of GELU: gate_act in common.h), u the up projection
+// (/root/reference/core/src/nn/activation.cpp:27-50, /root/reference/core/src/model/emit.cpp:364-374).
 #include "common.h"
 
 namespace {
 
 template <typename TO, typename TI>
-__global__ void silu_mul_kernel(TO *__restrict__ out, const TI *__restrict__ gu, int width,
-                                size_t total) {
+__global__ void gate_mul_kernel(TO *__restrict__ out, const TI *__restrict__ gu, int width,
+                                size_t total, int gate) {
   const size_t idx = size_t(blockIdx.x) * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const size_t row = idx / width;
@@ -17,8 +17,7 @@ __global__ void silu_mul_kernel(TO *__restrict__ out, const TI *__restrict__ gu,
   const TI *g_row = gu + row * size_t(2 * width);
   const float g = ld_f(g_row, col);
   const float u = ld_f(g_row, size_t(width) + col);
-  const float act = g / (1.0f + expf(-g));
-  st_f(out, idx, act * u);
+  st_f(out, idx, gate_act(g, gate) * u);
 }
 
 template <typename TI>
@@ -37,22 +36,28 @@ inline unsigned blocks_for(size_t n, int threads) { return unsigned((n + threads
 
 }  // namespace
 
-extern "C" int sb_silu_mul(void *out, int out_dtype, const void *gu, int gu_dtype, int n_rows,
-                           int width, void *stream) {
-  SB_REQUIRE(out && gu, "sb_silu_mul: null pointer");
-  SB_REQUIRE(n_rows >= 0 && width > 0, "sb_silu_mul: bad sizes rows=%d width=%d", n_rows, width);
-  SB_REQUIRE(sb::valid_dtype(out_dtype) && sb::valid_dtype(gu_dtype), "sb_silu_mul: unknown dtype");
+extern "C" int sb_gate_mul(void *out, int out_dtype, const void *gu, int gu_dtype, int n_rows,
+                           int width, int gate, void *stream) {
+  SB_REQUIRE(out && gu, "sb_gate_mul: null pointer");
+  SB_REQUIRE(n_rows >= 0 && width > 0, "sb_gate_mul: bad sizes rows=%d width=%d", n_rows, width);
+  SB_REQUIRE(sb::valid_dtype(out_dtype) && sb::valid_dtype(gu_dtype), "sb_gate_mul: unknown dtype");
+  SB_SUPPORT(gate == SB_GATE_SILU || gate == SB_GATE_GELU_TANH, "sb_gate_mul: unknown gate activation %d", gate);
   const size_t total = size_t(n_rows) * width;
   if (total == 0) return SB_OK;
   hipStream_t s = (hipStream_t)stream;
   const unsigned nb = blocks_for(total, 256);
-#define SB_GO(TO, TI) silu_mul_kernel<TO, TI><<<nb, 256, 0, s>>>((TO *)out, (const TI *)gu, width, total)
+#define SB_GO(TO, TI) gate_mul_kernel<TO, TI><<<nb, 256, 0, s>>>((TO *)out, (const TI *)gu, width, total, gate)
   if (out_dtype == SB_F32 && gu_dtype == SB_F32) SB_GO(float, float);
   else if (out_dtype == SB_BF16 && gu_dtype == SB_F32) SB_GO(bf16_t, float);
   else if (out_dtype == SB_BF16 && gu_dtype == SB_BF16) SB_GO(bf16_t, bf16_t);
   else SB_GO(float, bf16_t);
 #undef SB_GO
-  return sb::check_launch("sb_silu_mul");
+  return sb::check_launch("sb_gate_mul");
+}
+
+extern "C" int sb_silu_mul(void *out, int out_dtype, const void *gu, int gu_dtype, int n_rows,
+                           int width, void *stream) {
+  return sb_gate_mul(out, out_dtype, gu, gu_dtype, n_rows, width, SB_GATE_SILU, stream);
 }
 
 extern "C" int sb_add_into(float *resid, const void *y, int y_dtype, size_t n, void *stream) {

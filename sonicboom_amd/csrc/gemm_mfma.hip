@@ -32,7 +32,7 @@ struct Args {
   int bias_dtype;
   const float *resid;
   int n_rows, n_out, n_in;
-  int gated;       // W is [2*n_out, n_in]: rows n (gate) and n_out + n (up)
+  int gated;       // an sb_gate; not 0: W is [2*n_out, n_in], rows n (gate) and n_out + n (up)
   int tiles_m, tiles_n;
   int w_tiles;     // packed W: 16-row tiles of one half (ceil(n_out / 16))
   int w_steps;     // packed W: 32-wide k-steps (ceil(n_in / 32))
@@ -48,7 +48,6 @@ __device__ __forceinline__ int swz(int row, int chunk) {
   return row * CPR + (chunk ^ ((row / (16 / CPR)) & (CPR - 1)));
 }
 
-__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
 // PACKED: W comes in the packed tile layout (1 KB blocks of 16 rows x 32 k in fragment order,
 // zero padded), which makes its global loads contiguous and free of bounds checks.
@@ -293,7 +292,7 @@ gemm_mfma_kernel(Args a) {
       if (GATED) {
         const int n = n0 + wn * 32 + col;
         if (n < a.n_out) {
-          const float v = silu_f(acc[i][0][e]) * acc[i][1][e];
+          const float v = gate_act(acc[i][0][e], GATED) * acc[i][1][e];     // GATED: the sb_gate, fixed at compile time
           const size_t idx = size_t(t) * a.n_out + n;
           if (a.y_dtype == SB_F32) ((float *)a.y)[idx] = v;
           else ((bf16_t *)a.y)[idx] = f32_to_bf16(v);
@@ -338,8 +337,11 @@ int launch_one(const Args &a, long long blocks, hipStream_t s) {
 
 template <int MT, int NW, int BK, int DEPTH, bool PLAIN_TOO>
 int launch(const Args &a, long long blocks, int packed, hipStream_t s) {
-  const int which = (a.gated ? 4 : 0) + (packed ? 2 : 0) + (a.n_in % BK == 0 ? 1 : 0);
+  // the gate's activation is a template argument: the SiLU kernels hold no code of the others
+  const int which = a.gated * 4 + (packed ? 2 : 0) + (a.n_in % BK == 0 ? 1 : 0);
   switch (which) {
+    case 11: return launch_one<MT, NW, BK, DEPTH, 2, true, true>(a, blocks, s);
+    case 10: return launch_one<MT, NW, BK, DEPTH, 2, true, false>(a, blocks, s);
     case 7: return launch_one<MT, NW, BK, DEPTH, 1, true, true>(a, blocks, s);
     case 6: return launch_one<MT, NW, BK, DEPTH, 1, true, false>(a, blocks, s);
     case 3: return launch_one<MT, NW, BK, DEPTH, 0, true, true>(a, blocks, s);
@@ -348,6 +350,8 @@ int launch(const Args &a, long long blocks, int packed, hipStream_t s) {
   }
   if constexpr (PLAIN_TOO) {
     switch (which) {
+      case 9: return launch_one<MT, NW, BK, DEPTH, 2, false, true>(a, blocks, s);
+      case 8: return launch_one<MT, NW, BK, DEPTH, 2, false, false>(a, blocks, s);
       case 5: return launch_one<MT, NW, BK, DEPTH, 1, false, true>(a, blocks, s);
       case 4: return launch_one<MT, NW, BK, DEPTH, 1, false, false>(a, blocks, s);
       case 1: return launch_one<MT, NW, BK, DEPTH, 0, false, true>(a, blocks, s);
@@ -361,14 +365,25 @@ int launch(const Args &a, long long blocks, int packed, hipStream_t s) {
 struct Shape { int bm, bn; };
 constexpr Shape kShapes[3] = {{128, 128}, {256, 128}, {256, 256}};
 
-// Rough cost of a shape for a problem: rounds of the grid over the CUs times the work of a block,
-// the bigger tiles getting credit for the operand traffic they save.
-int pick_shape(int n_rows, int n_out, int gated) {
+// The tile shape for a problem, from what was measured on MI355X (cold weights, 2,048 to 16,384
+// rows).  The gated product (a wide matrix, SiLU epilogue): rounds of the grid over the CUs times
+// the work of a block, the bigger tiles getting credit for the operand traffic they save; that
+// ends at 256 x 256 for every size tried.  Plain products against narrower matrices: two blocks
+// of 128 x 128 share a CU (64 KB of LDS and 128 registers each), one block's first loads and
+// epilogue hide behind the other's loop, and with an inner size of a few thousand that beats the
+// lone 256 x 128 block by 7 to 47 % (output product of 3,584 x 3,584 at 16,384 rows: 618 against
+// 910 us); only a long inner size with few blocks (the down product up to 4,096 rows) is better
+// off with 256 x 128, by 10 %.
+int pick_shape(int n_rows, int n_out, int n_in, int gated) {
+  if (!gated) {
+    const long long blocks_1 = (long long)((n_rows + 255) / 256) * ((n_out + 127) / 128);
+    return (n_in >= 8192 && blocks_1 <= 2 * kCus) ? 1 : 0;
+  }
   double best = 0;
   int pick = 0;
   const double speed[3] = {1.0, 1.2, 1.3};    // measured rate of a full grid, relative
   for (int v = 0; v < 3; ++v) {
-    const int bn = gated ? kShapes[v].bn / 2 : kShapes[v].bn;
+    const int bn = kShapes[v].bn / 2;
     const long long blocks = (long long)((n_rows + kShapes[v].bm - 1) / kShapes[v].bm) * ((n_out + bn - 1) / bn);
     const long long rounds = (blocks + kCus - 1) / kCus;
     const double cost = double(rounds) * kShapes[v].bm * kShapes[v].bn / speed[v];
@@ -394,13 +409,14 @@ extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void
   SB_SUPPORT((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w)) % 16 == 0,
              "sb_gemm_mfma_bf16: operands must be 16-byte aligned");
   SB_REQUIRE(!(gated && (bias || resid)), "sb_gemm_mfma_bf16: the gated form takes no bias or residual");
+  SB_SUPPORT(gated >= SB_GATE_NONE && gated <= SB_GATE_GELU_TANH, "sb_gemm_mfma_bf16: unknown gate activation %d", gated);
   if (n_rows == 0) return SB_OK;
   Args a;
   a.y = y; a.y_dtype = y_dtype; a.x = (const bf16_t *)x; a.w = (const bf16_t *)w;
   a.bias = bias; a.bias_dtype = bias_dtype; a.resid = resid;
-  a.n_rows = n_rows; a.n_out = n_out; a.n_in = n_in; a.gated = gated ? 1 : 0;
+  a.n_rows = n_rows; a.n_out = n_out; a.n_in = n_in; a.gated = gated;
   a.partial = nullptr; a.stages_per_slice = 0;
-  int variant = pick_shape(n_rows, n_out, a.gated);
+  int variant = pick_shape(n_rows, n_out, n_in, a.gated);
   if (tile_shape >= 0 && tile_shape < 3) variant = tile_shape;      // a test's or a measurement's choice
   if (!packed) variant = 0;       // the bigger tiles are built for packed weights only
   const int bm = kShapes[variant].bm, bn = gated ? kShapes[variant].bn / 2 : kShapes[variant].bn;

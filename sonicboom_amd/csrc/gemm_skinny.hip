@@ -31,7 +31,6 @@ struct Epilogue {
   int gated;
 };
 
-__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
 __device__ __forceinline__ void store_out(const Epilogue &e, int t, int n, float v) {
   if (e.bias) v = v + ld_dyn(e.bias, e.bias_dtype, n);
@@ -163,7 +162,7 @@ gemm_skinny_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ w, E
       for (int c = 0; c < 4; ++c) {
         if (nb + c >= ep.n_out) continue;
         float val = v[0][c];
-        if (G == 2) val = silu_f(val) * v[1][c];
+        if (G == 2) val = gate_act(val, ep.gated) * v[1][c];
         store_out(ep, t, nb + c, val);
       }
     }
@@ -183,7 +182,7 @@ reduce_slices_kernel(const float *__restrict__ partial, Epilogue ep, int n_slice
     g += p[n];
     if (ep.gated) u += p[ep.n_out + n];
   }
-  store_out(ep, t, n, ep.gated ? silu_f(g) * u : g);
+  store_out(ep, t, n, ep.gated ? gate_act(g, ep.gated) * u : g);
 }
 
 template <int R, int TT, int G, bool PACKED>
@@ -285,7 +284,8 @@ extern "C" int sb_gemm_skinny_bf16(void *y, int y_dtype, const void *x, const vo
   SB_REQUIRE(need == 0 || (scratch && scratch_floats >= need),
              "sb_gemm_skinny_bf16: scratch of %zu floats needed, %zu given", need, scratch_floats);
   hipStream_t s = (hipStream_t)stream;
-  Epilogue ep{y, y_dtype, bias, bias_dtype, resid, n_rows, n_out, gated ? 1 : 0};
+  SB_SUPPORT(gated >= SB_GATE_NONE && gated <= SB_GATE_GELU_TANH, "sb_gemm_skinny_bf16: unknown gate activation %d", gated);
+  Epilogue ep{y, y_dtype, bias, bias_dtype, resid, n_rows, n_out, gated};
   float *partial = p.n_slices > 1 ? scratch : nullptr;
   const bf16_t *xb = (const bf16_t *)x, *wb = (const bf16_t *)w;
   if (gated && packed) launch_rt<2, true>(p.R, p.TT, xb, wb, ep, partial, n_in, p.n_slices, p.steps_per_slice, s);

@@ -43,9 +43,9 @@ struct StreamArgs {
   // one slice and the epilogues below
   float *partial;
   int steps_per_slice;
+  int gate;        // the gate's activation (an sb_gate) of the gated form
 };
 
-__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
 
 template <int TT, int G, int R, int W>
 __global__ void __launch_bounds__(64 * W)
@@ -174,7 +174,7 @@ gemm_stream_kernel(const bf16_t *__restrict__ x, const bf16_t *__restrict__ w, S
         const int n = nb + e;
         if (n >= a.n_out) continue;
         float v = acc[i][j][e];
-        if (G == 2) v = silu_f(v) * acc[R + i][j][e];
+        if (G == 2) v = gate_act(v, a.gate) * acc[R + i][j][e];
         if (a.bias) v = v + ld_dyn(a.bias, a.bias_dtype, n);
         if (a.resid) v = v + a.resid[row_off + n];
         if (a.y_dtype == SB_F32) ((float *)a.y)[row_off + n] = v;
@@ -295,7 +295,8 @@ extern "C" int sb_gemm_stream_bf16(void *y, int y_dtype, const void *x, const vo
              "sb_gemm_stream_bf16: inner size %d is too large", n_in);
   if (n_rows == 0) return SB_OK;
   hipStream_t s = (hipStream_t)stream;
-  const StreamArgs a{y, y_dtype, bias, bias_dtype, resid, n_rows, n_out, n_in, nullptr, 0};
+  SB_SUPPORT(gated >= SB_GATE_NONE && gated <= SB_GATE_GELU_TANH, "sb_gemm_stream_bf16: unknown gate activation %d", gated);
+  const StreamArgs a{y, y_dtype, bias, bias_dtype, resid, n_rows, n_out, n_in, nullptr, 0, gated};
   const bf16_t *xb = (const bf16_t *)x, *wb = (const bf16_t *)w;
   const int tt = row_tiles(n_rows);
   if (gated) {
@@ -332,7 +333,7 @@ extern "C" int sb_gemm_stream_partial_bf16(float *partial, const void *x, const 
              "sb_gemm_stream_partial_bf16: inner size %d is too large", n_in);
   if (n_rows == 0) return SB_OK;
   const Cut c = cut_for((n_out + 15) / 16, (n_in + kStepK - 1) / kStepK, row_tiles(n_rows), hint);
-  const StreamArgs a{nullptr, SB_F32, nullptr, 0, nullptr, n_rows, n_out, n_in, partial, c.steps_per_slice};
+  const StreamArgs a{nullptr, SB_F32, nullptr, 0, nullptr, n_rows, n_out, n_in, partial, c.steps_per_slice, 0};
   const bf16_t *xb = (const bf16_t *)x, *wb = (const bf16_t *)w;
   hipStream_t s = (hipStream_t)stream;
   if (n_rows <= 16) launch_cut<1>(xb, wb, a, c.waves, s);

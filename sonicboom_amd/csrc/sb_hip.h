@@ -37,6 +37,10 @@ typedef enum sb_status {
 
 typedef enum sb_dtype { SB_F32 = 0, SB_BF16 = 1 } sb_dtype;
 
+/* The `gated` argument of the products and of sb_gate_mul: not gated, or the activation of the
+ * gate in Y = act(X Wg^T) * (X Wu^T). */
+typedef enum sb_gate { SB_GATE_NONE = 0, SB_GATE_SILU = 1, SB_GATE_GELU_TANH = 2 } sb_gate;
+
 /* Message of this thread's last failed call ("" if none). Never NULL. */
 const char *sb_last_error(void);
 /* A JSON object naming the target architecture, the page size and the build flags. */
@@ -64,7 +68,11 @@ int sb_gemm(void *y, int y_dtype, const void *x, int x_dtype, const void *w, int
             const void *bias, int bias_dtype, const float *resid,
             int n_rows, int n_out, int n_in, void *stream);
 
-/* out[t,i] = silu(gu[t,i]) * gu[t,width+i];  gu is [t, 2*width]. */
+/* out[t,i] = act(gu[t,i]) * gu[t,width+i];  gu is [t, 2*width]; gate: SB_GATE_SILU or
+ * SB_GATE_GELU_TANH. */
+int sb_gate_mul(void *out, int out_dtype, const void *gu, int gu_dtype, int n_rows, int width, int gate,
+                void *stream);
+/* The same with the SiLU gate. */
 int sb_silu_mul(void *out, int out_dtype, const void *gu, int gu_dtype,
                 int n_rows, int width, void *stream);
 
@@ -149,7 +157,8 @@ int sb_top_candidates(int32_t *cand_id, float *cand_z, const float *logits, int 
  * aligned.  W bf16 [n_out, n_in] row-major, or (packed != 0, or always for the
  * stream kernel) re-laid in 16 x 32 tiles of 1 KB in MFMA fragment order, rows
  * padded to 16 and k to 32, tiles of a row block consecutive in k; gated: the two
- * halves [gate; up] packed one after the other, Y = silu(X Wg^T) * (X Wu^T).
+ * halves [gate; up] packed one after the other, Y = act(X Wg^T) * (X Wu^T) with the activation
+ * that `gated` names (an sb_gate).
  * Y f32 or bf16; bias [n_out] f32 or bf16 or NULL; resid f32 [n_rows, n_out] or
  * NULL (may be Y itself).  The *_partial_* forms write the raw product in K
  * slices, f32 [slices][n_rows][n_out], slices as the matching *_slices says. */

@@ -127,16 +127,36 @@ def gemm_plain(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], r
     return out
 
 
-def silu_mul(gu: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-    """silu(gu[:, :w]) * gu[:, w:] for gu [n, 2w]."""
+GATES = {"silu": 1, "gelu_tanh": 2}      # sb_gate of csrc/sb_hip.h
+
+
+def gate_code(activation) -> int:
+    """The kernels' number of a gate activation given by name (or already by number)."""
+    if isinstance(activation, bool):
+        return 1 if activation else 0
+    if isinstance(activation, int):
+        return activation
+    try:
+        return GATES[activation]
+    except KeyError:
+        raise KernelLibraryError(f"unknown gate activation {activation!r}; known: {sorted(GATES)}") from None
+
+
+def gate_mul(gu: torch.Tensor, out_dtype: torch.dtype, activation="silu") -> torch.Tensor:
+    """act(gu[:, :w]) * gu[:, w:] for gu [n, 2w]; ``activation``: "silu" or "gelu_tanh"."""
     _dev(gu)
     if gu.dim() != 2 or gu.shape[1] % 2:
-        raise KernelLibraryError("silu_mul input must be [rows, 2*width]")
+        raise KernelLibraryError("gate_mul input must be [rows, 2*width]")
     n, w2 = gu.shape
     out = torch.empty((n, w2 // 2), dtype=out_dtype, device=gu.device)
     lib = library.core()
-    check(lib.sb_silu_mul(_p(out), _dt(out), _p(gu), _dt(gu), n, w2 // 2, _stream()))
+    check(lib.sb_gate_mul(_p(out), _dt(out), _p(gu), _dt(gu), n, w2 // 2, gate_code(activation), _stream()))
     return out
+
+
+def silu_mul(gu: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """silu(gu[:, :w]) * gu[:, w:] for gu [n, 2w]."""
+    return gate_mul(gu, out_dtype, "silu")
 
 
 def add_into(resid: torch.Tensor, y: torch.Tensor) -> None:
@@ -404,7 +424,7 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], re
               out_dtype: torch.dtype, out: Optional[torch.Tensor] = None, gated: bool = False,
               packed_shape=None) -> Optional[torch.Tensor]:
     """bfloat16 product on the matrix cores: y = x w^T (+bias) (+resid), or with ``gated``
-    y = silu(x wg^T) * (x wu^T) for w = [wg; wu].  Up to 64 rows go to one of the two
+    (True or "silu", or "gelu_tanh") y = act(x wg^T) * (x wu^T) for w = [wg; wu].  Up to 64 rows go to one of the two
     weight-streaming kernels, more to the tiled one.  ``packed_shape`` = (rows of w, inner size) says that ``w`` is
     in the layout of :func:`pack_weight`.  Returns None when the sizes fit neither kernel (an
     inner size that is not a multiple of 8): the caller then takes the plain kernel."""
@@ -415,6 +435,7 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], re
     if x.dim() != 2 or x.shape[1] != w_k or (packed_shape is None and w.dim() != 2):
         raise KernelLibraryError(f"gemm shapes do not match: x {tuple(x.shape)}, w {(w_rows, w_k)}")
     t, k = x.shape
+    gate = gate_code(gated)
     n = w_rows // 2 if gated else w_rows
     if k % 8 or x.data_ptr() % 16 or w.data_ptr() % 16 or (gated and w_rows % 2):
         return None
@@ -445,15 +466,15 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], re
                 which = "tiled"
     if t <= STREAM_MAX_ROWS and which == "stream" and packed:
         check(lib.sb_gemm_stream_bf16(_p(out), _dt(out), _p(x), _p(w), _p(bias), bdt, _p(resid), t, n, k,
-                                      1 if gated else 0, _hints.stream, _stream()))
+                                      gate, _hints.stream, _stream()))
     elif t <= SKINNY_MAX_ROWS and which != "tiled":
-        need = lib.sb_gemm_skinny_scratch(t, n, k, 1 if gated else 0)
+        need = lib.sb_gemm_skinny_scratch(t, n, k, gate)
         scratch = torch.empty((need,), dtype=torch.float32, device=x.device) if need else None
         check(lib.sb_gemm_skinny_bf16(_p(out), _dt(out), _p(x), _p(w), _p(bias), bdt, _p(resid), t, n, k,
-                                      1 if gated else 0, packed, _p(scratch), need, _stream()))
+                                      gate, packed, _p(scratch), need, _stream()))
     else:
         check(lib.sb_gemm_mfma_bf16(_p(out), _dt(out), _p(x), _p(w), _p(bias), bdt, _p(resid), t, n, k,
-                                    1 if gated else 0, packed, _hints.tile_shape, _stream()))
+                                    gate, packed, _hints.tile_shape, _stream()))
     return out
 
 

@@ -23,6 +23,7 @@ _CORE_SIGNATURES = {
     "sb_rmsnorm": [_P, _I, _P, _P, _I, _P, _I, _I, _F, _P],
     "sb_gemm": [_P, _I, _P, _I, _P, _I, _P, _I, _P, _I, _I, _I, _P],
     "sb_silu_mul": [_P, _I, _P, _I, _I, _I, _P],
+    "sb_gate_mul": [_P, _I, _P, _I, _I, _I, _I, _P],
     "sb_add_into": [_P, _P, _I, _Z, _P],
     "sb_cast": [_P, _I, _P, _I, _Z, _P],
     "sb_rope_kv_store": [_P, _I, _P, _I, _I, _I, _P, _P, _P, _I, _P, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],

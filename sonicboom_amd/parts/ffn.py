@@ -1,8 +1,9 @@
 """Gated dense feed-forward: y = W_down (act(W_gate f) * (W_up f)).
 
 /root/reference/core/src/model/emit.cpp:364-374; the activation is a parameter
-of the spec ("silu": g / (1 + exp(-g)),
-/root/reference/core/src/nn/activation.cpp:41-50).  The gate and up matrices
+of the spec: "silu", g / (1 + exp(-g)) (/root/reference/core/src/nn/activation.cpp:41-50),
+or "gelu_tanh", 0.5 g (1 + tanh(sqrt(2/pi) g (1 + 0.044715 g^2))) (:27-36); the product
+kernels apply either in their epilogue.  The gate and up matrices
 are stacked into one [2*inner, width] matrix when the part is built, so a
 step runs one product for both; its float32 result feeds the activation
 kernel, whose output is rounded once to the activation type.
@@ -15,7 +16,7 @@ from .base import Part, register_part
 from .linear import Linear
 from .spec import PartSpec, TensorSpec
 
-ACTIVATIONS = ("silu",)
+ACTIVATIONS = ("silu", "gelu_tanh")    # the gates the product kernels apply in their epilogue
 
 
 def gated_ffn_spec(prefix: str, width: int, inner: int, activation: str = "silu") -> PartSpec:
@@ -40,7 +41,8 @@ class GatedDenseFFN(Part):
         g, u = tensors["gate_weight"], tensors["up_weight"]
         if g.dtype != u.dtype:
             g, u = g.float(), u.float()
-        self.gate_up = Linear(torch.cat([g, u], dim=0), None, rt.fast_kernels, gated=True)
+        self.gate_up = Linear(torch.cat([g, u], dim=0), None, rt.fast_kernels, gated=True,
+                              activation=self.activation)
         self.down = Linear(tensors["down_weight"], None, rt.fast_kernels)
 
     fuses_norm = True

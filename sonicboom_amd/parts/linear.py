@@ -13,7 +13,7 @@ call this helper, which picks the kernel from the types and sizes at hand:
   weight and the plain kernel.
 
 ``gated=True`` marks a stacked weight [W_gate; W_up] whose product is
-silu(x W_gate^T) * (x W_up^T).
+act(x W_gate^T) * (x W_up^T), ``activation`` naming the gate's ("silu" or "gelu_tanh").
 """
 from __future__ import annotations
 
@@ -26,10 +26,12 @@ from .. import ops
 
 class Linear:
     def __init__(self, weight: torch.Tensor, bias: Optional[torch.Tensor], fast: bool = True,
-                 gated: bool = False):
+                 gated: bool = False, activation: str = "silu"):
         if weight.dim() != 2:
             raise ValueError("a projection weight must be [out, in]")
         self.gated = gated
+        self.activation = activation
+        ops.gate_code(activation)             # an unknown name is refused when the part is built
         self.rows, self.n_in = weight.shape
         self.n_out = self.rows // 2 if gated else self.rows
         if gated and self.rows % 2:
@@ -82,14 +84,14 @@ class Linear:
         return None
 
     def gated_product(self, x: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
-        """silu(x Wg^T) * (x Wu^T): one fused kernel on the matrix cores, or the product in
+        """act(x Wg^T) * (x Wu^T): one fused kernel on the matrix cores, or the product in
         float32 followed by the activation kernel."""
         if self.packed is not None:
             if x.dtype != torch.bfloat16:
                 x = ops.cast(x, torch.bfloat16)
-            return ops.gemm_bf16(x, self.packed, None, None, out_dtype, gated=True,
+            return ops.gemm_bf16(x, self.packed, None, None, out_dtype, gated=self.activation,
                                  packed_shape=(self.rows, self.n_in))
         w = self._row_major()
         if w.dtype == torch.float32 and x.dtype != torch.float32:
             x = ops.cast(x, torch.float32)
-        return ops.silu_mul(ops.gemm_plain(x, w, None, None, torch.float32), out_dtype)
+        return ops.gate_mul(ops.gemm_plain(x, w, None, None, torch.float32), out_dtype, self.activation)

@@ -1,0 +1,188 @@
+"""Every kernel against its plain C++ twin on host memory (sonicboom_amd/csrc/plain_host.cpp),
+at sizes other than the engine's.  The twins themselves are pinned, without a GPU, by the
+reference's vectors and by the NumPy implementation (test_host_twins_agree_with_the_plain_implementation)."""
+import ctypes
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from plain import qwen2_plain as P
+
+F32, BF16 = torch.float32, torch.bfloat16
+DEV = "cuda:0"
+
+
+def twins():
+    from sonicboom_amd.csrc import build
+    lib = ctypes.CDLL(build.ensure_plain_host())
+    for name in ("sbp_embed", "sbp_rmsnorm", "sbp_reduce_resid_norm", "sbp_gemm", "sbp_silu_mul", "sbp_add_into",
+                 "sbp_rope_kv_store", "sbp_attention", "sbp_argmax"):
+        getattr(lib, name).restype = ctypes.c_int
+    return lib
+
+
+def ptr(a):
+    return None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+
+
+def f32(*shape, seed=0, scale=1.0):
+    return (np.random.default_rng(seed).standard_normal(shape) * scale).astype(np.float32)
+
+
+def i32(values):
+    return np.ascontiguousarray(values, dtype=np.int32)
+
+
+C = ctypes.c_int
+
+
+def host_gemm(lib, x, w, bias=None, resid=None):
+    y = np.empty((x.shape[0], w.shape[0]), np.float32)
+    assert lib.sbp_gemm(ptr(y), ptr(x), ptr(w), ptr(bias), ptr(resid), C(x.shape[0]), C(w.shape[0]), C(x.shape[1])) == 0
+    return y
+
+
+def host_rmsnorm(lib, x, w, eps, rows=None):
+    n = x.shape[0] if rows is None else len(rows)
+    y = np.empty((n, x.shape[1]), np.float32)
+    assert lib.sbp_rmsnorm(ptr(y), ptr(x), ptr(w), ptr(rows), C(n), C(x.shape[1]), ctypes.c_float(eps)) == 0
+    return y
+
+
+def host_paged(lib, qkv, bias, inv_freq, ff, rot, pos, seq, table, n_pages, hq, hkv, hd):
+    """(q, k_cache, v_cache) of the rotate-and-store twin on empty caches."""
+    n = qkv.shape[0]
+    q = np.empty((n, hq * hd), np.float32)
+    kc = np.zeros((n_pages, hkv, 64, hd), np.float32)
+    vc = np.zeros((n_pages, hkv, hd, 64), np.float32)
+    assert lib.sbp_rope_kv_store(ptr(q), ptr(qkv), C(qkv.shape[1]), ptr(bias), ptr(inv_freq), ptr(ff), C(rot),
+                                 ptr(pos), ptr(seq), ptr(kc), ptr(vc), ptr(table), C(table.shape[1]), C(n_pages),
+                                 C(n), C(hq), C(hkv), C(hd)) == 0
+    return q, kc, vc
+
+
+def host_attention(lib, q, kc, vc, table, pos, seq, hq, hkv, hd, scale, window):
+    out = np.empty((q.shape[0], hq * hd), np.float32)
+    assert lib.sbp_attention(ptr(out), ptr(q), C(q.shape[1]), ptr(kc), ptr(vc), ptr(table), C(table.shape[1]),
+                             C(kc.shape[0]), ptr(pos), ptr(seq), C(q.shape[0]), C(hq), C(hkv), C(hd),
+                             ctypes.c_float(scale), C(window)) == 0
+    return out
+
+
+# ---- the twins themselves, without a GPU -------------------------------------------------------
+def test_host_twins_agree_with_the_plain_implementation():
+    lib = twins()
+    # norm: the reference's vectors (/root/reference/tests/core/test_nn.cpp:172-219), then NumPy
+    assert np.allclose(host_rmsnorm(lib, np.full((1, 4), 2, np.float32), None, 0.0), 1.0, atol=1e-6)
+    assert np.array_equal(host_rmsnorm(lib, np.array([[1, 0, 0, 0]], np.float32), None, 0.75), [[1, 0, 0, 0]])
+    x, w = f32(5, 201, seed=1, scale=3.0), f32(201, seed=2)
+    assert np.allclose(host_rmsnorm(lib, x, w, 1e-5), P.rms_norm(x, w, 1e-5), atol=1e-6)
+    assert np.array_equal(host_rmsnorm(lib, x, w, 1e-5, i32([4, 0])), host_rmsnorm(lib, x, w, 1e-5)[[4, 0]])
+    # product, bias, residual
+    x, w, b, r = f32(7, 50, seed=3), f32(13, 50, seed=4), f32(13, seed=5), f32(7, 13, seed=6)
+    assert np.allclose(host_gemm(lib, x, w, b, r), P.linear(x, w, b) + r, atol=1e-5)
+    # silu * up
+    gu = f32(3, 24, seed=7, scale=3.0)
+    out = np.empty((3, 12), np.float32)
+    assert lib.sbp_silu_mul(ptr(out), ptr(gu), C(3), C(12)) == 0
+    assert np.allclose(out, P.silu(gu[:, :12]) * gu[:, 12:], atol=1e-6)
+    # rotation (pairs (i, i + half): the vector of test_nn.cpp:221-290), store, attention
+    hq, hkv, hd = 4, 2, 8
+    inv = np.exp(-2.0 * np.arange(hd // 2, dtype=np.float32) / hd * np.log(np.float32(1e4))).astype(np.float32)
+    pos, seq = i32([0, 1, 2, 70, 0]), i32([0, 0, 0, 1, 1])
+    table = i32([[2, 5], [1, 0]])
+    qkv, bias = f32(5, (hq + 2 * hkv) * hd, seed=8), f32((hq + 2 * hkv) * hd, seed=9, scale=0.1)
+    q, kc, vc = host_paged(lib, qkv, bias, inv, None, hd, pos, seq, table, 6, hq, hkv, hd)
+    full = qkv + bias
+    assert np.allclose(q, P.rope_neox(full[:, :hq * hd], pos, hd, 1e4), atol=1e-6)
+    k_want = P.rope_neox(full[:, hq * hd:(hq + hkv) * hd], pos, hd, 1e4).reshape(5, hkv, hd)
+    assert np.allclose(kc[2, :, 1, :], k_want[1], atol=1e-6) and np.allclose(kc[0, :, 6, :], k_want[3], atol=1e-6)
+    assert np.array_equal(vc[1, :, :, 0], full[4, (hq + hkv) * hd:].reshape(hkv, hd))
+    y = np.array([[1.0, 0.0, 2.0, 3.0] * 3], np.float32)
+    quarter = np.full(2, math.pi / 2, np.float32)
+    qq, _, _ = host_paged(lib, y, None, quarter, None, 4, i32([1]), i32([0]), i32([[0]]), 1, 1, 1, 4)
+    assert np.allclose(qq, [[-2.0, -3.0, 1.0, 0.0]], atol=1e-6)
+    # attention over the three keys of sequence 0, against the plain routine; a window of 2 drops key 0
+    for window in (0, 2):
+        got = host_attention(lib, q[:3], kc, vc, table, pos[:3], seq[:3], hq, hkv, hd, 0.35, window)
+        v_rows = full[:3, (hq + hkv) * hd:]
+        want = P.attention(q[:3], k_want[:3].reshape(3, -1), v_rows, pos[:3], pos[:3], hq, hkv, hd, 0.35, window=window)
+        assert np.allclose(got, want, atol=1e-6)
+    ids = np.empty(3, np.int32)
+    logits = np.array([[0.5, 0.5, 0.1], [1, 3, 3], [-np.inf] * 3], np.float32)
+    assert lib.sbp_argmax(ptr(ids), ptr(logits), C(3), C(3)) == 0 and ids.tolist() == [0, 1, 0]
+
+
+# ---- kernels against twins ---------------------------------------------------------------------
+@pytest.mark.gpu
+def test_kernels_equal_their_host_twins():
+    from sonicboom_amd import ops
+    lib = twins()
+    dev = lambda a, dt=None: None if a is None else torch.from_numpy(a).to(DEV if dt is None else DEV).to(dt or torch.from_numpy(a).dtype)  # noqa: E731
+    # embedding
+    table, ids = f32(37, 50, seed=1), i32([0, 36, 5, 5])
+    want = np.empty((4, 50), np.float32)
+    assert lib.sbp_embed(ptr(want), ptr(table), ptr(ids), C(4), C(50), C(37)) == 0
+    assert np.array_equal(ops.embed(dev(table), dev(ids)).cpu().numpy(), want)
+    # norm, float32 out: to rounding of the sum's order; rows picked
+    for width, n_rows in ((96, 3), (3584, 5), (1001, 300)):
+        x, w = f32(n_rows, width, seed=width, scale=2.0), f32(width, seed=2)
+        got = ops.rmsnorm(dev(x), dev(w), 1e-6, F32).cpu().numpy()
+        assert np.allclose(got, host_rmsnorm(lib, x, w, 1e-6), atol=1e-6, rtol=1e-6), width
+    rows = i32([2, 0])
+    assert np.allclose(ops.rmsnorm(dev(x), dev(w), 1e-6, F32, dev(rows)).cpu().numpy(),
+                       host_rmsnorm(lib, x, w, 1e-6, rows), atol=1e-6, rtol=1e-6)
+    # the plain product: the same fused multiply-adds in the same order, equal to the bit
+    for t, n, k in ((3, 70, 33), (65, 17, 128), (9, 300, 1000)):
+        x, w, b, r = f32(t, k, seed=t), f32(n, k, seed=n), f32(n, seed=3), f32(t, n, seed=4)
+        got = ops.gemm_plain(dev(x), dev(w), dev(b), dev(r), F32).cpu().numpy()
+        assert np.array_equal(got, host_gemm(lib, x, w, b, r)), (t, n, k)
+    # the matrix-core products (bf16 operands, float sums) against the twin on the same rounded operands
+    for t, n, k in ((8, 512, 256), (40, 200, 264), (300, 384, 512)):
+        x = torch.from_numpy(f32(t, k, seed=5)).to(BF16)
+        w = torch.from_numpy(f32(n, k, seed=6, scale=0.05)).to(BF16)
+        want = host_gemm(lib, x.float().numpy(), w.float().numpy())
+        got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(w.to(DEV)), None, None, F32, packed_shape=(n, k))
+        assert np.allclose(got.cpu().numpy(), want, atol=2e-3, rtol=2e-3), (t, n, k)
+    # slices + bias + residual + norm in one pass
+    part, b, x, w = f32(3, 6, 256, seed=7), f32(256, seed=8), f32(6, 256, seed=9), f32(256, seed=10)
+    x_host, y_host = x.copy(), np.empty((6, 256), np.float32)
+    assert lib.sbp_reduce_resid_norm(ptr(y_host), ptr(x_host), ptr(part), C(3), ptr(b), ptr(w), C(6), C(256),
+                                     ctypes.c_float(1e-5), C(1)) == 0
+    x_dev = dev(x)
+    y_dev = ops.reduce_resid_norm(dev(part), dev(b), x_dev, dev(w), 1e-5, F32)
+    assert np.array_equal(x_dev.cpu().numpy(), x_host) and np.allclose(y_dev.cpu().numpy(), y_host, atol=1e-6)
+    # silu * up, add
+    gu = f32(5, 2 * 77, seed=11, scale=3.0)
+    want = np.empty((5, 77), np.float32)
+    lib.sbp_silu_mul(ptr(want), ptr(gu), C(5), C(77))
+    assert np.allclose(ops.silu_mul(dev(gu), F32).cpu().numpy(), want, atol=1e-6, rtol=1e-6)
+    # rotate-and-store, then attention over what was stored: both kernels against both twins
+    for hq, hkv, hd, rot in ((6, 2, 48, 48), (4, 4, 64, 32), (8, 1, 128, 128)):
+        lens = [130, 3, 64]
+        table = i32([[4, 0, 7], [1, -1, -1], [5, -1, -1]])
+        pos = i32(np.concatenate([np.arange(n) for n in lens]))
+        seq = i32(np.concatenate([np.full(n, s) for s, n in enumerate(lens)]))
+        width = (hq + 2 * hkv) * hd
+        qkv, bias = f32(len(pos), width, seed=hd), f32(width, seed=12, scale=0.2)
+        inv = np.exp(-2.0 * np.arange(rot // 2, dtype=np.float32) / rot * np.log(np.float32(5e4))).astype(np.float32)
+        ff = (1.0 + np.arange(rot // 2, dtype=np.float32) / rot).astype(np.float32)
+        q_h, kc_h, vc_h = host_paged(lib, qkv, bias, inv, ff, rot, pos, seq, table, 8, hq, hkv, hd)
+        kc = torch.zeros((8, hkv, 64, hd), device=DEV)
+        vc = torch.zeros((8, hkv, hd, 64), device=DEV)
+        q_d = ops.rope_kv_store(dev(qkv), F32, dev(inv), dev(ff), rot, dev(pos), dev(seq), kc, vc, dev(table), hq, hkv,
+                                hd, bias=dev(bias))
+        for got, want in ((q_d, q_h), (kc, kc_h), (vc, vc_h)):
+            assert np.allclose(got.cpu().numpy(), want, atol=2e-5, rtol=1e-5), (hq, hkv, hd)
+        for window in (0, 50):
+            want = host_attention(lib, q_h, kc_h, vc_h, table, pos, seq, hq, hkv, hd, hd ** -0.5, window)
+            got = ops.attention_plain(q_d, kc, vc, dev(table), dev(pos), dev(seq), hq, hkv, hd, hd ** -0.5, window)
+            assert np.allclose(got.cpu().numpy(), want, atol=1e-5, rtol=1e-4), (hq, hkv, hd, window)
+    # the first maximum
+    logits = f32(4, 20001, seed=13)
+    logits[1, 7] = logits[1, 15000] = 9.0
+    ids = np.empty(4, np.int32)
+    lib.sbp_argmax(ptr(ids), ptr(logits), C(4), C(20001))
+    assert ops.argmax(dev(logits)).cpu().numpy().tolist() == ids.tolist() and ids[1] == 7

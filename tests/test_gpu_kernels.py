@@ -159,6 +159,38 @@ def test_gemm_bf16_gated(t, inner, k):
     close(got, want, atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"gated t={t}")
 
 
+def gelu_tanh(g):
+    """0.5 g (1 + tanh(sqrt(2/pi) g (1 + 0.044715 g^2))), /root/reference/core/src/nn/activation.cpp:27-36."""
+    return 0.5 * g * (1.0 + torch.tanh(0.7978845608028654 * g * (1.0 + 0.044715 * g * g)))
+
+
+@pytest.mark.parametrize("t", [1, 8, 40, 64, 65, 128, 300])
+def test_gemm_bf16_gate_activations(t):
+    """The gate's activation is an argument of every product kernel and of the elementwise
+    kernel: SiLU and the tanh form of GELU, through the stream, the K-splitting and the tiled
+    kernels, against the formula and against torch's own GELU."""
+    from sonicboom_amd import ops
+    inner, k = 1040, 264
+    x, w = randn(t, k, dtype=BF16), randn(2 * inner, k, dtype=BF16, scale=0.15)
+    gu = x.double() @ w.double().T
+    g, u = gu[:, :inner], gu[:, inner:]
+    assert torch.allclose(gelu_tanh(g), torch.nn.functional.gelu(g, approximate="tanh"), atol=1e-12)
+    want = {"silu": g / (1.0 + torch.exp(-g)) * u, "gelu_tanh": gelu_tanh(g) * u}
+    assert (want["silu"] - want["gelu_tanh"]).abs().max() > 0.05          # the two differ visibly
+    packed = ops.pack_weight(w.to(DEV), True)
+    for act in ("silu", "gelu_tanh"):
+        for which in ("stream", "skinny", "tiled"):
+            if (which == "stream" and t > 128) or (which == "skinny" and t > 64):
+                continue
+            with ops.gemm_few_rows_kernel(which):
+                got = ops.gemm_bf16(x.to(DEV), packed, None, None, F32, gated=act, packed_shape=(2 * inner, k))
+            close(got, want[act], atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"{act} through {which}, t={t}")
+        got = ops.gate_mul(gu.float().to(DEV), F32, act)
+        close(got, want[act], atol=1e-5, rtol=1e-5, what=f"{act}, elementwise")
+    with pytest.raises(ops.KernelLibraryError, match="unknown gate activation"):
+        ops.gate_mul(gu.float().to(DEV), F32, "relu")
+
+
 @pytest.mark.parametrize("shape", [0, 1, 2])
 @pytest.mark.parametrize("packed", [False, True])
 @pytest.mark.parametrize("t, n, k", [(65, 100, 96), (300, 224, 200), (520, 264, 128), (257, 1000, 448), (130, 72, 2368)])

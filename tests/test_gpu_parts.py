@@ -87,6 +87,30 @@ def test_feed_forward_alone(dtype):
         close(xd, want, dtype, f"ffn rows={rows}")
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_feed_forward_with_a_gelu_gate(dtype):
+    """The gate's activation is a constant of the part: the same feed-forward with the tanh form
+    of GELU, in 32-bit (product, then the activation kernel) and bfloat16 (fused epilogues)."""
+    from sonicboom_amd.parts import build_part
+    from sonicboom_amd.parts.ffn import gated_ffn_spec
+    spec = gated_ffn_spec("m.", 72, 200, activation="gelu_tanh")
+    dev, ref = tensors_for(spec, dtype)
+    ffn = build_part(spec, dev, runtime(dtype))
+    for rows in (3, 70):
+        h, x = rand(rows, 72).to(dtype), rand(rows, 72, seed=5)
+        xd = x.to(DEV)
+        ffn.forward(h.to(DEV), xd, None)
+        f = h.float().numpy()
+        g, u = P.linear(f, ref["m.gate_proj.weight"]), P.linear(f, ref["m.up_proj.weight"])
+        gelu = 0.5 * g * (1.0 + np.tanh(0.7978845608028654 * g * (1.0 + 0.044715 * g * g)))
+        want = P.linear((gelu * u).astype(np.float32), ref["m.down_proj.weight"]) + x.numpy()
+        close(xd, want, dtype, f"gelu ffn rows={rows}")
+        silu = P.swiglu(f, ref["m.gate_proj.weight"], ref["m.up_proj.weight"], ref["m.down_proj.weight"]) + x.numpy()
+        assert np.abs(silu - want).max() > 1e-3          # not the SiLU result
+    with pytest.raises(ValueError, match="unknown activation"):
+        build_part(gated_ffn_spec("m.", 72, 200, activation="relu"), dev, runtime(dtype))
+
+
 def run_mixer(mixer, rt, h_rows, cuts, width):
     """Feed rows of one sequence to a mixer in the given cuts; returns what it added to a zero stream."""
     from sonicboom_amd.cache import PagedCache, group_entries
