@@ -684,16 +684,220 @@ __device__ __forceinline__ void finish_decode_block(const WaveState<1> &st, floa
   }
 }
 
-template <bool BOTH>
+// ---- decode with the rotation and the store folded in ------------------------------------------
+// A decode step's queries come out of the qkv product as float32 rows [queries | keys | values]
+// (in K slices that are still to be added, plus a bias), have to be rotated and rounded, and the
+// row's key and value have to go into the cache before the row attends.  Done by a kernel of its
+// own that is a launch more per layer; folded in here, every block builds the queries of its heads
+// itself (sums, bias, rotation: the arithmetic and the order of sb_rope_kv_store, so the same
+// bits), and the block whose pages hold the row's own position also builds the new key and value,
+// stores them, and only then reads that page (a fence and a barrier within the block: the
+// stores and the loads come from the same CU).
+struct RopeArgs {
+  const float *qkv;            // [n_slices][n_seqs][row_stride]
+  int row_stride, n_slices;
+  size_t slice_stride;
+  const float *bias;           // [row] or NULL
+  const float *inv_freq;       // [rot_dims / 2] or NULL: no rotation
+  const float *freq_factors;   // [rot_dims / 2] or NULL
+  int rot_dims;                // a multiple of 16
+  int store;                   // keys and values go into the cache (0: a layer that reads another's)
+};
+
+// Eight consecutive elements e0 .. e0+7 of sequence seq's qkv row: slices in ascending order, then the bias.
+__device__ __forceinline__ void qkv8(float (&v)[8], const RopeArgs &ra, int seq, size_t e0) {
+  const float *r = ra.qkv + size_t(seq) * ra.row_stride + e0;
+  float4 a = *reinterpret_cast<const float4 *>(r), b = *reinterpret_cast<const float4 *>(r + 4);
+  for (int s = 1; s < ra.n_slices; ++s) {
+    const float4 c = *reinterpret_cast<const float4 *>(r + s * ra.slice_stride);
+    const float4 d = *reinterpret_cast<const float4 *>(r + s * ra.slice_stride + 4);
+    a.x += c.x; a.y += c.y; a.z += c.z; a.w += c.w;
+    b.x += d.x; b.y += d.y; b.z += d.z; b.w += d.w;
+  }
+  if (ra.bias) {       // 16-byte aligned like the row: e0 is a multiple of 8
+    const float4 c = *reinterpret_cast<const float4 *>(ra.bias + e0), d = *reinterpret_cast<const float4 *>(ra.bias + e0 + 4);
+    a.x += c.x; a.y += c.y; a.z += c.z; a.w += c.w;
+    b.x += d.x; b.y += d.y; b.z += d.z; b.w += d.w;
+  }
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
+// Eight floats rounded as sb_rope_kv_store rounds (to nearest even, a NaN stays one), packed.
+__device__ __forceinline__ uint4 pack8(const float (&y)[8]) {
+  return make_uint4(uint32_t(f32_to_bf16(y[0])) | uint32_t(f32_to_bf16(y[1])) << 16,
+                    uint32_t(f32_to_bf16(y[2])) | uint32_t(f32_to_bf16(y[3])) << 16,
+                    uint32_t(f32_to_bf16(y[4])) | uint32_t(f32_to_bf16(y[5])) << 16,
+                    uint32_t(f32_to_bf16(y[6])) | uint32_t(f32_to_bf16(y[7])) << 16);
+}
+
+constexpr int kQStride = HD / 8 + 1;     // 16-byte units of a staged query row: one of padding against bank conflicts
+constexpr int kPerHead = HD / 8;         // work items (of eight elements) per head
+
+// LDS of the folded form: the block's cosines and sines, and the rotated, rounded queries of its
+// (up to 16) heads, which the four waves then read as fragments.
+struct RopeShared {
+  float cs[HD / 2], sn[HD / 2];
+  uint4 q[16 * kQStride];
+  uint4 k[HD / 8];      // the row's own key, rotated and rounded
+  bf16_t v[HD];         // and its value
+};
+
+// Work item `it` of a block of the folded form: eight elements d0 .. d0+7 of one head of the qkv
+// row; items [0, group * HD/8) are the queries of the block's heads, the next HD/8 the key of its
+// kv head, the last HD/8 the value.  x: the elements, p: their partners in the rotation (d0 a
+// multiple of 8, half and rot_dims multiples of 8: the eight lie on one side of every border).
+struct RopeItem {
+  float x[8], p[8];
+};
+__device__ __forceinline__ size_t item_head(int it, int n_q, int kvh, int group, int heads_q, int heads_kv) {
+  if (it < n_q) return size_t(kvh * group + it / kPerHead) * HD;
+  return size_t((it < n_q + kPerHead ? heads_q : heads_q + heads_kv) + kvh) * HD;
+}
+__device__ __forceinline__ void fetch_item(RopeItem &v, const RopeArgs &ra, int seq, int it, int n_q, int kvh,
+                                           int group, int heads_q, int heads_kv, int half) {
+  const size_t hoff = item_head(it, n_q, kvh, group, heads_q, heads_kv);
+  const int d0 = (it < n_q ? it % kPerHead : (it - n_q) % kPerHead) * 8;
+  qkv8(v.x, ra, seq, hoff + d0);
+  if (it < n_q + kPerHead && d0 < 2 * half) qkv8(v.p, ra, seq, hoff + (d0 < half ? d0 + half : d0 - half));
+}
+// The item's eight results: rotated queries and keys, the value as it is.
+__device__ __forceinline__ void finish_item(float (&y)[8], const RopeItem &v, int it, int n_q, int half,
+                                            const float *cs, const float *sn) {
+  const int d0 = (it < n_q ? it % kPerHead : (it - n_q) % kPerHead) * 8;
+  if (it >= n_q + kPerHead || d0 >= 2 * half) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = v.x[i];
+    return;
+  }
+  const bool low = d0 < half;
+  const int i0 = low ? d0 : d0 - half;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float y0, y1;
+    if (low) rotate_pair(v.x[i], v.p[i], cs[i0 + i], sn[i0 + i], y0, y1);
+    else rotate_pair(v.p[i], v.x[i], cs[i0 + i], sn[i0 + i], y0, y1);
+    y[i] = low ? y0 : y1;
+  }
+}
+
+// The block's queries into LDS, and in the block whose pages hold the row's own position (`mine`)
+// the row's key and value into the cache and into LDS.  All threads of the block; `first` holds
+// the thread's first item and `freq` the frequency of the angle it works out, whose loads went
+// out at the kernel's start (they depend on the block's and the thread's number only).  Ends with
+// a barrier after which the queries, the key and the value can be read from LDS; with
+// `visible` the stored key and value are also visible to the block's own loads from the cache
+// (a wait for the stores: the kernels that can patch their fragments from LDS do without).
+__device__ __forceinline__ void rope_store(RopeShared &sh, const RopeItem &first, float freq, const RopeArgs &ra,
+                                           int seq, int pos, int kvh, int group, int heads_q, int heads_kv,
+                                           bool mine, bool visible, bf16_t *k_cache, bf16_t *v_cache,
+                                           const int32_t *page_table, int max_pages, int n_pages_total) {
+  const int half = ra.inv_freq ? ra.rot_dims / 2 : 0;
+  if (int(threadIdx.x) < 2 * half) {
+    const int j = threadIdx.x, i = j < half ? j : j - half;
+    float theta = float(pos) * freq;
+    if (ra.freq_factors) theta = theta / ra.freq_factors[i];       // as sb_rope_kv_store: the product first
+    if (j < half) sh.cs[i] = cosf(theta);
+    else sh.sn[i] = sinf(theta);
+  }
+  int page = -1;
+  if (ra.store && mine) {
+    const int lp = pos / SB_PAGE;
+    page = lp < max_pages ? page_table[size_t(seq) * max_pages + lp] : -1;
+    if (page >= n_pages_total) page = -1;
+  }
+  if (half > 0) __syncthreads();
+  const int n_q = group * kPerHead;
+  const int n_items = n_q + (page >= 0 ? 2 * kPerHead : 0);
+  for (int it = threadIdx.x; it < n_items; it += blockDim.x) {
+    RopeItem later;
+    if (it != int(threadIdx.x)) fetch_item(later, ra, seq, it, n_q, kvh, group, heads_q, heads_kv, half);
+    float y[8];
+    finish_item(y, it == int(threadIdx.x) ? first : later, it, n_q, half, sh.cs, sh.sn);
+    if (it < n_q) {
+      sh.q[(it / kPerHead) * kQStride + it % kPerHead] = pack8(y);
+      continue;
+    }
+    const size_t base = (size_t(page) * heads_kv + kvh) * SB_PAGE * HD;
+    const int d0 = ((it - n_q) % kPerHead) * 8;
+    if (it < n_q + kPerHead) {
+      const uint4 packed = pack8(y);
+      sh.k[d0 / 8] = packed;
+      *reinterpret_cast<uint4 *>(k_cache + base + size_t(pos % SB_PAGE) * HD + d0) = packed;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const bf16_t b = f32_to_bf16(y[i]);
+        sh.v[d0 + i] = b;
+        v_cache[base + size_t(d0 + i) * SB_PAGE + pos % SB_PAGE] = b;
+      }
+    }
+  }
+  if (visible) __threadfence_block();
+  __syncthreads();
+}
+
+// The frequency of the rotation that thread t of a block works out a cosine or sine for
+// (threads [0, half) the cosines, [half, 2 half) the sines).
+__device__ __forceinline__ float rope_freq(const RopeArgs &ra) {
+  const int half = ra.inv_freq ? ra.rot_dims / 2 : 0;
+  const int j = threadIdx.x;
+  if (j >= 2 * half) return 0.f;
+  const int i = j < half ? j : j - half;
+  return ra.inv_freq[i];
+}
+
+// Half `half` of the page that holds the row's own position, as loaded from the cache before the
+// row's key and value were stored: the fragments' elements of slot `slot` (the row's position in
+// the page) replaced by the key and value in LDS.  A lane's key fragments are eight d of one key
+// each, its value fragments eight consecutive keys of one d.
+__device__ __forceinline__ void patch_half(HalfPage &hp, const RopeShared &sh, int half, int slot, int lane) {
+  const int r = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    const int key = 32 * half + 8 * (r >> 2) + 4 * t + (r & 3);
+    if (key == slot) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int d = ks * 32 + g * 8;
+        if (d < HD) hp.k[t][ks] = sh.k[d / 8];
+      }
+    }
+  }
+  const int e = slot - (32 * half + 8 * g);
+  if (e >= 0 && e < 8) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      uint32_t w[4] = {hp.v[dt].x, hp.v[dt].y, hp.v[dt].z, hp.v[dt].w};
+      const uint32_t val = sh.v[dt * 16 + r];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (i == (e >> 1)) w[i] = (e & 1) ? ((w[i] & 0xffffu) | (val << 16)) : ((w[i] & 0xffff0000u) | val);
+      hp.v[dt] = make_uint4(w[0], w[1], w[2], w[3]);
+    }
+  }
+}
+
+// A wave's query fragments from the staged queries.
+__device__ __forceinline__ void staged_q(bf16x8_t (&qf)[KS], const RopeShared &sh, int hq, bool col_ok, int lane) {
+  const int g = lane >> 4;
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d = ks * 32 + g * 8;
+    qf[ks] = as_bf16x8((col_ok && d < HD) ? sh.q[hq * kQStride + d / 8] : make_uint4(0u, 0u, 0u, 0u));
+  }
+}
+
+template <bool BOTH, bool FUSED>
 __global__ void __launch_bounds__(256)
 attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
-                   const bf16_t *__restrict__ q,
-                   const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
+                   const bf16_t *__restrict__ q, const RopeArgs ra,
+                   const bf16_t *k_cache, const bf16_t *v_cache,
                    const int32_t *__restrict__ page_table, int max_pages, int n_pages_total,
                    const int32_t *__restrict__ row_pos, int heads_q, int heads_kv, int n_chunks,
                    float scale_log2, int window, int n_seqs) {
   __shared__ float lds_o[4][HD * 16];   // [wave][d][col]
   __shared__ float lds_m[4][16], lds_l[4][16];
+  __shared__ std::conditional_t<FUSED, RopeShared, int> rope_sh;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int group = heads_q / heads_kv;
   const int head_tiles = (group + 15) / 16;
@@ -701,6 +905,15 @@ attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *
   const DecodeBlock blk = decode_block(tiles, n_seqs);
   const int chunk = blk.chunk, seq = blk.seq;
   const int kvh = blk.tile / head_tiles, ht = blk.tile - kvh * head_tiles;
+  // the folded form: this thread's share of the qkv row depends on the block's number only, so
+  // its loads go out before anything else
+  RopeItem first;
+  if constexpr (FUSED) {
+    const int n_q = group * kPerHead, n_all = n_q + (ra.store ? 2 * kPerHead : 0);
+    if (int(threadIdx.x) < n_all)
+      fetch_item(first, ra, seq, threadIdx.x, n_q, kvh, group, heads_q, heads_kv, ra.inv_freq ? ra.rot_dims / 2 : 0);
+  }
+  const float freq = FUSED ? rope_freq(ra) : 0.f;
   // the wave's page number does not depend on the position: both look-ups go out together
   const int pg = chunk * kPagesPerChunk + wave;
   const int page_looked_up = page_table[size_t(seq) * max_pages + min(pg, max_pages - 1)];
@@ -714,16 +927,45 @@ attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *
   const int hq = ht * 16 + r;                 // query head within the group
   const bool col_ok = hq < group;
   const int head = kvh * group + (col_ok ? hq : 0);
+  const bool have_page = pg >= key_lo / SB_PAGE && pg <= pos / SB_PAGE && pg < max_pages && page_looked_up >= 0 &&
+                         page_looked_up < n_pages_total;
+  const size_t off = (size_t(have_page ? page_looked_up : 0) * heads_kv + kvh) * SB_PAGE * HD;
+  const int col_pos = col_ok ? pos : -1;
   bf16x8_t qf[1][KS];
-  load_q(qf[0], q + (size_t(seq) * heads_q + head) * HD, col_ok, lane);
   WaveState<1> st;
   init_state<1>(st);
-  if (pg >= key_lo / SB_PAGE && pg <= pos / SB_PAGE && pg < max_pages) {
-    const int page = page_looked_up;
-    if (page >= 0 && page < n_pages_total) {
-      const size_t off = (size_t(page) * heads_kv + kvh) * SB_PAGE * HD;
-      attend_page<1, BOTH>(st, qf, k_cache + off, v_cache + off, pg * SB_PAGE, col_ok ? pos : -1, key_lo, key_lo,
-                           pos, scale_log2, lane);
+  if constexpr (!FUSED) {
+    load_q(qf[0], q + (size_t(seq) * heads_q + head) * HD, col_ok, lane);
+    if (have_page)
+      attend_page<1, BOTH>(st, qf, k_cache + off, v_cache + off, pg * SB_PAGE, col_pos, key_lo, key_lo, pos, scale_log2,
+                           lane);
+  } else {
+    // The page's keys and values do not depend on the queries: their loads go out first and are
+    // in flight while the block builds its queries.  The page that receives the row's own key
+    // and value is read like the others, before they are stored, and its fragments are patched
+    // from LDS afterwards.
+    const int page_pos = pg * SB_PAGE;
+    const bool use0 = have_page && !(page_pos > pos || page_pos + 31 < key_lo);
+    const bool use1 = have_page && !(page_pos + 32 > pos || page_pos + 63 < key_lo);
+    const bool own_page = ra.store && have_page && pg == pos / SB_PAGE;
+    constexpr bool kEarly = BOTH && HD <= 128;
+    HalfPage h0, h1;
+    if (kEarly) {
+      if (use0) load_half(h0, k_cache + off, v_cache + off, 0, lane);
+      if (use1) load_half(h1, k_cache + off, v_cache + off, 1, lane);
+    }
+    rope_store(rope_sh, first, freq, ra, seq, pos, kvh, group, heads_q, heads_kv, chunk == last_chunk, !kEarly,
+               const_cast<bf16_t *>(k_cache), const_cast<bf16_t *>(v_cache), page_table, max_pages, n_pages_total);
+    staged_q(qf[0], rope_sh, hq, col_ok, lane);
+    if (kEarly) {
+      const int slot = pos % SB_PAGE;
+      if (own_page && slot < 32 && use0) patch_half(h0, rope_sh, 0, slot, lane);
+      if (own_page && slot >= 32 && use1) patch_half(h1, rope_sh, 1, slot, lane);
+      if (use0) attend_half<1>(st, qf, h0, page_pos, col_pos, key_lo, key_lo, pos, scale_log2, lane);
+      if (use1) attend_half<1>(st, qf, h1, page_pos + 32, col_pos, key_lo, key_lo, pos, scale_log2, lane);
+    } else if (have_page) {
+      attend_page<1, BOTH>(st, qf, k_cache + off, v_cache + off, page_pos, col_pos, key_lo, key_lo, pos, scale_log2,
+                           lane);
     }
   }
   finish_decode_block(st, lds_o, lds_m, lds_l, out, part_o, part_ml, wave, lane, chunk, first_chunk == last_chunk,
@@ -736,15 +978,17 @@ attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *
 // fixed costs of a block (look-ups, queries, the merge through LDS, the partial results) are paid
 // once per 4 * ppw pages.  Block (chunk of 4 * ppw pages, kv head x head tile, sequence); wave w
 // takes pages chunk * 4 * ppw + w * ppw + 0 .. ppw-1.  Head sizes up to 128.
+template <bool FUSED>
 __global__ void __launch_bounds__(256, 2)
 attn_decode_long_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *__restrict__ part_ml,
-                        const bf16_t *__restrict__ q,
-                        const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
+                        const bf16_t *__restrict__ q, const RopeArgs ra,
+                        const bf16_t *k_cache, const bf16_t *v_cache,
                         const int32_t *__restrict__ page_table, int max_pages, int n_pages_total,
                         const int32_t *__restrict__ row_pos, int heads_q, int heads_kv, int n_chunks,
                         float scale_log2, int window, int ppw, int n_seqs) {
   __shared__ float lds_o[4][HD * 16];   // [wave][d][col]
   __shared__ float lds_m[4][16], lds_l[4][16];
+  __shared__ std::conditional_t<FUSED, RopeShared, int> rope_sh;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int group = heads_q / heads_kv;
@@ -753,6 +997,13 @@ attn_decode_long_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, fl
   const DecodeBlock blk = decode_block(tiles, n_seqs);
   const int chunk = blk.chunk, seq = blk.seq;
   const int kvh = blk.tile / head_tiles, ht = blk.tile - kvh * head_tiles;
+  RopeItem first;       // the folded form: see attn_decode_kernel
+  if constexpr (FUSED) {
+    const int n_q = group * kPerHead, n_all = n_q + (ra.store ? 2 * kPerHead : 0);
+    if (int(threadIdx.x) < n_all)
+      fetch_item(first, ra, seq, threadIdx.x, n_q, kvh, group, heads_q, heads_kv, ra.inv_freq ? ra.rot_dims / 2 : 0);
+  }
+  const float freq = FUSED ? rope_freq(ra) : 0.f;
   const int pages_per_chunk = kPagesPerChunk * ppw;
   const int pos = row_pos[seq];
   const int key_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
@@ -765,7 +1016,6 @@ attn_decode_long_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, fl
   const bool col_ok = hq < group;
   const int head = kvh * group + (col_ok ? hq : 0);
   bf16x8_t qf[1][KS];
-  load_q(qf[0], q + (size_t(seq) * heads_q + head) * HD, col_ok, lane);
   WaveState<1> st;
   init_state<1>(st);
 
@@ -780,10 +1030,30 @@ attn_decode_long_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, fl
     ok = page >= 0 && page < n_pages_total;
     return size_t(ok ? page : 0) * page_elems + head_off;
   };
+  HalfPage h0, h1;
+  bool ok = false;
+  size_t off = 0;
+  // The folded form: the first half page's loads go out before the block builds its queries.  The
+  // page that receives the row's own key and value is read like the others (before or after they
+  // are stored: the stores are not waited for) and its fragments are patched from LDS.
   if (pg_begin < pg_end) {
-    HalfPage h0, h1;
+    off = page_of(pg_begin, ok);
+    load_half_straight(h0, k_cache + off, v_cache + off, 0, lane);
+  }
+  if constexpr (FUSED) {
+    rope_store(rope_sh, first, freq, ra, seq, pos, kvh, group, heads_q, heads_kv, chunk == last_chunk, false,
+               const_cast<bf16_t *>(k_cache), const_cast<bf16_t *>(v_cache), page_table, max_pages, n_pages_total);
+    staged_q(qf[0], rope_sh, hq, col_ok, lane);
+  } else {
+    load_q(qf[0], q + (size_t(seq) * heads_q + head) * HD, col_ok, lane);
+  }
+  if (pg_begin < pg_end) {
     // 32 keys from `base` on: all visible and written (the common case), or tested one by one
-    auto attend = [&](const HalfPage &h, int base, bool ok) {
+    const int own_base = (FUSED && ra.store) ? (pos / 32) * 32 : -1;     // the half page of the row's own slot
+    auto attend = [&](HalfPage &h, int base, bool ok) {
+      if constexpr (FUSED) {
+        if (ok && base == own_base) patch_half(h, rope_sh, (base >> 5) & 1, pos % SB_PAGE, lane);
+      }
       if (ok && base >= key_lo && base + 31 <= pos) {
         attend_half<1, false>(st, qf, h, base, pos, key_lo, key_lo, pos, scale_log2, lane);
       } else {
@@ -792,9 +1062,6 @@ attn_decode_long_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, fl
                              lane);
       }
     };
-    bool ok;
-    size_t off = page_of(pg_begin, ok);
-    load_half_straight(h0, k_cache + off, v_cache + off, 0, lane);
     int pg = pg_begin;
     // every page but the last: the loads of the next half page go out before this half's
     // products, with no branch between a load and its use
@@ -868,26 +1135,20 @@ extern "C" size_t sb_attn_decode_part_ml(int n_seqs, int heads_q, int heads_kv, 
   return size_t(n_seqs) * tiles * sb_attn_decode_chunks(max_pages) * 32;
 }
 
-// q, out: bf16 [n_seqs, heads_q * HD], one row per sequence; k_cache bf16 [pages][heads_kv][64][HD],
-// v_cache bf16 [pages][heads_kv][HD][64].  part_o / part_ml: float buffers of the sizes the two
-// functions above give (may be NULL when max_pages fits one chunk).
-extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
-                                   const int32_t *page_table, int max_pages, int n_pages_total,
-                                   const int32_t *row_pos, float *part_o, float *part_ml, int n_seqs,
-                                   int heads_q, int heads_kv, float scale, int window, int pages_per_wave,
-                                   void *stream) {
-  int rc = check_common(out, q, k_cache, v_cache, page_table, row_pos, max_pages, n_pages_total, heads_q,
-                        heads_kv, window, "sb_attn_decode_bf16");
-  if (rc != SB_OK) return rc;
-  SB_REQUIRE(n_seqs >= 0, "sb_attn_decode_bf16: bad batch");
-  SB_SUPPORT(n_seqs <= 65535, "sb_attn_decode_bf16: more than 65535 sequences in a step");
-  if (n_seqs == 0) return SB_OK;
+namespace {
+
+// The decode launch, for queries that are given (q) or still to be built (ra.qkv).
+int decode_launch(const char *who, void *out, const void *q, const RopeArgs &ra, const void *k_cache,
+                  const void *v_cache, const int32_t *page_table, int max_pages, int n_pages_total,
+                  const int32_t *row_pos, float *part_o, float *part_ml, int n_seqs, int heads_q, int heads_kv,
+                  float scale, int window, int pages_per_wave, void *stream) {
+  const bool fused = ra.qkv != nullptr;
   const int chunks_1 = sb_attn_decode_chunks(max_pages);      // what the partial buffers are sized for
-  SB_REQUIRE(chunks_1 == 1 || (part_o && part_ml), "sb_attn_decode_bf16: no buffers for the partial results");
+  SB_REQUIRE(chunks_1 == 1 || (part_o && part_ml), "%s: no buffers for the partial results", who);
   const int group = heads_q / heads_kv;
   const int head_tiles = (group + 15) / 16;
   hipStream_t s = (hipStream_t)stream;
-  SB_SUPPORT(heads_kv * head_tiles <= 65535, "sb_attn_decode_bf16: too many heads");
+  SB_SUPPORT(heads_kv * head_tiles <= 65535, "%s: too many heads", who);
   // A wave takes one page and asks for all of it at once (one round trip to memory), or, when
   // two pages per wave still leave a block for every CU, several pages in a row with half a page
   // in flight while the half before it is multiplied.
@@ -913,9 +1174,9 @@ extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache
       const double rate = busy * 27e3 < 5.3e6 ? busy * 27e3 : 5.3e6;            // bytes per us
       const int run = c < pages ? c : pages;
       // a block spends about 4 us on what is not streaming (look-ups, queries, the merge)
-      const double stream = double(per_chunk) * pages * page_bytes / rate * (1.0 + 4.0 / (run * 3.3));
+      const double stream_us = double(per_chunk) * pages * page_bytes / rate * (1.0 + 4.0 / (run * 3.3));
       const double in_a_row = run * 3.3 + 4.0;
-      const double t = (stream > in_a_row ? stream : in_a_row) + (chunks > 1 ? 8.0 : 0.0);
+      const double t = (stream_us > in_a_row ? stream_us : in_a_row) + (chunks > 1 ? 8.0 : 0.0);
       if (best < 0.0 || t < best) best = t, ppw = c;
     }
   }
@@ -923,28 +1184,91 @@ extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache
   if (pages_per_wave > 0 && (pages_per_wave == 1 || HD <= 128)) ppw = pages_per_wave;
   const int pages_per_chunk = kPagesPerChunk * ppw;
   const int n_chunks = (max_pages + pages_per_chunk - 1) / pages_per_chunk;
-  SB_SUPPORT((long long)n_chunks * per_chunk <= 0x7fffffffLL, "sb_attn_decode_bf16: too many blocks");
+  SB_SUPPORT((long long)n_chunks * per_chunk <= 0x7fffffffLL, "%s: too many blocks", who);
   const unsigned grid = unsigned((long long)n_chunks * per_chunk);
-  if (ppw > 1)
-    attn_decode_long_kernel<<<grid, 256, 0, s>>>((bf16_t *)out, part_o, part_ml, (const bf16_t *)q,
-                                                 (const bf16_t *)k_cache, (const bf16_t *)v_cache, page_table,
-                                                 max_pages, n_pages_total, row_pos, heads_q, heads_kv, n_chunks,
-                                                 scale * kLog2e, window, ppw, n_seqs);
-  else if ((long long)n_chunks * per_chunk <= 1536)
-    attn_decode_kernel<true><<<grid, 256, 0, s>>>((bf16_t *)out, part_o, part_ml, (const bf16_t *)q,
-                                                  (const bf16_t *)k_cache, (const bf16_t *)v_cache, page_table,
-                                                  max_pages, n_pages_total, row_pos, heads_q, heads_kv,
-                                                  n_chunks, scale * kLog2e, window, n_seqs);
-  else
-    attn_decode_kernel<false><<<grid, 256, 0, s>>>((bf16_t *)out, part_o, part_ml, (const bf16_t *)q,
-                                                   (const bf16_t *)k_cache, (const bf16_t *)v_cache, page_table,
-                                                   max_pages, n_pages_total, row_pos, heads_q, heads_kv,
-                                                   n_chunks, scale * kLog2e, window, n_seqs);
-  rc = sb::check_launch("sb_attn_decode_bf16");
+#define SB_ARGS                                                                                           \
+  (bf16_t *)out, part_o, part_ml, (const bf16_t *)q, ra, (const bf16_t *)k_cache, (const bf16_t *)v_cache, \
+      page_table, max_pages, n_pages_total, row_pos, heads_q, heads_kv, n_chunks, scale *kLog2e, window
+  if (ppw > 1) {
+    if (fused) attn_decode_long_kernel<true><<<grid, 256, 0, s>>>(SB_ARGS, ppw, n_seqs);
+    else attn_decode_long_kernel<false><<<grid, 256, 0, s>>>(SB_ARGS, ppw, n_seqs);
+  } else if ((long long)n_chunks * per_chunk <= 1536) {
+    if (fused) attn_decode_kernel<true, true><<<grid, 256, 0, s>>>(SB_ARGS, n_seqs);
+    else attn_decode_kernel<true, false><<<grid, 256, 0, s>>>(SB_ARGS, n_seqs);
+  } else {
+    if (fused) attn_decode_kernel<false, true><<<grid, 256, 0, s>>>(SB_ARGS, n_seqs);
+    else attn_decode_kernel<false, false><<<grid, 256, 0, s>>>(SB_ARGS, n_seqs);
+  }
+#undef SB_ARGS
+  int rc = sb::check_launch(who);
   if (rc != SB_OK || n_chunks == 1) return rc;
   attn_decode_merge_kernel<<<dim3((HD * 16 + 255) / 256, heads_kv * head_tiles, n_seqs), 256, 0, s>>>(
       (bf16_t *)out, part_o, part_ml, row_pos, heads_q, heads_kv, n_chunks, window, pages_per_chunk);
-  return sb::check_launch("sb_attn_decode_bf16 (merge)");
+  return sb::check_launch(who);
+}
+
+}  // namespace
+
+// q, out: bf16 [n_seqs, heads_q * HD], one row per sequence; k_cache bf16 [pages][heads_kv][64][HD],
+// v_cache bf16 [pages][heads_kv][HD][64].  part_o / part_ml: float buffers of the sizes the two
+// functions above give (may be NULL when max_pages fits one chunk).  pages_per_wave: 0, or a
+// test's or a measurement's choice of how many pages in a row a wave takes.
+extern "C" int sb_attn_decode_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
+                                   const int32_t *page_table, int max_pages, int n_pages_total,
+                                   const int32_t *row_pos, float *part_o, float *part_ml, int n_seqs,
+                                   int heads_q, int heads_kv, float scale, int window, int pages_per_wave,
+                                   void *stream) {
+  int rc = check_common(out, q, k_cache, v_cache, page_table, row_pos, max_pages, n_pages_total, heads_q,
+                        heads_kv, window, "sb_attn_decode_bf16");
+  if (rc != SB_OK) return rc;
+  SB_REQUIRE(n_seqs >= 0, "sb_attn_decode_bf16: bad batch");
+  SB_SUPPORT(n_seqs <= 65535, "sb_attn_decode_bf16: more than 65535 sequences in a step");
+  if (n_seqs == 0) return SB_OK;
+  const RopeArgs none{nullptr, 0, 0, 0, nullptr, nullptr, nullptr, 0, 0};
+  return decode_launch("sb_attn_decode_bf16", out, q, none, k_cache, v_cache, page_table, max_pages, n_pages_total,
+                       row_pos, part_o, part_ml, n_seqs, heads_q, heads_kv, scale, window, pages_per_wave, stream);
+}
+
+// 1 when sb_attn_decode_rope_bf16 takes these sizes (else: sb_rope_kv_store, then sb_attn_decode_bf16).
+extern "C" int sb_attn_decode_rope_ok(int heads_q, int heads_kv, int rot_dims, int row_stride) {
+  return heads_kv > 0 && heads_q % heads_kv == 0 && heads_q / heads_kv <= 16 && rot_dims >= 0 && rot_dims % 16 == 0 &&
+         rot_dims <= HD && row_stride % 4 == 0;
+}
+
+// The same attention for a step whose queries, keys and values are still the float32 rows of the
+// qkv product: qkv [n_slices][n_seqs][row_stride], a row [heads_q*HD queries | heads_kv*HD keys |
+// heads_kv*HD values], the slices added in ascending order, then `bias` (float [row] or NULL).
+// Queries and keys are rotated as sb_rope_kv_store rotates them (inv_freq NULL: not at all), the
+// row's key and value are stored at its position (store_kv = 0: nothing is stored, for a layer
+// that reads another layer's cache), and the row attends over the cache including itself: the
+// results and the cache contents are those of sb_rope_kv_store followed by sb_attn_decode_bf16,
+// bit for bit, in one launch less.  Sizes: sb_attn_decode_rope_ok.
+extern "C" int sb_attn_decode_rope_bf16(void *out, const float *qkv, int row_stride, int n_slices, const float *bias,
+                                        const float *inv_freq, const float *freq_factors, int rot_dims,
+                                        int store_kv, void *k_cache, void *v_cache, const int32_t *page_table,
+                                        int max_pages, int n_pages_total, const int32_t *row_pos, float *part_o,
+                                        float *part_ml, int n_seqs, int heads_q, int heads_kv, float scale,
+                                        int window, int pages_per_wave, void *stream) {
+  int rc = check_common(out, qkv, k_cache, v_cache, page_table, row_pos, max_pages, n_pages_total, heads_q,
+                        heads_kv, window, "sb_attn_decode_rope_bf16");
+  if (rc != SB_OK) return rc;
+  SB_REQUIRE(n_seqs >= 0 && n_slices >= 1 && n_slices <= 8, "sb_attn_decode_rope_bf16: bad batch or slice count");
+  SB_SUPPORT(n_seqs <= 65535, "sb_attn_decode_rope_bf16: more than 65535 sequences in a step");
+  SB_REQUIRE(row_stride >= (heads_q + (store_kv ? 2 * heads_kv : 0)) * HD,
+             "sb_attn_decode_rope_bf16: row stride %d is shorter than a row of queries%s", row_stride,
+             store_kv ? ", keys and values" : "");
+  if (!inv_freq) rot_dims = 0;
+  SB_SUPPORT(sb_attn_decode_rope_ok(heads_q, heads_kv, rot_dims, row_stride),
+             "sb_attn_decode_rope_bf16: takes up to 16 query heads per kv head, a rotary width in steps of 16 and a "
+             "row stride in steps of 4 (heads %d / %d, rotary width %d, stride %d)", heads_q, heads_kv, rot_dims,
+             row_stride);
+  SB_SUPPORT(!bias || reinterpret_cast<uintptr_t>(bias) % 4 == 0, "sb_attn_decode_rope_bf16: unaligned bias");
+  if (n_seqs == 0) return SB_OK;
+  const RopeArgs ra{qkv, row_stride, n_slices, size_t(n_seqs) * row_stride, bias, inv_freq, freq_factors, rot_dims,
+                    store_kv ? 1 : 0};
+  return decode_launch("sb_attn_decode_rope_bf16", out, nullptr, ra, k_cache, v_cache, page_table, max_pages,
+                       n_pages_total, row_pos, part_o, part_ml, n_seqs, heads_q, heads_kv, scale, window,
+                       pages_per_wave, stream);
 }
 
 // q, out: bf16 [n_rows, heads_q * HD]; tiles int32 [n_tiles][4] = (first row, rows <= 16, sequence, 0),

@@ -37,6 +37,15 @@ __device__ __forceinline__ float gate_act(float g, int kind) {
   return g / (1.0f + expf(-g));
 }
 
+// The rotation of one pair (x0, x1) by the angle whose cosine and sine are c and s: every product
+// and sum rounded on its own (no fused multiply-add), so that every kernel that rotates a pair
+// gives the same bits (/root/reference/core/src/nn/rope.cpp:46-55).
+__device__ __forceinline__ void rotate_pair(float x0, float x1, float c, float s, float &y0, float &y1) {
+#pragma clang fp contract(off)
+  y0 = x0 * c - x1 * s;
+  y1 = x0 * s + x1 * c;
+}
+
 // Value of element i of a buffer whose type is only known at run time.
 __device__ __forceinline__ float ld_dyn(const void *p, int dtype, size_t i) {
   return dtype == SB_F32 ? ((const float *)p)[i] : bf16_to_f32(((const bf16_t *)p)[i]);

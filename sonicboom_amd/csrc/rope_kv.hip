@@ -126,8 +126,8 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
       const bool have = preloaded && it == int(threadIdx.x);
       const float x0 = have ? pre0 : qkv_at<SLICES>(r, hoff + i, n_slices, slice_stride, bias);
       const float x1 = have ? pre1 : qkv_at<SLICES>(r, hoff + i + half, n_slices, slice_stride, bias);
-      const float y0 = x0 * c - x1 * sv;
-      const float y1 = x0 * sv + x1 * c;
+      float y0, y1;
+      rotate_pair(x0, x1, c, sv, y0, y1);
       if (is_q) {
         st_f(qo, hoff + i, y0);
         st_f(qo, hoff + i + half, y1);

@@ -547,6 +547,67 @@ def attention_decode_mfma(q, k_cache, v_cache, page_table, seq_pos, heads_q, hea
     return out
 
 
+def attention_decode_rope_ok(qkv: torch.Tensor, q_dtype, cache_dtype, heads_q: int, heads_kv: int, head_dim: int,
+                             rot_dims: int) -> bool:
+    """Whether :func:`attention_decode_rope` takes these operands (else: :func:`rope_kv_store`, then
+    :func:`attention`)."""
+    if not attention_mfma_ok(q_dtype, cache_dtype, head_dim) or qkv.dtype != torch.float32:
+        return False
+    lib = library.attention_library(head_dim)
+    return bool(lib.sb_attn_decode_rope_ok(heads_q, heads_kv, int(rot_dims), qkv.shape[-1]))
+
+
+def attention_decode_rope(qkv: torch.Tensor, inv_freq: Optional[torch.Tensor], freq_factors: Optional[torch.Tensor],
+                          rot_dims: int, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor,
+                          seq_pos: torch.Tensor, heads_q: int, heads_kv: int, head_dim: int, scale: float, window: int,
+                          bias: Optional[torch.Tensor] = None, store: bool = True) -> torch.Tensor:
+    """A decode step's rotation, store and attention in one kernel: ``qkv`` float32 [n, width] or
+    [slices, n, width] (partial sums of the projection, added in ascending order, then ``bias``),
+    one row per sequence at position ``seq_pos[i]``.  Queries and keys are rotated as
+    :func:`rope_kv_store` rotates them, the row's key and value go into the cache (``store``), and the
+    row attends over its sequence's keys, its own among them.  Returns the attention output in
+    bfloat16 [n, heads_q * head_dim]: the bits of the two kernels one after the other."""
+    _dev(qkv, inv_freq, freq_factors, k_cache, v_cache, page_table, seq_pos, bias)
+    n_slices = 1
+    if qkv.dim() == 3:
+        n_slices = qkv.shape[0]
+        qkv = qkv.view(-1, qkv.shape[2])
+    n = qkv.shape[0] // n_slices
+    need = (heads_q + (2 * heads_kv if store else 0)) * head_dim
+    if qkv.dtype != torch.float32 or qkv.shape[1] < need:
+        raise KernelLibraryError(f"qkv rows must be float32 with at least {need} elements")
+    if bias is not None and (bias.dtype != torch.float32 or bias.numel() < need):
+        raise KernelLibraryError("the qkv bias must be float32 and cover a whole row")
+    if inv_freq is not None:
+        if inv_freq.dtype != torch.float32 or inv_freq.numel() != rot_dims // 2:
+            raise KernelLibraryError("inv_freq must be float32 [rot_dims/2]")
+        if freq_factors is not None and (freq_factors.dtype != torch.float32 or freq_factors.numel() < rot_dims // 2):
+            raise KernelLibraryError("freq_factors must be float32 [rot_dims/2]")
+    _check_cache(k_cache, v_cache, heads_kv, head_dim)
+    if k_cache.dtype != torch.bfloat16:
+        raise KernelLibraryError("the fused decode kernel takes a bfloat16 cache")
+    _i32(seq_pos, n, "sequence positions")
+    if page_table.dtype != torch.int32 or page_table.dim() != 2 or page_table.shape[0] < n:
+        raise KernelLibraryError("page table must be int32 [sequences, pages]")
+    lib = library.attention_library(head_dim)
+    max_pages = page_table.shape[1]
+    chunks = lib.sb_attn_decode_chunks(max_pages)
+    out = torch.empty((n, heads_q * head_dim), dtype=torch.bfloat16, device=qkv.device)
+    part_o = part_ml = None
+    if chunks > 1:
+        part_o = torch.empty((lib.sb_attn_decode_part_o(n, heads_q, heads_kv, max_pages),), dtype=torch.float32,
+                             device=qkv.device)
+        part_ml = torch.empty((lib.sb_attn_decode_part_ml(n, heads_q, heads_kv, max_pages),), dtype=torch.float32,
+                              device=qkv.device)
+    check(lib.sb_attn_decode_rope_bf16(_p(out), _p(qkv), qkv.shape[1], n_slices, _p(bias), _p(inv_freq),
+                                       _p(freq_factors), int(rot_dims) if inv_freq is not None else 0,
+                                       1 if store else 0, _p(k_cache), _p(v_cache), _p(page_table), max_pages,
+                                       k_cache.shape[0], _p(seq_pos), _p(part_o), _p(part_ml), n, heads_q, heads_kv,
+                                       float(scale), int(window), _hints.decode_pages, _stream()),
+          lib, "sb_attn_last_error")
+    return out
+
+
 @contextlib.contextmanager
 def attention_decode_pages_per_wave(head_dim: int, pages: int):
     """For tests and measurements: inside the block this thread's decode attention gives every

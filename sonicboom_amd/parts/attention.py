@@ -97,6 +97,7 @@ class Attention(Mixer):
 
     fuses_norm = True
     graph_safe = True     # its launches depend on device buffers only
+    fold_rotation = True  # decode steps: rotate and store inside the attention kernel where it takes the sizes
 
     def forward(self, h, x, ctx, binding, then_norm=None):
         """x += attention(h).  Returns then_norm(x) when the output projection could apply the
@@ -119,6 +120,14 @@ class Attention(Mixer):
             tables = (None, None, 0)
         inv_freq, freq_factors, rot_dims = tables
         page_table = ctx.page_table(binding.group)
+        if ctx.is_decode and rt.fast_kernels and self.fold_rotation and ops.attention_decode_rope_ok(
+                qkv, rt.act_dtype, binding.k_cache.dtype, self.heads_q, self.heads_kv, self.head_dim,
+                rot_dims if inv_freq is not None else 0):
+            # one token per sequence: rotation, store and attention in one kernel
+            a = ops.attention_decode_rope(qkv, inv_freq, freq_factors, rot_dims, binding.k_cache, binding.v_cache,
+                                          page_table, ctx.row_pos, self.heads_q, self.heads_kv, self.head_dim,
+                                          self.scale, self.window, bias=bias, store=writes)
+            return self.out.add_into(a, x, then_norm, rt.act_dtype)
         q = ops.rope_kv_store(
             qkv, rt.act_dtype, inv_freq, freq_factors, rot_dims, ctx.row_pos, ctx.row_seq,
             binding.k_cache if writes else None, binding.v_cache if writes else None,

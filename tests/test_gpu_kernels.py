@@ -797,6 +797,70 @@ def test_attention_prefill_window_edge(hq, hkv, hd, window):
         close(got, want, atol=2e-2, rtol=1e-2, what=f"window {window}, dominant key {d}")
 
 
+FOLDED_SHAPES = [(4, 2, 16, 16), (3, 1, 32, 32), (5, 5, 48, 16), (6, 2, 80, 64), (28, 4, 128, 128), (16, 1, 64, 0),
+                 (2, 1, 256, 256)]
+
+
+@pytest.mark.parametrize("hq, hkv, hd, rot, pages", [(*sh, p) for sh in FOLDED_SHAPES for p in (0, 1, 2, 8)
+                                                     if p <= 1 or sh[2] <= 128])     # several pages per wave: up to head size 128
+@pytest.mark.parametrize("window", [0, 70])
+def test_attention_decode_with_rotation_and_store_folded_in(hq, hkv, hd, rot, window, pages):
+    """A decode step's rotation, store and attention in one kernel against the two kernels one
+    after the other: the same output and the same cache, bit for bit.  The qkv rows come as one
+    array and as three K slices with a bias; rows stand at a page's first and last slot, on the
+    first token of a sequence, and behind a window; one row has no page at all (a row added to
+    fill a batch: nothing is stored, nothing seen)."""
+    from sonicboom_amd import ops
+    lens = [1, 64, 65, 128, 300, 700, 1]          # the row is the sequence's last token
+    n_seq = len(lens)
+    width_pages = max((n + 63) // 64 for n in lens)
+    perm = torch.randperm(n_seq * width_pages + 3, generator=torch.Generator().manual_seed(5))
+    table = torch.full((n_seq, width_pages), -1, dtype=torch.int32)
+    it = iter(perm.tolist())
+    for s_, n in enumerate(lens[:-1]):            # the last sequence keeps a table of -1
+        for pg in range((n + 63) // 64):
+            table[s_, pg] = next(it)
+    n_pages = n_seq * width_pages + 3
+    kc0 = randn(n_pages, hkv, 64, hd, seed=1).to(BF16)
+    vc0 = randn(n_pages, hkv, hd, 64, seed=2).to(BF16)
+    pos = torch.tensor([n - 1 for n in lens], dtype=torch.int32)
+    pos[-1] = 0
+    seq = torch.arange(n_seq, dtype=torch.int32)
+    width = (hq + 2 * hkv) * hd
+    inv = ff = None
+    if rot:
+        inv = torch.exp(-2.0 * torch.arange(rot // 2, dtype=F32) / rot * math.log(1e4)).to(DEV)
+        ff = (1.0 + torch.arange(rot // 2, dtype=F32) / rot).to(DEV)
+    scale = 1.0 / math.sqrt(hd)
+    for n_slices in (1, 3):
+        qkv = randn(n_slices, n_seq, width, seed=3 + n_slices).to(DEV)
+        bias = randn(width, seed=9, scale=0.3).to(DEV) if n_slices > 1 else None
+        arg = qkv if n_slices > 1 else qkv[0].contiguous()
+        # two kernels
+        kc1, vc1 = kc0.clone().to(DEV), vc0.clone().to(DEV)
+        q = ops.rope_kv_store(arg, BF16, inv, ff, rot, pos.to(DEV), seq.to(DEV), kc1, vc1, table.to(DEV), hq, hkv, hd,
+                              bias=bias)
+        with ops.attention_decode_pages_per_wave(hd, pages):
+            want = ops.attention_decode_mfma(q, kc1, vc1, table.to(DEV), pos.to(DEV), hq, hkv, hd, scale, window)
+            # one kernel
+            kc2, vc2 = kc0.clone().to(DEV), vc0.clone().to(DEV)
+            assert ops.attention_decode_rope_ok(arg, BF16, BF16, hq, hkv, hd, rot)
+            got = ops.attention_decode_rope(arg, inv, ff, rot, kc2, vc2, table.to(DEV), pos.to(DEV), hq, hkv, hd, scale,
+                                            window, bias=bias)
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16)), f"slices {n_slices}"
+            assert torch.equal(kc2.view(torch.int16), kc1.view(torch.int16))
+            assert torch.equal(vc2.view(torch.int16), vc1.view(torch.int16))
+            assert not torch.equal(kc2.view(torch.int16), kc0.to(DEV).view(torch.int16))     # something was stored
+            # queries only (a layer that reads another layer's cache): nothing is stored
+            kc3, vc3 = kc1.clone(), vc1.clone()
+            only_q = arg[..., : hq * hd].contiguous()
+            got = ops.attention_decode_rope(only_q, inv, ff, rot, kc3, vc3, table.to(DEV), pos.to(DEV), hq, hkv, hd,
+                                            scale, window, bias=bias, store=False)
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+            assert torch.equal(kc3.view(torch.int16), kc1.view(torch.int16))
+    assert not ops.attention_decode_rope_ok(arg, BF16, BF16, 34, 2, hd, rot)          # 17 heads per kv head
+
+
 @pytest.mark.parametrize("vocab", [5, 256, 1000, 152064])
 def test_argmax_first_maximum(vocab):
     from sonicboom_amd import ops
