@@ -73,6 +73,48 @@ def decode_bytes(m, batch, lengths):
     return weights + kv
 
 
+class ClockSampler:
+    """Samples the GPU's engine clock with ``rocm-smi --showclocks`` in a thread while work runs
+    (``--clocks``): what the matrix pipes' peak has to be scaled by under load."""
+
+    def __init__(self, period=0.4):
+        import threading
+        self.period, self.mhz, self._stop = period, [], threading.Event()
+        self._thread = threading.Thread(target=self._run, daemon=True)
+
+    @staticmethod
+    def read():
+        import re
+        import subprocess
+        try:
+            out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=20).stdout
+        except (OSError, subprocess.SubprocessError):
+            return None
+        m = re.search(r"sclk clock level: \S+ \((\d+)Mhz\)", out)
+        return int(m.group(1)) if m else None
+
+    def _run(self):
+        while not self._stop.is_set():
+            v = self.read()
+            if v is not None:
+                self.mhz.append(v)
+            self._stop.wait(self.period)
+
+    def __enter__(self):
+        self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop.set()
+        self._thread.join()
+
+    def summary(self):
+        if not self.mhz:
+            return None
+        return {"samples": len(self.mhz), "min_mhz": min(self.mhz), "max_mhz": max(self.mhz),
+                "median_mhz": int(statistics.median(self.mhz))}
+
+
 class OpTimer:
     """Times the kernel calls of one step that runs kernel by kernel: every function of
     ``sonicboom_amd.ops`` that launches is wrapped between two events on the stream, and the
@@ -173,6 +215,8 @@ def main() -> int:
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--no-graph", action="store_true", help="launch decode steps kernel by kernel")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel rates")
+    ap.add_argument("--clocks", action="store_true",
+                    help="also run prompt steps back to back for a few seconds and sample the engine clock meanwhile")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported")
@@ -294,6 +338,22 @@ def main() -> int:
             engine.step([StepEntry(slot, random_prompts([PROMPT])[0], (PROMPT - 1,))])
         engine.free_slot(slot)
         prefill["kernels"] = kernel_rates(m, timer.totals(), PROMPT, 0, prefill_lengths=[PROMPT])
+    if a.clocks:
+        idle = ClockSampler.read()
+        p = random_prompts([PROMPT])[0]
+        with ClockSampler() as sampler:
+            t_end = time.time() + 6.0
+            n_runs, t_run = 0, 0.0
+            while time.time() < t_end:
+                slot = engine.alloc_slot()
+                t_run += sync_time(lambda: engine.step([StepEntry(slot, p, (PROMPT - 1,))]))
+                engine.free_slot(slot)
+                n_runs += 1
+        clocks = sampler.summary()
+        if clocks is not None:
+            clocks.update(idle_mhz=idle, prompt_steps=n_runs, ms_per_prompt_step=round(t_run / n_runs * 1e3, 3),
+                          frac_at_median_clock=round(pf / (t_run / n_runs) / (PEAK_FLOPS["bf16"] * clocks["median_mhz"] / 2400.0), 4))
+        prefill["clocks"] = clocks
     print(f"[bench] prefill {prefill}", file=sys.stderr, flush=True)
     del engine
 
