@@ -1,9 +1,9 @@
 // bf16 matrix product for many rows (prefill):  Y[t,n] = sum_k X[t,k] W[n,k]
 // on the matrix cores, with the model's epilogues fused: bias, float32
-// residual, SiLU gate, float32 or bfloat16 output.
+// residual, gate activation, float32 or bfloat16 output.
 //
-// A block of 256 threads (2 x 2 waves) owns a BM x 128 tile of Y (BM = 128 or
-// 256 rows) and walks K in stages of BK (32 or 64).  Both operand tiles go
+// A block of 2 x NW waves owns a BM x BN tile of Y (128 x 128, 256 x 128 or
+// 256 x 256) and walks K in stages of BK.  Both operand tiles go
 // global -> registers -> LDS, the next stage's loads being issued before the
 // current stage's MFMAs (two LDS buffers, one barrier per stage).  An LDS row
 // holds BK k (BK / 8 chunks of 16 bytes); chunk c of row r is stored at chunk
@@ -11,7 +11,7 @@
 // rows fall on distinct banks.  A wave owns (BM / 2) x 64: MT x 2 tiles of
 // v_mfma_f32_32x32x16_bf16, A = rows of X, B = rows of W, so a lane holds one
 // output column of 16 rows.  The taller tile halves the LDS reads per MFMA;
-// the launcher picks it when the grid still fills the chip.
+// the launcher picks the shape from the problem's sizes.
 //
 // Block order: consecutive block numbers go to different XCDs (each with its
 // own L2).  The grid is walked so that the blocks one XCD runs at a time share
@@ -91,7 +91,17 @@ gemm_mfma_kernel(Args a) {
   // row have to be zeroed by hand (EVEN_K: there are none).  Load i + 1 lands kThreads chunks
   // after load i in LDS (its rows are a multiple of 16 further on, so the swizzle term repeats).
   static_assert((kThreads / CPR) % 16 == 0, "rows per load must keep the swizzle term");
-  uint32_t off[kLoads];       // byte offset of the load at stage 0
+  // Byte offset of load i at stage 0.  With packed weights the loads of an operand lie a constant
+  // stride apart (nothing is clamped: what lies past an operand's end is out of the descriptor's
+  // range and reads as zero), so two offsets and two strides stand for all of them; kept as an
+  // array they did not fit the registers beside 128 accumulators, and the one the compiler
+  // spilled came back through a scratch load whose wait (the memory counter runs in order) also
+  // waited for every global load just issued, once in every two stages.
+  constexpr bool kLinear = PACKED && (kThreads / 64) % kSteps32 == 0 &&
+                           (!GATED || (kThreads / 64 / kSteps32) % 4 == 0);   // see the loads of W below
+  constexpr int kOffsets = kLinear ? 2 : kLoads;
+  uint32_t off[kOffsets];
+  uint32_t stride_a = 0, stride_b = 0;
   int kpos[kLoads];           // !EVEN_K: first k of the chunk within the stage (packed: of its k-step)
   int slot_a0, slot_b0;       // LDS chunk index of loads 0 of A and of B
   const size_t w_rows_total = size_t(GATED ? 2 : 1) * (PACKED ? size_t(a.w_tiles) * 16 : size_t(a.n_out));
@@ -103,8 +113,15 @@ gemm_mfma_kernel(Args a) {
 #pragma unroll
   for (int i = 0; i < kLoadsA; ++i) {
     const int id = tid + kThreads * i, row = id / CPR, c = id % CPR;
-    const int t = min(t0 + row, a.n_rows);          // n_rows: one past the end, reads zeros
-    off[i] = uint32_t((size_t(t) * a.n_in + c * 8) * 2);
+    if (kLinear) {
+      // rows past the last one lie past the descriptor's end (the host has checked that their
+      // offsets still fit 32 bits)
+      if (i == 0) off[0] = uint32_t((size_t(t0 + row) * a.n_in + c * 8) * 2);
+      stride_a = uint32_t(size_t(kThreads / CPR) * a.n_in * 2);
+    } else {
+      const int t = min(t0 + row, a.n_rows);          // n_rows: one past the end, reads zeros
+      off[i] = uint32_t((size_t(t) * a.n_in + c * 8) * 2);
+    }
     if (i == 0) slot_a0 = swz<CPR>(row, c);
     kpos[i] = c * 8;
   }
@@ -115,14 +132,32 @@ gemm_mfma_kernel(Args a) {
       // load id -> 1 KB block (id / 64) = (row tile of the LDS tile, k-step), lane id % 64
       const int blk = id >> 6, l = id & 63;
       const int rt = blk / kSteps32, j = blk % kSteps32;   // LDS rows rt * 16 .., k-step j of the stage
-      int tile;
-      if (GATED) {
-        const int half = rt >> 2, within = rt & 3;
-        tile = (within >> 1) * a.w_tiles + min(n0 / 16 + half * 2 + (within & 1), a.w_tiles - 1);
+      if constexpr (kLinear) {
+        // load i + 1 takes the block kThreads / 64 further on: the same k-step, row tile
+        // rt + kThreads / 64 / kSteps32, which is a constant number of tiles of W further on
+        if (i == 0) {
+          int tile;
+          if (GATED) {
+            const int half = rt >> 2, within = rt & 3;
+            tile = (within >> 1) * a.w_tiles + n0 / 16 + half * 2 + (within & 1);
+          } else {
+            tile = n0 / 16 + rt;
+          }
+          // a tile past the last: past the half's (or the matrix's) end; its columns are not stored
+          off[1] = uint32_t(((size_t(tile) * a.w_steps + j) * 512 + size_t(l) * 8) * 2);
+          constexpr int kTilesApart = GATED ? (kThreads / 64 / kSteps32) / 2 : kThreads / 64 / kSteps32;
+          stride_b = uint32_t(size_t(kTilesApart) * a.w_steps * 1024);
+        }
       } else {
-        tile = min(n0 / 16 + rt, a.w_tiles - 1);
+        int tile;
+        if (GATED) {
+          const int half = rt >> 2, within = rt & 3;
+          tile = (within >> 1) * a.w_tiles + min(n0 / 16 + half * 2 + (within & 1), a.w_tiles - 1);
+        } else {
+          tile = min(n0 / 16 + rt, a.w_tiles - 1);
+        }
+        off[kLoadsA + i] = uint32_t(((size_t(tile) * a.w_steps + j) * 512 + size_t(l) * 8) * 2);
       }
-      off[kLoadsA + i] = uint32_t(((size_t(tile) * a.w_steps + j) * 512 + size_t(l) * 8) * 2);
       if (i == 0) slot_b0 = swz<CPR>(rt * 16 + (l & 15), j * 4 + (l >> 4));
       kpos[kLoadsA + i] = j * 32;
     } else {
@@ -160,8 +195,11 @@ gemm_mfma_kernel(Args a) {
     const bool is_a = i < kLoadsA;
     // uniform part of the address: the stage's offset along K
     const int stage_off = (PACKED && !is_a) ? kt * (kSteps32 * 1024) : kt * (BK * 2);
+    uint32_t offset;
+    if constexpr (kLinear) offset = is_a ? off[0] + uint32_t(i) * stride_a : off[1] + uint32_t(i - kLoadsA) * stride_b;
+    else offset = off[i];
     bf16x8_t v = __builtin_bit_cast(
-        bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(is_a ? rsrc_x : rsrc_w, int(off[i]), stage_off, 0));
+        bf16x8_t, __builtin_amdgcn_raw_buffer_load_b128(is_a ? rsrc_x : rsrc_w, int(offset), stage_off, 0));
     if (!EVEN_K) {
       const bool ok = (PACKED && !is_a) ? (kt * BK + kpos[i] < a.w_steps * 32) : (kt * BK + kpos[i] < a.n_in);
       if (!ok) v = bf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
@@ -427,8 +465,10 @@ extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void
   // the kernel addresses both operands with 32-bit byte offsets
   const unsigned long long w_rows = (unsigned long long)((n_out + 15) / 16 * 16) * (gated ? 2 : 1);
   const unsigned long long k_padded = (unsigned long long)((n_in + 31) / 32 * 32);
-  SB_SUPPORT(((unsigned long long)n_rows + 1) * n_in * 2 < (1ull << 32) - (1ull << 20) &&
-                 w_rows * k_padded * 2 < (1ull << 32) - (1ull << 20),
+  // ... also for the rows and row tiles past an operand's end that a block at the edge asks for
+  // (they lie past the descriptor's end and read as zero, but must not wrap around)
+  SB_SUPPORT(((unsigned long long)n_rows + 257) * n_in * 2 < (1ull << 32) - (1ull << 20) &&
+                 (w_rows + 512) * k_padded * 2 < (1ull << 32) - (1ull << 20),
              "sb_gemm_mfma_bf16: an operand of 4 GiB or more (rows=%d out=%d in=%d)", n_rows, n_out, n_in);
   hipStream_t s = (hipStream_t)stream;
   a.w_tiles = (n_out + 15) / 16;
@@ -481,8 +521,9 @@ extern "C" int sb_gemm_mfma_partial_bf16(float *partial, const void *x, const vo
   SB_SUPPORT(blocks <= 0x7fffffffLL, "sb_gemm_mfma_partial_bf16: too many tiles");
   const unsigned long long w_rows = (unsigned long long)((n_out + 15) / 16 * 16);
   const unsigned long long k_padded = (unsigned long long)((n_in + 31) / 32 * 32);
-  SB_SUPPORT(((unsigned long long)n_rows + 1) * n_in * 2 < (1ull << 32) - (1ull << 20) &&
-                 w_rows * k_padded * 2 < (1ull << 32) - (1ull << 20),
+  // with room for the rows and row tiles past an operand's end that a block at the edge asks for
+  SB_SUPPORT(((unsigned long long)n_rows + 257) * n_in * 2 < (1ull << 32) - (1ull << 20) &&
+                 (w_rows + 512) * k_padded * 2 < (1ull << 32) - (1ull << 20),
              "sb_gemm_mfma_partial_bf16: an operand of 4 GiB or more");
   a.w_tiles = (n_out + 15) / 16;
   a.w_steps = (n_in + 31) / 32;
