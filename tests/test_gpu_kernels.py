@@ -215,6 +215,64 @@ def test_gemm_bf16_every_tile_shape(shape, packed, t, n, k):
         close(got, g / (1.0 + torch.exp(-g)) * u, atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"gated shape {shape}")
 
 
+@pytest.mark.parametrize("shape, path", [(0, "direct"), (1, "direct"), (2, "direct"), (3, "direct"),
+                                         (2, "direct, a block a tile"), (0, "registers"), (2, "registers")])
+@pytest.mark.parametrize("t, n, k", [(65, 100, 64), (300, 226, 192), (520, 264, 128), (257, 1001, 448), (130, 72, 2368)])
+def test_gemm_bf16_every_path(shape, path, t, n, k):
+    """The kernel that loads its tiles straight into LDS (inner sizes in 64s, packed weights) and
+    the one that stages them through registers, forced for every tile shape: rows and columns
+    that end inside a tile, widths that are no multiple of 4 (single stores in the epilogue),
+    bias and residual, bfloat16 and float32 results, plain and gated."""
+    from sonicboom_amd import ops
+    x, w = randn(t, k, dtype=BF16), randn(n, k, dtype=BF16, scale=0.05)
+    bias, resid = randn(n, scale=0.1), randn(t, n)
+    wd = w.to(DEV)
+    with ops.gemm_tile_shape(shape, path):
+        got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(wd), bias.to(DEV), resid.to(DEV), F32, packed_shape=(n, k))
+        close(got, ref_gemm(x, w, bias, resid), atol=3e-5 * math.sqrt(k), rtol=1e-5, what=f"shape {shape} {path}")
+        got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(wd), bias.to(DEV), None, BF16, packed_shape=(n, k))
+        close(got, ref_gemm(x, w, bias, None), atol=0.01 * math.sqrt(k) * 0.05 + 0.01, rtol=0.01, what=f"bf16 shape {shape} {path}")
+        inner = n // 2
+        gu = x.double() @ w[:2 * inner].double().T
+        g, u = gu[:, :inner], gu[:, inner:]
+        wg = wd[:2 * inner].contiguous()
+        for act, want in (("silu", g / (1.0 + torch.exp(-g)) * u),
+                          ("gelu_tanh", 0.5 * g * (1 + torch.tanh(0.7978845608028654 * g * (1 + 0.044715 * g * g))) * u)):
+            got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(wg, True), None, None, F32, gated=act, packed_shape=(2 * inner, k))
+            close(got, want, atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"gated {act} shape {shape} {path}")
+
+
+def test_gemm_bf16_blocks_that_go_from_tile_to_tile():
+    """More 256 x 256 tiles than the GPU has CUs: the blocks of the kernel that loads straight into
+    LDS go on to a second tile, whose first stage the first tile's last stage has loaded; in
+    bands of eight tiles along the rows, the last band lower.  Every tile has a value of its own."""
+    from sonicboom_amd import ops
+    t, n, k = 4400, 4200, 128                  # 18 x 17 = 306 tiles; gated: 18 x 33 tiles of 256 x 128
+    x, w = randn(t, k, dtype=BF16), randn(n, k, dtype=BF16, scale=0.05)
+    want = ref_gemm(x, w, None, None)
+    wd = w.to(DEV)
+    for path in ("direct", "direct, a block a tile"):
+        with ops.gemm_tile_shape(2, path):
+            got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(wd), None, None, F32, packed_shape=(n, k))
+            close(got, want, atol=3e-5 * math.sqrt(k), rtol=1e-5, what=path)
+            inner = n // 2
+            g, u = want[:, :inner].double(), want[:, inner:2 * inner].double()
+            got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(wd[:2 * inner].contiguous(), True), None, None, F32,
+                                gated=True, packed_shape=(2 * inner, k))
+            close(got, g / (1.0 + torch.exp(-g)) * u, atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"gated {path}")
+
+
+def test_gemm_bf16_direct_path_refuses_what_it_cannot_take():
+    from sonicboom_amd import ops
+    x, w = randn(70, 96, dtype=BF16).to(DEV), randn(64, 96, dtype=BF16).to(DEV)
+    with ops.gemm_tile_shape(0, "direct"):
+        with pytest.raises(ops.KernelLibraryError, match="inner size in 64s"):
+            ops.gemm_bf16(x, ops.pack_weight(w), None, None, F32, packed_shape=(64, 96))
+    with ops.gemm_tile_shape(3, "registers"):
+        with pytest.raises(ops.KernelLibraryError, match="direct path only"):
+            ops.gemm_bf16(x, ops.pack_weight(w), None, None, F32, packed_shape=(64, 96))
+
+
 @pytest.mark.parametrize("t", [1, 16, 17, 40, 64, 65, 100, 128])
 @pytest.mark.parametrize("waves", [0, 4, 5, 6, 7, 8])
 @pytest.mark.parametrize("n, k", [(100, 96), (1000, 520), (264, 2368), (4099, 264)])
