@@ -584,7 +584,8 @@ gemm_direct16_kernel(Args a) {
   // 0, 1 are the gate and 2, 3 the up projection of the same 32 features.  PITCH = NC + 4: the
   // four row groups of a store fall on four different quarters of the banks.
   constexpr int NC = GATED ? 32 : 64, kPitch = NC + 4;
-  static_assert(kBufChunks * 16 >= kWaves * 16 * kPitch * 4, "the turning areas must fit a stage buffer");
+  static_assert((NBUF == 2 ? 1 : NBUF) * kBufChunks * 16 >= kWaves * 16 * kPitch * 4,
+                "the turning areas must fit a stage buffer (two buffers: the other one may hold the next tile)");
   auto epilogue = [&](int m, int n, int buf_free) {
     store_tile<MT16, 16, NW, NC, kPitch>(
         a, reinterpret_cast<float *>(lds + buf_free * kBufChunks), m * BM, n * (GATED ? BN / 2 : BN), !GATED,
