@@ -704,22 +704,78 @@ struct RopeArgs {
   int store;                   // keys and values go into the cache (0: a layer that reads another's)
 };
 
-// Eight consecutive elements e0 .. e0+7 of sequence seq's qkv row: slices in ascending order, then the bias.
-__device__ __forceinline__ void qkv8(float (&v)[8], const RopeArgs &ra, int seq, size_t e0) {
+// Eight consecutive elements e0 .. e0+7 of sequence seq's qkv row, and the eight from p0 on (the
+// partners in the rotation, or anything valid if there are none): slices in ascending order,
+// then the bias.  The loads of four slices of both go out before the first sum (a loop that adds
+// slice after slice waits for memory once per slice: three slices and a partner cost the kernel
+// six trips to L2 in a row); a slice past the last is the last once more and is not added, so
+// the sums have the bits of the loop.  More than four slices: a second round of four.
+struct Row8 { float4 lo, hi; };
+__device__ __forceinline__ void add_if(Row8 &a, const Row8 &c, bool use) {
+  a.lo.x = use ? a.lo.x + c.lo.x : a.lo.x; a.lo.y = use ? a.lo.y + c.lo.y : a.lo.y;
+  a.lo.z = use ? a.lo.z + c.lo.z : a.lo.z; a.lo.w = use ? a.lo.w + c.lo.w : a.lo.w;
+  a.hi.x = use ? a.hi.x + c.hi.x : a.hi.x; a.hi.y = use ? a.hi.y + c.hi.y : a.hi.y;
+  a.hi.z = use ? a.hi.z + c.hi.z : a.hi.z; a.hi.w = use ? a.hi.w + c.hi.w : a.hi.w;
+}
+__device__ __forceinline__ Row8 load8(const float *p) {
+  return Row8{*reinterpret_cast<const float4 *>(p), *reinterpret_cast<const float4 *>(p + 4)};
+}
+// What qkv8x2_issue has asked for: the first four slices and the bias of both runs of eight.
+struct Raw8x2 {
+  Row8 cx[4], cp[4], bx, bp;
+  size_t e0, p0;
+};
+__device__ __forceinline__ void qkv8x2_issue(Raw8x2 &raw, const RopeArgs &ra, int seq, size_t e0, size_t p0) {
+  const float *rx = ra.qkv + size_t(seq) * ra.row_stride + e0, *rp = ra.qkv + size_t(seq) * ra.row_stride + p0;
+  raw.e0 = e0;
+  raw.p0 = p0;
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    const size_t so = size_t(min(s, ra.n_slices - 1)) * ra.slice_stride;
+    raw.cx[s] = load8(rx + so);
+    raw.cp[s] = load8(rp + so);
+  }
+  // 16-byte aligned like the row: e0 and p0 are multiples of 8 (without a bias: the row itself, not added)
+  raw.bx = load8(ra.bias ? ra.bias + e0 : rx);
+  raw.bp = load8(ra.bias ? ra.bias + p0 : rp);
+}
+__device__ __forceinline__ void qkv8x2_finish(float (&x)[8], float (&p)[8], const Raw8x2 &raw, const RopeArgs &ra, int seq) {
+  Row8 ax = raw.cx[0], ap = raw.cp[0];
+#pragma unroll
+  for (int s = 1; s < 4; ++s) {
+    add_if(ax, raw.cx[s], s < ra.n_slices);
+    add_if(ap, raw.cp[s], s < ra.n_slices);
+  }
+  if (ra.n_slices > 4) {     // uniform
+    const float *rx = ra.qkv + size_t(seq) * ra.row_stride + raw.e0, *rp = ra.qkv + size_t(seq) * ra.row_stride + raw.p0;
+    Row8 cx[4], cp[4];
+#pragma unroll
+    for (int s = 4; s < 8; ++s) {
+      const size_t so = size_t(min(s, ra.n_slices - 1)) * ra.slice_stride;
+      cx[s - 4] = load8(rx + so);
+      cp[s - 4] = load8(rp + so);
+    }
+#pragma unroll
+    for (int s = 4; s < 8; ++s) {
+      add_if(ax, cx[s - 4], s < ra.n_slices);
+      add_if(ap, cp[s - 4], s < ra.n_slices);
+    }
+  }
+  add_if(ax, raw.bx, ra.bias != nullptr);
+  add_if(ap, raw.bp, ra.bias != nullptr);
+  x[0] = ax.lo.x; x[1] = ax.lo.y; x[2] = ax.lo.z; x[3] = ax.lo.w; x[4] = ax.hi.x; x[5] = ax.hi.y; x[6] = ax.hi.z; x[7] = ax.hi.w;
+  p[0] = ap.lo.x; p[1] = ap.lo.y; p[2] = ap.lo.z; p[3] = ap.lo.w; p[4] = ap.hi.x; p[5] = ap.hi.y; p[6] = ap.hi.z; p[7] = ap.hi.w;
+}
+
+// The same sums slice after slice, with few registers: for the items past a block's first 256,
+// which are fetched while the page's fragments are held (only a group of fifteen or sixteen
+// heads has any).
+__device__ __forceinline__ void qkv8_in_turn(float (&v)[8], const RopeArgs &ra, int seq, size_t e0) {
   const float *r = ra.qkv + size_t(seq) * ra.row_stride + e0;
-  float4 a = *reinterpret_cast<const float4 *>(r), b = *reinterpret_cast<const float4 *>(r + 4);
-  for (int s = 1; s < ra.n_slices; ++s) {
-    const float4 c = *reinterpret_cast<const float4 *>(r + s * ra.slice_stride);
-    const float4 d = *reinterpret_cast<const float4 *>(r + s * ra.slice_stride + 4);
-    a.x += c.x; a.y += c.y; a.z += c.z; a.w += c.w;
-    b.x += d.x; b.y += d.y; b.z += d.z; b.w += d.w;
-  }
-  if (ra.bias) {       // 16-byte aligned like the row: e0 is a multiple of 8
-    const float4 c = *reinterpret_cast<const float4 *>(ra.bias + e0), d = *reinterpret_cast<const float4 *>(ra.bias + e0 + 4);
-    a.x += c.x; a.y += c.y; a.z += c.z; a.w += c.w;
-    b.x += d.x; b.y += d.y; b.z += d.z; b.w += d.w;
-  }
-  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  Row8 a = load8(r);
+  for (int s = 1; s < ra.n_slices; ++s) add_if(a, load8(r + s * ra.slice_stride), true);
+  if (ra.bias) add_if(a, load8(ra.bias + e0), true);
+  v[0] = a.lo.x; v[1] = a.lo.y; v[2] = a.lo.z; v[3] = a.lo.w; v[4] = a.hi.x; v[5] = a.hi.y; v[6] = a.hi.z; v[7] = a.hi.w;
 }
 
 // Eight floats rounded as sb_rope_kv_store rounds (to nearest even, a NaN stays one), packed.
@@ -740,6 +796,7 @@ struct RopeShared {
   uint4 q[16 * kQStride];
   uint4 k[HD / 8];      // the row's own key, rotated and rounded
   bf16_t v[HD];         // and its value
+  int page_of_wave[4];  // the page numbers the block's waves have looked up (kernels with a page a wave)
 };
 
 // Work item `it` of a block of the folded form: eight elements d0 .. d0+7 of one head of the qkv
@@ -753,12 +810,33 @@ __device__ __forceinline__ size_t item_head(int it, int n_q, int kvh, int group,
   if (it < n_q) return size_t(kvh * group + it / kPerHead) * HD;
   return size_t((it < n_q + kPerHead ? heads_q : heads_q + heads_kv) + kvh) * HD;
 }
-__device__ __forceinline__ void fetch_item(RopeItem &v, const RopeArgs &ra, int seq, int it, int n_q, int kvh,
-                                           int group, int heads_q, int heads_kv, int half) {
+__device__ __forceinline__ void item_offsets(size_t &e0, size_t &p0, bool &paired, int it, int n_q, int kvh, int group,
+                                             int heads_q, int heads_kv, int half) {
   const size_t hoff = item_head(it, n_q, kvh, group, heads_q, heads_kv);
   const int d0 = (it < n_q ? it % kPerHead : (it - n_q) % kPerHead) * 8;
-  qkv8(v.x, ra, seq, hoff + d0);
-  if (it < n_q + kPerHead && d0 < 2 * half) qkv8(v.p, ra, seq, hoff + (d0 < half ? d0 + half : d0 - half));
+  paired = it < n_q + kPerHead && d0 < 2 * half;
+  e0 = hoff + d0;
+  // an item without a partner (a value, an element past the rotated ones) stands in for it itself
+  p0 = hoff + (!paired ? d0 : d0 < half ? d0 + half : d0 - half);
+}
+// a thread's first item: all its loads at once ...
+__device__ __forceinline__ void fetch_item(RopeItem &v, const RopeArgs &ra, int seq, int it, int n_q, int kvh,
+                                           int group, int heads_q, int heads_kv, int half) {
+  size_t e0, p0;
+  bool paired;
+  item_offsets(e0, p0, paired, it, n_q, kvh, group, heads_q, heads_kv, half);
+  Raw8x2 raw;
+  qkv8x2_issue(raw, ra, seq, e0, p0);
+  qkv8x2_finish(v.x, v.p, raw, ra, seq);
+}
+// ... and a later one, slice after slice
+__device__ __forceinline__ void fetch_item_in_turn(RopeItem &v, const RopeArgs &ra, int seq, int it, int n_q, int kvh,
+                                                   int group, int heads_q, int heads_kv, int half) {
+  size_t e0, p0;
+  bool paired;
+  item_offsets(e0, p0, paired, it, n_q, kvh, group, heads_q, heads_kv, half);
+  qkv8_in_turn(v.x, ra, seq, e0);
+  if (paired) qkv8_in_turn(v.p, ra, seq, p0);
 }
 // The item's eight results: rotated queries and keys, the value as it is.
 __device__ __forceinline__ void finish_item(float (&y)[8], const RopeItem &v, int it, int n_q, int half,
@@ -790,7 +868,8 @@ __device__ __forceinline__ void finish_item(float (&y)[8], const RopeItem &v, in
 __device__ __forceinline__ void rope_store(RopeShared &sh, const RopeItem &first, float freq, const RopeArgs &ra,
                                            int seq, int pos, int kvh, int group, int heads_q, int heads_kv,
                                            bool mine, bool visible, bf16_t *k_cache, bf16_t *v_cache,
-                                           const int32_t *page_table, int max_pages, int n_pages_total) {
+                                           const int32_t *page_table, int max_pages, int n_pages_total,
+                                           int first_page_of_block = -1) {
   const int half = ra.inv_freq ? ra.rot_dims / 2 : 0;
   if (int(threadIdx.x) < 2 * half) {
     const int j = threadIdx.x, i = j < half ? j : j - half;
@@ -799,18 +878,26 @@ __device__ __forceinline__ void rope_store(RopeShared &sh, const RopeItem &first
     if (j < half) sh.cs[i] = cosf(theta);
     else sh.sn[i] = sinf(theta);
   }
+  // The page that takes the row's own key and value.  first_page_of_block >= 0: wave w of the
+  // block has looked up page first_page_of_block + w of the row already and left its number in
+  // sh.page_of_wave[w], which saves a trip to memory that could only start once the position was known.
   int page = -1;
-  if (ra.store && mine) {
-    const int lp = pos / SB_PAGE;
+  const int lp = pos / SB_PAGE;
+  if (ra.store && mine && first_page_of_block < 0) {
     page = lp < max_pages ? page_table[size_t(seq) * max_pages + lp] : -1;
     if (page >= n_pages_total) page = -1;
   }
-  if (half > 0) __syncthreads();
+  if (half > 0 || first_page_of_block >= 0) __syncthreads();
+  if (ra.store && mine && first_page_of_block >= 0) {
+    const int w = lp - first_page_of_block;
+    page = (w >= 0 && w < 4 && lp < max_pages) ? sh.page_of_wave[w] : -1;
+    if (page >= n_pages_total) page = -1;
+  }
   const int n_q = group * kPerHead;
   const int n_items = n_q + (page >= 0 ? 2 * kPerHead : 0);
   for (int it = threadIdx.x; it < n_items; it += blockDim.x) {
     RopeItem later;
-    if (it != int(threadIdx.x)) fetch_item(later, ra, seq, it, n_q, kvh, group, heads_q, heads_kv, half);
+    if (it != int(threadIdx.x)) fetch_item_in_turn(later, ra, seq, it, n_q, kvh, group, heads_q, heads_kv, half);
     float y[8];
     finish_item(y, it == int(threadIdx.x) ? first : later, it, n_q, half, sh.cs, sh.sn);
     if (it < n_q) {
@@ -905,8 +992,13 @@ attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *
   const DecodeBlock blk = decode_block(tiles, n_seqs);
   const int chunk = blk.chunk, seq = blk.seq;
   const int kvh = blk.tile / head_tiles, ht = blk.tile - kvh * head_tiles;
+  // the wave's page number does not depend on the position: both look-ups go out together, and
+  // before everything else, since the page's loads wait for them
+  const int pg = chunk * kPagesPerChunk + wave;
+  const int page_looked_up = page_table[size_t(seq) * max_pages + min(pg, max_pages - 1)];
+  const int pos = row_pos[seq];
   // the folded form: this thread's share of the qkv row depends on the block's number only, so
-  // its loads go out before anything else
+  // its loads go out right behind them
   RopeItem first;
   if constexpr (FUSED) {
     const int n_q = group * kPerHead, n_all = n_q + (ra.store ? 2 * kPerHead : 0);
@@ -914,10 +1006,6 @@ attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *
       fetch_item(first, ra, seq, threadIdx.x, n_q, kvh, group, heads_q, heads_kv, ra.inv_freq ? ra.rot_dims / 2 : 0);
   }
   const float freq = FUSED ? rope_freq(ra) : 0.f;
-  // the wave's page number does not depend on the position: both look-ups go out together
-  const int pg = chunk * kPagesPerChunk + wave;
-  const int page_looked_up = page_table[size_t(seq) * max_pages + min(pg, max_pages - 1)];
-  const int pos = row_pos[seq];
   const int key_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
   const int first_chunk = key_lo / (SB_PAGE * kPagesPerChunk);
   const int last_chunk = min(pos / (SB_PAGE * kPagesPerChunk), n_chunks - 1);
@@ -954,8 +1042,10 @@ attn_decode_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, float *
       if (use0) load_half(h0, k_cache + off, v_cache + off, 0, lane);
       if (use1) load_half(h1, k_cache + off, v_cache + off, 1, lane);
     }
+    if (lane == 0) rope_sh.page_of_wave[wave] = page_looked_up;
     rope_store(rope_sh, first, freq, ra, seq, pos, kvh, group, heads_q, heads_kv, chunk == last_chunk, !kEarly,
-               const_cast<bf16_t *>(k_cache), const_cast<bf16_t *>(v_cache), page_table, max_pages, n_pages_total);
+               const_cast<bf16_t *>(k_cache), const_cast<bf16_t *>(v_cache), page_table, max_pages, n_pages_total,
+               chunk * kPagesPerChunk);
     staged_q(qf[0], rope_sh, hq, col_ok, lane);
     if (kEarly) {
       const int slot = pos % SB_PAGE;
@@ -997,6 +1087,7 @@ attn_decode_long_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, fl
   const DecodeBlock blk = decode_block(tiles, n_seqs);
   const int chunk = blk.chunk, seq = blk.seq;
   const int kvh = blk.tile / head_tiles, ht = blk.tile - kvh * head_tiles;
+  const int pos = row_pos[seq];
   RopeItem first;       // the folded form: see attn_decode_kernel
   if constexpr (FUSED) {
     const int n_q = group * kPerHead, n_all = n_q + (ra.store ? 2 * kPerHead : 0);
@@ -1005,7 +1096,6 @@ attn_decode_long_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, fl
   }
   const float freq = FUSED ? rope_freq(ra) : 0.f;
   const int pages_per_chunk = kPagesPerChunk * ppw;
-  const int pos = row_pos[seq];
   const int key_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
   const int first_chunk = key_lo / (SB_PAGE * pages_per_chunk);
   const int last_chunk = min(pos / (SB_PAGE * pages_per_chunk), n_chunks - 1);
@@ -1093,14 +1183,50 @@ attn_decode_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ par
   const int head_tiles = (group + 15) / 16;
   const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y - kvh * head_tiles;
   const int pos = row_pos[seq];
+  const int e = blockIdx.x * 256 + threadIdx.x;
+  const size_t tile_index = size_t(seq) * gridDim.y + blockIdx.y;
+  const float *po = part_o + (tile_index * n_chunks) * (HD * 16), *pml = part_ml + (tile_index * n_chunks) * 32;
+  // Up to kAtOnce chunks: the partial results of all of them are asked for together with the
+  // position, which says which of them count (a chunk past the last is the last once more);
+  // waiting for the position first costs this short kernel a trip to memory of its two.
+  constexpr int kAtOnce = 16;
+  float mv[kAtOnce], lv[kAtOnce], ov[kAtOnce];
+  const bool at_once = n_chunks <= kAtOnce && e < HD * 16;
+  if (at_once) {
+    const int c = e & 15;
+#pragma unroll
+    for (int ch = 0; ch < kAtOnce; ++ch) {
+      const size_t cc = size_t(min(ch, n_chunks - 1));
+      mv[ch] = pml[cc * 32 + c];
+      lv[ch] = pml[cc * 32 + 16 + c];
+      ov[ch] = po[cc * (HD * 16) + e];
+    }
+  }
   const int key_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
   const int first = key_lo / (SB_PAGE * pages_per_chunk), last = min(pos / (SB_PAGE * pages_per_chunk), n_chunks - 1);
   if (first == last) return;      // the decode kernel has written the result itself
-  const int e = blockIdx.x * 256 + threadIdx.x;
   if (e >= HD * 16) return;
-  const size_t tile_index = size_t(seq) * gridDim.y + blockIdx.y;
-  merge_element(out, part_o + (tile_index * n_chunks) * (HD * 16), part_ml + (tile_index * n_chunks) * 32, e,
-                first, last, seq, heads_q, kvh, ht, group);
+  if (!at_once) {
+    merge_element(out, po, pml, e, first, last, seq, heads_q, kvh, ht, group);
+    return;
+  }
+  // as merge_element: rescaled to the common maximum and added in ascending chunk order
+  const int c = e & 15, d = e >> 4;
+  const int hh = ht * 16 + c;
+  if (hh >= group) return;
+  float m = -__builtin_inff();
+#pragma unroll
+  for (int ch = 0; ch < kAtOnce; ++ch) m = (ch >= first && ch <= last) ? fmaxf(m, mv[ch]) : m;
+  const float m_use = m == -__builtin_inff() ? 0.f : m;
+  float o = 0.f, l = 0.f;
+#pragma unroll
+  for (int ch = 0; ch < kAtOnce; ++ch) {
+    const bool use = ch >= first && ch <= last;
+    const float f = __builtin_amdgcn_exp2f(mv[ch] - m_use);
+    o = use ? o + ov[ch] * f : o;
+    l = use ? l + lv[ch] * f : l;
+  }
+  out[(size_t(seq) * heads_q + kvh * group + hh) * HD + d] = f32_to_bf16(l > 0.f ? o / l : 0.f);
 }
 
 int check_common(const void *out, const void *q, const void *k, const void *v, const void *pt,
