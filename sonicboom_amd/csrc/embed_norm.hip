@@ -46,14 +46,41 @@ __device__ __forceinline__ double squares(const float4 &v) {
   return double(v.x * v.x) + double(v.y * v.y) + double(v.z * v.z) + double(v.w * v.w);
 }
 
+// Group g (four elements) of a normed row: (x * inv) * w, rounded to the output's type.  Rows and
+// weights that start on 16 bytes (every tensor of the engine) take the weight and leave the
+// result as one load and one store of 8 or 16 bytes; the arithmetic is the same either way.
 template <typename TO>
 __device__ __forceinline__ void write_normed(TO *yr, const float4 &v, int g, float inv, const void *w, int w_dtype) {
   const float x[4] = {v.x, v.y, v.z, v.w};
+  float wv[4] = {1.f, 1.f, 1.f, 1.f};
+  const bool aligned = ((reinterpret_cast<uintptr_t>(yr) | reinterpret_cast<uintptr_t>(w)) & 15) == 0;
+  if (w) {
+    if (aligned && w_dtype == SB_F32) {
+      const float4 t = reinterpret_cast<const float4 *>(w)[g];
+      wv[0] = t.x; wv[1] = t.y; wv[2] = t.z; wv[3] = t.w;
+    } else if (aligned) {
+      const uint2 t = reinterpret_cast<const uint2 *>(w)[g];
+      wv[0] = bf16_to_f32(bf16_t(t.x & 0xffffu)); wv[1] = bf16_to_f32(bf16_t(t.x >> 16));
+      wv[2] = bf16_to_f32(bf16_t(t.y & 0xffffu)); wv[3] = bf16_to_f32(bf16_t(t.y >> 16));
+    } else {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) wv[e] = ld_dyn(w, w_dtype, g * 4 + e);
+    }
+  }
+  float o[4];
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    float o = x[e] * inv;
-    if (w) o = o * ld_dyn(w, w_dtype, g * 4 + e);
-    st_f(yr, g * 4 + e, o);
+    o[e] = x[e] * inv;
+    if (w) o[e] = o[e] * wv[e];
+  }
+  if (!aligned) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) st_f(yr, g * 4 + e, o[e]);
+  } else if constexpr (sizeof(TO) == 4) {
+    reinterpret_cast<float4 *>(yr)[g] = make_float4(o[0], o[1], o[2], o[3]);
+  } else {
+    reinterpret_cast<uint2 *>(yr)[g] = make_uint2(uint32_t(f32_to_bf16(o[0])) | uint32_t(f32_to_bf16(o[1])) << 16,
+                                                   uint32_t(f32_to_bf16(o[2])) | uint32_t(f32_to_bf16(o[3])) << 16);
   }
 }
 

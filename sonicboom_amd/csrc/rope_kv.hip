@@ -144,6 +144,101 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
   }
 }
 
+// Many rows without slices or a bias (a prompt step's qkv rows as the tiled product leaves
+// them), bfloat16 queries and cache, head size and rotary width in 16s: a thread moves eight
+// pairs at a time, 16 bytes per load and store instead of two or four.  One block per row.  The
+// arithmetic is rope_kv_kernel's (every element through float, the same rotate_pair), so the
+// bits are the same.
+__device__ __forceinline__ void load_eight(float (&f)[8], const float *p) {
+  const float4 a = *reinterpret_cast<const float4 *>(p), b = *reinterpret_cast<const float4 *>(p + 4);
+  f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
+}
+__device__ __forceinline__ void load_eight(float (&f)[8], const bf16_t *p) {
+  const uint4 u = *reinterpret_cast<const uint4 *>(p);
+  const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    f[2 * e] = bf16_to_f32(bf16_t(w[e] & 0xffffu));
+    f[2 * e + 1] = bf16_to_f32(bf16_t(w[e] >> 16));
+  }
+}
+template <typename TI>
+__global__ void __launch_bounds__(256)
+rope_kv_rows_kernel(bf16_t *__restrict__ q_out, const TI *__restrict__ qkv, int row_stride,
+                    const float *__restrict__ inv_freq, const float *__restrict__ freq_factors, int rot_dims,
+                    const int32_t *__restrict__ row_pos, const int32_t *__restrict__ row_seq,
+                    bf16_t *__restrict__ k_cache, bf16_t *__restrict__ v_cache,
+                    const int32_t *__restrict__ page_table, int max_pages, int n_pages_total, int heads_q,
+                    int heads_kv, int head_dim) {
+  const int row = blockIdx.x;
+  const int pos = row_pos[row];
+  const TI *r = qkv + size_t(row) * row_stride;
+  bf16_t *qo = q_out + size_t(row) * heads_q * head_dim;
+  const bool rotate = inv_freq != nullptr;
+  const int half = rotate ? rot_dims / 2 : 0;
+  int page_of_row = 0;
+  bool store = heads_kv > 0;
+  if (store) {
+    const int seq = row_seq[row];
+    const int lp = pos / SB_PAGE;
+    const int page = (lp >= 0 && lp < max_pages) ? page_table[size_t(seq) * max_pages + lp] : -1;
+    if (page < 0 || page >= n_pages_total) store = false;  // refused on the host; never write astray
+    page_of_row = page < 0 ? 0 : page;
+  }
+  const size_t head_step = size_t(SB_PAGE) * head_dim;
+  const size_t page_base = size_t(page_of_row) * heads_kv * head_step;
+  const size_t k_base = page_base + size_t(pos % SB_PAGE) * head_dim;
+  const size_t v_base = page_base + size_t(pos % SB_PAGE);
+  __shared__ float cs[kMaxPairs], sn[kMaxPairs];
+  for (int j = threadIdx.x; j < 2 * half; j += blockDim.x) {
+    const int i = j < half ? j : j - half;
+    float theta = float(pos) * inv_freq[i];
+    if (freq_factors) theta = theta / freq_factors[i];
+    if (j < half) cs[i] = cosf(theta);
+    else sn[i] = sinf(theta);
+  }
+  __syncthreads();
+  auto pack = [](const float (&f)[8]) {
+    return make_uint4(uint32_t(f32_to_bf16(f[0])) | uint32_t(f32_to_bf16(f[1])) << 16,
+                      uint32_t(f32_to_bf16(f[2])) | uint32_t(f32_to_bf16(f[3])) << 16,
+                      uint32_t(f32_to_bf16(f[4])) | uint32_t(f32_to_bf16(f[5])) << 16,
+                      uint32_t(f32_to_bf16(f[6])) | uint32_t(f32_to_bf16(f[7])) << 16);
+  };
+  // queries and keys: per head half / 8 groups of eight pairs, then (head_dim - rot_dims) / 8 groups copied
+  const int pair_groups = half / 8, per_head = pair_groups + (head_dim - 2 * half) / 8;
+  const int n_qk = (heads_q + (store ? heads_kv : 0)) * per_head;
+  for (int it = threadIdx.x; it < n_qk; it += blockDim.x) {
+    const int head = it / per_head, w = it % per_head;
+    const TI *src = r + size_t(head) * head_dim;
+    bf16_t *dst = head < heads_q ? qo + size_t(head) * head_dim : k_cache + k_base + size_t(head - heads_q) * head_step;
+    if (w < pair_groups) {
+      const int i0 = w * 8;
+      float lo[8], hi[8], y0[8], y1[8];
+      load_eight(lo, src + i0);
+      load_eight(hi, src + i0 + half);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) rotate_pair(lo[e], hi[e], cs[i0 + e], sn[i0 + e], y0[e], y1[e]);
+      *reinterpret_cast<uint4 *>(dst + i0) = pack(y0);
+      *reinterpret_cast<uint4 *>(dst + i0 + half) = pack(y1);
+    } else {
+      const int d0 = 2 * half + (w - pair_groups) * 8;
+      float v[8];
+      load_eight(v, src + d0);
+      *reinterpret_cast<uint4 *>(dst + d0) = pack(v);
+    }
+  }
+  // values: eight elements a time, each to its own row of the transposed page
+  if (!store) return;
+  const int groups = head_dim / 8;
+  for (int it = threadIdx.x; it < heads_kv * groups; it += blockDim.x) {
+    const int kh = it / groups, d0 = (it % groups) * 8;
+    float v[8];
+    load_eight(v, r + size_t(heads_q + heads_kv + kh) * head_dim + d0);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v_cache[v_base + kh * head_step + size_t(d0 + e) * SB_PAGE] = f32_to_bf16(v[e]);
+  }
+}
+
 }  // namespace
 
 extern "C" int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int qkv_dtype,
@@ -177,6 +272,20 @@ extern "C" int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int q
   if (n_rows == 0) return SB_OK;
   hipStream_t s = (hipStream_t)stream;
   const int n_heads = heads_q + 2 * heads_kv;
+  const uintptr_t addresses = reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(q_out) |
+                              reinterpret_cast<uintptr_t>(k_cache);
+  if (n_rows >= 512 && q_dtype == SB_BF16 && cache_dtype == SB_BF16 && n_slices == 1 && !bias && head_dim % 8 == 0 &&
+      row_stride % 8 == 0 && (!inv_freq || rot_dims % 16 == 0) && addresses % 16 == 0) {
+    if (qkv_dtype == SB_BF16)
+      rope_kv_rows_kernel<bf16_t><<<n_rows, 256, 0, s>>>(
+          (bf16_t *)q_out, (const bf16_t *)qkv, row_stride, inv_freq, freq_factors, rot_dims, row_pos, row_seq,
+          (bf16_t *)k_cache, (bf16_t *)v_cache, page_table, max_pages, n_pages_total, heads_q, heads_kv, head_dim);
+    else
+      rope_kv_rows_kernel<float><<<n_rows, 256, 0, s>>>(
+          (bf16_t *)q_out, (const float *)qkv, row_stride, inv_freq, freq_factors, rot_dims, row_pos, row_seq,
+          (bf16_t *)k_cache, (bf16_t *)v_cache, page_table, max_pages, n_pages_total, heads_q, heads_kv, head_dim);
+    return sb::check_launch("sb_rope_kv_store");
+  }
   const int heads_per_block = n_rows >= 512 ? n_heads : 4;
   const dim3 grid(n_rows, (n_heads + heads_per_block - 1) / heads_per_block);
   SB_SUPPORT(grid.y <= 65535, "sb_rope_kv_store: too many heads");

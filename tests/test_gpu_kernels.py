@@ -462,6 +462,37 @@ def test_rope_kv_store_many_rows_equals_few_rows(hq, hkv, hd, rot):
     close(results[0][0], want_q, atol=2e-2, rtol=8e-3, what="q of the long prompt")
 
 
+@pytest.mark.parametrize("hq, hkv, hd, rot", [(7, 1, 48, 0), (28, 4, 128, 0), (3, 3, 64, 32), (5, 2, 80, 0), (2, 0, 32, 0)])
+@pytest.mark.parametrize("rotate", [True, False])
+@pytest.mark.parametrize("in_dtype", [F32, BF16])
+def test_rope_kv_store_rows_eight_pairs_at_a_time(hq, hkv, hd, rot, rotate, in_dtype):
+    """A prompt step's qkv rows (float32 as the engine has them, or bfloat16; no slices, no bias)
+    go through the kernel that moves eight pairs per load and store: bitwise what the same rows
+    give in calls of 100, which take the element-wise kernel; with a partial rotary width,
+    without rotation, and for a layer that stores no keys."""
+    from sonicboom_amd import ops
+    n = 700
+    qkv = randn(n, (hq + 2 * hkv) * hd, dtype=in_dtype).to(DEV)
+    pos = (torch.arange(n, dtype=torch.int32) * 3 % 701).to(DEV)
+    seq = torch.zeros(n, dtype=torch.int32, device=DEV)
+    table = torch.tensor([[4, 9, 1, 7, 3, 10, 0, 6, 2, 8, 5]], dtype=torch.int32, device=DEV)
+    dims = rot or hd
+    inv = torch.exp(-2.0 * torch.arange(dims // 2, dtype=F32) / dims * math.log(1e6)).to(DEV) if rotate else None
+    results = []
+    for step in (n, 100):
+        kc, vc = make_cache(11, max(hkv, 1), hd, BF16, fill=0.0)
+        qs = [ops.rope_kv_store(qkv[r0:r0 + step], BF16, inv, None, dims, pos[r0:r0 + step], seq[r0:r0 + step], kc, vc,
+                                table, hq, hkv, hd) for r0 in range(0, n, step)]
+        results.append((torch.cat(qs), kc, vc))
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    if rotate:
+        want_q = plain.rope_neox(qkv.float().cpu()[:, :hq * hd].numpy(), pos.cpu().numpy(), hd, 1e6, rot, None)
+        close(results[0][0], want_q, atol=2e-2, rtol=8e-3, what="q of the long prompt")
+    else:
+        assert torch.equal(results[0][0], qkv[:, :hq * hd].to(BF16))
+
+
 def test_rope_reference_vectors():
     """/root/reference/tests/core/test_nn.cpp:221-290: position 0 is the identity; with
     head size 2 and an angle of pi/2, [1,0] turns into [0,1]; pairs are (i, i+half)."""
