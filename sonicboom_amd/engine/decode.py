@@ -22,7 +22,7 @@ import numpy as np
 import torch
 
 from .. import ops
-from ..cache.paged import CacheError
+from ..cache.paged import CacheError, pages_for
 from .step import StepError
 
 WIDTH_STEP = 16      # page-table widths are rounded up to this many pages (1024 tokens)
@@ -71,7 +71,7 @@ class _StaticContext:
         v = [self.dev[offs[i]:offs[i + 1]] for i in range(len(sizes))]
         (self.ids, self.row_pos, self.row_seq, self.cu_rows, self.len_before, self.slots, self.want_rows,
          flat_tiles) = v[:8]
-        self.tiles = flat_tiles.view(-1, 4)
+        self._tiles = flat_tiles.view(-1, 4)       # one row a sequence: the same for every height
         self._tables = [t.view(batch, width) for t in v[8:]]
         # the parts that never change for a decode step of this batch size
         ar = np.arange(batch, dtype=np.int32)
@@ -84,6 +84,9 @@ class _StaticContext:
 
     def page_table(self, group: int) -> torch.Tensor:
         return self._tables[group]
+
+    def row_tiles(self, height: int) -> torch.Tensor:
+        return self._tiles
 
     def refresh(self, cache, slots: Sequence[int], tokens: Sequence[int]) -> None:
         """This step's ids, positions and page tables, in one copy to the device.  Fewer
@@ -145,7 +148,7 @@ class DecodeLoop:
 
     def _key(self) -> Tuple[int, int]:
         cache = self.engine.cache
-        need = max((cache.length(s) + 1 + 63) // 64 for s in self.slots)
+        need = max(pages_for(cache.length(s) + 1) for s in self.slots)
         batch = batch_bucket(len(self.slots)) if self.pad_batches else len(self.slots)
         return batch, ((need + WIDTH_STEP - 1) // WIDTH_STEP) * WIDTH_STEP
 

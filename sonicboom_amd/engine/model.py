@@ -56,6 +56,9 @@ class DecoderModel:
         for b in self.blocks:
             if hasattr(b.mixer, "finish_build"):
                 b.mixer.finish_build()
+        # heights of the runs of rows that the mixers' kernels take together (a mixer says so with
+        # a row_tile attribute); a step's context describes its rows in runs of each of them
+        self.row_tiles = sorted({int(b.mixer.row_tile) for b in self.blocks if getattr(b.mixer, "row_tile", 0)})
         # What every cache entry stores, and which order entries want per-sequence state.
         self.cache_specs: Dict[int, tuple] = {}
         self.state_specs: Dict[int, tuple] = {}

@@ -20,7 +20,6 @@ from ..cache.paged import CacheError, PagedCache
 from .model import DecoderModel
 
 
-ROW_TILE = 16      # rows of one sequence that the attention kernels take together
 # Rows that run as one batch.  More than this and a step runs in portions: the tiled products
 # are at their best rate from a few thousand rows on, and their operands (rows x inner width,
 # two bytes each) must stay below 4 GiB.
@@ -68,15 +67,16 @@ class StepContext:
     positions, ``row_seq`` [rows] index of the row's sequence in the batch,
     ``cu_rows`` [seqs+1] first row of every sequence, ``len_before`` [seqs]
     cached length before the step, ``slots`` [seqs] (rows of the state
-    tensors), ``want_rows`` [wanted], ``tiles`` [n, 4] (first row, rows <= 16,
-    sequence, 0: runs of consecutive rows of one sequence);
+    tensors), ``want_rows`` [wanted]; ``row_tiles(h)`` [n, 4] (first row, rows <= h,
+    sequence, 0: runs of consecutive rows of one sequence, for every height ``h`` that a
+    mixer of the model has asked for with its ``row_tile`` attribute);
     ``page_table(group)`` [seqs, pages].
     Host: ``n_rows``, ``n_seqs``, ``n_new`` list, ``lengths_before`` list,
     ``is_decode`` (every sequence brings one token), ``max_new``,
     ``max_len_after``.
     """
 
-    def __init__(self, cache: PagedCache, entries: Sequence[StepEntry], device):
+    def __init__(self, cache: PagedCache, entries: Sequence[StepEntry], device, row_tiles: Sequence[int] = ()):
         self.n_seqs = len(entries)
         self.n_new = [len(e.tokens) for e in entries]
         self.slot_list = [e.slot for e in entries]
@@ -94,12 +94,14 @@ class StepContext:
         want = [int(cu[i]) + int(w) for i, e in enumerate(entries) for w in e.want]
         self.n_wanted = len(want)
         tables = [cache.page_table(g, self.slot_list) for g in range(len(cache.groups))]
-        # runs of up to 16 consecutive rows of one sequence: (first row, rows, sequence, 0)
-        tiles = np.asarray([(int(cu[i]) + r0, min(ROW_TILE, n - r0), i, 0)
-                            for i, n in enumerate(self.n_new) for r0 in range(0, n, ROW_TILE)], dtype=np.int32)
+        # runs of up to h consecutive rows of one sequence: (first row, rows, sequence, 0)
+        heights = sorted({int(h) for h in row_tiles})
+        tiles = [np.asarray([(int(cu[i]) + r0, min(h, n - r0), i, 0)
+                             for i, n in enumerate(self.n_new) for r0 in range(0, n, h)], dtype=np.int32)
+                 for h in heights]
         parts = [ids, row_pos, row_seq, cu, np.asarray(self.lengths_before, dtype=np.int32),
-                 np.asarray(self.slot_list, dtype=np.int32), np.asarray(want, dtype=np.int32),
-                 tiles.reshape(-1)]
+                 np.asarray(self.slot_list, dtype=np.int32), np.asarray(want, dtype=np.int32)]
+        parts += [t.reshape(-1) for t in tiles]
         parts += [t.reshape(-1) for t in tables]
         sizes = [p.size for p in parts]
         # One pinned staging buffer, one copy to the device, views into it.
@@ -112,14 +114,22 @@ class StepContext:
             views.append(dev[off:off + n])
             off += n
         (self.ids, self.row_pos, self.row_seq, self.cu_rows, self.len_before, self.slots,
-         self.want_rows, flat_tiles) = views[:8]
-        self.tiles = flat_tiles.view(-1, 4)
-        self._tables = [v.view(t.shape) for v, t in zip(views[8:], tables)]
+         self.want_rows) = views[:7]
+        self._tiles = {h: v.view(-1, 4) for h, v in zip(heights, views[7:7 + len(heights)])}
+        self._tables = [v.view(t.shape) for v, t in zip(views[7 + len(heights):], tables)]
         self.host_row_pos = row_pos
         self.trace = None            # set by the engine while a tracer listens
 
     def page_table(self, group: int) -> torch.Tensor:
         return self._tables[group]
+
+    def row_tiles(self, height: int) -> torch.Tensor:
+        """The step's rows in runs of up to ``height`` consecutive rows of one sequence."""
+        try:
+            return self._tiles[int(height)]
+        except KeyError:
+            raise StepError(f"no mixer of the model has asked for row tiles of {height} rows "
+                            f"(a mixer asks with its row_tile attribute; asked for: {sorted(self._tiles)})") from None
 
 
 class Engine:
@@ -203,7 +213,7 @@ class Engine:
             raise StepError(str(e)) from None
         portions = portion_rows(n_new, self.max_step_rows)
         if len(portions) == 1:
-            ctx = StepContext(self.cache, entries, self.device)
+            ctx = StepContext(self.cache, entries, self.device, self.model.row_tiles)
             logits = self.forward(ctx)
             self.cache.advance(slots, n_new)
             return logits
@@ -215,7 +225,7 @@ class Engine:
                 picked = [(k, w - a) for k, w in enumerate(e.want) if a <= w < b]
                 sub.append(StepEntry(e.slot, e.tokens[a:b], [w for _, w in picked]))
                 place += [(i, k) for k, _ in picked]
-            ctx = StepContext(self.cache, sub, self.device)
+            ctx = StepContext(self.cache, sub, self.device, self.model.row_tiles)
             pieces.append(self.forward(ctx))
             self.cache.advance([e.slot for e in sub], [len(e.tokens) for e in sub])
         logits = torch.cat(pieces, dim=0)

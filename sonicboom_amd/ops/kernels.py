@@ -650,6 +650,12 @@ def attention_prefill_mfma(q, k_cache, v_cache, page_table, row_pos, tiles, head
     return out
 
 
+# rows of one sequence that a block of the prefill attention kernels takes together; a mixer that
+# calls attention() carries it as its row_tile attribute, so that a step describes its rows in
+# runs of this height
+ATTENTION_ROW_TILE = 16
+
+
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor, ctx,
               heads_q: int, heads_kv: int, head_dim: int, scale: float, window: int,
               fast: bool = True) -> torch.Tensor:
@@ -660,7 +666,8 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, pag
         if ctx.is_decode:
             return attention_decode_mfma(q, k_cache, v_cache, page_table, ctx.row_pos, heads_q, heads_kv,
                                          head_dim, scale, window)
-        return attention_prefill_mfma(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.tiles, heads_q, heads_kv,
+        return attention_prefill_mfma(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_tiles(ATTENTION_ROW_TILE),
+                                      heads_q, heads_kv,
                                       head_dim, scale, window)
     return attention_plain(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_seq, heads_q, heads_kv,
                            head_dim, scale, window)

@@ -52,6 +52,9 @@ def attention_spec(prefix: str, width: int, heads_q: int, heads_kv: int, head_di
 
 @register_part("mixer", "attention")
 class Attention(Mixer):
+    # a step's context lists its rows in runs of this many for the mixer's prefill kernel
+    row_tile = ops.ATTENTION_ROW_TILE
+
     def __init__(self, spec, tensors, parts, rt):
         super().__init__(spec, tensors, parts, rt)
         p = spec.params
