@@ -7,7 +7,9 @@ per-sequence state of fixed size.
 * Cache entries (one per mixer that stores keys) with the same needs
   (kv heads, head size, window) form a **group** with storage and a page pool
   of its own: ``K: [entries, pages, kv_heads, PAGE, head_dim]`` and ``V`` with
-  the last two axes swapped.  A group
+  the last two axes swapped.  A mixer may keep something else per token instead:
+  rows of a shape of its own, ``[entries, pages, PAGE, *shape]``, in groups by
+  (shape, window).  A group
   that only reads a window of keys gives pages back as the window leaves them.
 * ``max_tokens`` sizes every pool: the most tokens live sequences hold at any
   time, each sequence's count rounded up to a whole page (PAGE = 64 tokens).
@@ -71,6 +73,7 @@ class GroupSpec:
     head_dim: int
     window: int                  # 0: every key is kept
     entries: Tuple[int, ...]     # cache entry numbers stored in this group
+    row_shape: Tuple[int, ...] = ()   # not empty: a row of this shape per token instead of keys and values
 
 
 @dataclass
@@ -104,8 +107,12 @@ class PagedCache:
         if allocate:
             import torch
             for spec in self.groups:
-                # keys [.., position, d]; values transposed [.., d, position] (see csrc/sb_hip.h)
                 n = len(spec.entries)
+                if spec.row_shape:
+                    self.k.append(torch.zeros((n, self.n_pages, PAGE, *spec.row_shape), dtype=dtype, device=device))
+                    self.v.append(None)
+                    continue
+                # keys [.., position, d]; values transposed [.., d, position] (see csrc/sb_hip.h)
                 self.k.append(torch.zeros((n, self.n_pages, spec.kv_heads, PAGE, spec.head_dim),
                                           dtype=dtype, device=device))
                 self.v.append(torch.zeros((n, self.n_pages, spec.kv_heads, spec.head_dim, PAGE),
@@ -204,14 +211,16 @@ class PagedCache:
     # ---- storage -------------------------------------------------------------
     def entry_views(self, entry: int):
         """(keys [pages, kv_heads, PAGE, head_dim], values [pages, kv_heads, head_dim, PAGE]) of one
-        cache entry, and its group."""
+        cache entry, and its group; for an entry of a group of rows (rows [pages, PAGE, *shape], None)."""
         g, i = self.entry_place[entry]
-        return self.k[g][i], self.v[g][i], g
+        return self.k[g][i], (None if self.v[g] is None else self.v[g][i]), g
 
 
-def group_entries(specs: Dict[int, Tuple[int, int, int]]) -> List[GroupSpec]:
-    """Group cache entries {entry: (kv_heads, head_dim, window)} by equal needs, in order of first use."""
-    by_need: Dict[Tuple[int, int, int], List[int]] = {}
+def group_entries(specs: Dict[int, tuple]) -> List[GroupSpec]:
+    """Group cache entries {entry: (kv_heads, head_dim, window)}, or {entry: ("rows", shape, window)}
+    for entries that keep a row of their own shape per token, by equal needs, in order of first use."""
+    by_need: Dict[tuple, List[int]] = {}
     for e in sorted(specs):
         by_need.setdefault(tuple(specs[e]), []).append(e)
-    return [GroupSpec(k[0], k[1], k[2], tuple(v)) for k, v in by_need.items()]
+    return [GroupSpec(0, 0, k[2], tuple(v), tuple(k[1])) if k[0] == "rows" else GroupSpec(k[0], k[1], k[2], tuple(v))
+            for k, v in by_need.items()]

@@ -68,11 +68,11 @@ class DecoderModel:
                 cs = mixer.cache_spec()
                 if cs is None:
                     raise ValueError(f"order entry {i} names cache {e.cache} but its mixer keeps no keys")
-                need = (cs.kv_heads, cs.head_dim, cs.window)
+                need = cs.key()          # (kv heads, head size, window), or ("rows", shape, window)
                 if e.writes_cache:
                     self.cache_specs[e.cache] = need
                 elif self.cache_specs.get(e.cache, need)[:2] != need[:2]:
-                    raise ValueError(f"order entry {i} reads cache {e.cache} whose heads differ from its own")
+                    raise ValueError(f"order entry {i} reads cache {e.cache} whose heads (or rows) differ from its own")
             ss = mixer.state_spec()
             if ss is not None:
                 self.state_specs[i] = (tuple(ss.shape), ss.dtype)

@@ -14,7 +14,7 @@ copy in the activation type, ``ctx`` the step's
                 and, for encodings that are not rotary, ``apply(qkv, ctx, heads_q,
                 heads_kv, head_dim)`` acting in place on float32 qkv rows;
                 ``score_scale`` multiplies the attention scale.
-* **mixer**     ``cache_spec() -> KVSpec | None``, ``state_spec() -> StateSpec | None``,
+* **mixer**     ``cache_spec() -> KVSpec | RowsSpec | None``, ``state_spec() -> StateSpec | None``,
                 ``forward(h, x, ctx, binding)`` adds the mixer's output into ``x``.
 * **ffn**       ``forward(h, x, ctx)`` adds the feed-forward's output into ``x``.
                 Mixers and feed-forwards may set ``fuses_norm`` (their ``forward`` then
@@ -62,6 +62,22 @@ class KVSpec:
     head_dim: int
     window: int = 0
 
+    def key(self):
+        return (int(self.kv_heads), int(self.head_dim), int(self.window))
+
+
+@dataclass(frozen=True)
+class RowsSpec:
+    """What a mixer keeps per token when that is not keys and values of heads: one row of
+    ``shape`` (a compressed key-value vector, say) in the cache's dtype, paged like keys;
+    ``window`` > 0 when only the last ``window`` rows are read.  The mixer's binding then
+    carries the rows as ``k_cache`` [pages, PAGE, *shape] and no ``v_cache``."""
+    shape: Tuple[int, ...]
+    window: int = 0
+
+    def key(self):
+        return ("rows", tuple(int(n) for n in self.shape), int(self.window))
+
 
 @dataclass(frozen=True)
 class StateSpec:
@@ -82,7 +98,7 @@ class Part:
 class Mixer(Part):
     category = "mixer"
 
-    def cache_spec(self) -> Optional[KVSpec]:
+    def cache_spec(self) -> "Optional[KVSpec | RowsSpec]":
         return None
 
     def state_spec(self) -> Optional[StateSpec]:

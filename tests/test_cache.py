@@ -143,3 +143,19 @@ def test_groups_by_need():
         (2, 16, 0, (0, 1)), (2, 16, 128, (2,)), (4, 16, 0, (3,))]
     with pytest.raises(CacheError, match="two groups"):
         PagedCache([GroupSpec(1, 16, 0, (0,)), GroupSpec(1, 16, 4, (0,))], 64, allocate=False)
+
+
+def test_groups_of_rows_beside_keys_and_values():
+    """Entries that keep a row of their own shape per token form groups by (shape, window), apart
+    from the groups of keys and values; their pages are counted and given back like the others'."""
+    g = group_entries({0: ("rows", (12,), 0), 1: (1, 16, 0), 2: ("rows", (12,), 0), 3: ("rows", (12,), 70),
+                       4: ("rows", (3, 4), 0)})
+    assert [(x.row_shape, x.kv_heads, x.head_dim, x.window, x.entries) for x in g] == [
+        ((12,), 0, 0, 0, (0, 2)), ((), 1, 16, 0, (1,)), ((12,), 0, 0, 70, (3,)), ((3, 4), 0, 0, 0, (4,))]
+    c = PagedCache(g, 64 * 6, allocate=False)
+    s = c.alloc_slot()
+    c.reserve([s], [200])
+    c.advance([s], [200])
+    assert [c.held_pages(i) for i in range(4)] == [4, 4, 2, 4]      # the window of 70 has let two pages go
+    c.free_slot(s)
+    assert [c.held_pages(i) for i in range(4)] == [0, 0, 0, 0]

@@ -192,6 +192,37 @@ def register_toys():
                     x[r] += self.w_out @ s
                 row += n
 
+    from sonicboom_amd.cache import PAGE
+    from sonicboom_amd.parts import RowsSpec
+
+    @register_part("mixer", "toy_latent")
+    class LatentMixer(Mixer):
+        """Keeps one compressed row c_t = W_c h_t per token in the cache (no heads, no values) and
+        adds W_o times the mean of the rows of the last ``window`` tokens (of all, if 0)."""
+
+        def __init__(self, spec, tensors, parts, rt):
+            super().__init__(spec, tensors, parts, rt)
+            self.rank, self.window = int(spec.params["rank"]), int(spec.params["window"])
+            self.w_c, self.w_o = tensors["w_c"].float(), tensors["w_o"].float()
+
+        def cache_spec(self):
+            return RowsSpec((self.rank,), self.window)
+
+        def forward(self, h, x, ctx, binding):
+            rows, table = binding.k_cache, ctx.page_table(binding.group).long()      # [pages, PAGE, rank]
+            assert binding.v_cache is None and tuple(rows.shape[1:]) == (PAGE, self.rank)
+            pos = ctx.row_pos.long()
+            if binding.writes_cache:
+                c = (h.float() @ self.w_c.T).to(rows.dtype)
+                rows[table[ctx.row_seq.long(), pos // PAGE], pos % PAGE] = c
+            row = 0
+            for i, n in enumerate(ctx.n_new):
+                for r in range(row, row + n):
+                    last = int(ctx.host_row_pos[r])
+                    idx = torch.arange(max(0, last - self.window + 1) if self.window else 0, last + 1, device=x.device)
+                    x[r] += self.w_o @ rows[table[i, idx // PAGE], idx % PAGE].float().mean(0)
+                row += n
+
     @register_part("position", "toy_alibi_free_shift")
     class ShiftPosition(Position):
         """Not rotary: adds position * slope to the first element of every query and key head."""
@@ -269,6 +300,9 @@ def toy_spec(cfg):
         if kind == "decay":
             mixer = PartSpec("mixer", "toy_decay", {"decay": layer["decay"], "inner": layer["inner"]}, {
                 "w_in": TensorSpec(p + "w_in", (layer["inner"], w)), "w_out": TensorSpec(p + "w_out", (w, layer["inner"]))})
+        elif kind == "latent":
+            mixer = PartSpec("mixer", "toy_latent", {"rank": layer["rank"], "window": layer.get("window", 0)}, {
+                "w_c": TensorSpec(p + "w_c", (layer["rank"], w)), "w_o": TensorSpec(p + "w_o", (w, layer["rank"]))})
         else:
             if layer.get("position") == "shift":
                 pos = PartSpec("position", "toy_alibi_free_shift", {"slope": layer["slope"]})
@@ -310,6 +344,12 @@ def plain_toy(cfg, w, tokens, margins=None):
             for t in range(n):
                 s = np.float32(layer["decay"]) * s + u[t]
                 out[t] = w[p + "w_out"] @ s
+        elif layer["mixer"] == "latent":
+            if e.get("writes", True):
+                kv[e["cache"]] = P.linear(h, w[p + "w_c"])
+            c, win = kv[e["cache"]].astype(np.float64), layer.get("window", 0)
+            out = np.stack([w[p + "w_o"].astype(np.float64) @ c[max(0, t - win + 1) if win else 0:t + 1].mean(0)
+                            for t in range(n)]).astype(np.float32)
         else:
             hq, hkv, hd = layer["heads"], layer["kv_heads"], layer["head_dim"]
             bias = (lambda nm: w[p + f"attn.{nm}_proj.bias"]) if layer.get("bias", True) else (lambda nm: None)
@@ -370,6 +410,17 @@ TOY_WINDOWS = {
     # the two windowed layers have different needs, so three cache groups exist
     "order": [{"block": 0, "cache": 0}, {"block": 0, "cache": 0, "writes": False}, {"block": 1, "cache": 1},
               {"block": 2, "cache": 2}, {"block": 0, "cache": 3}],
+}
+
+
+TOY_LATENT = {
+    "architectures": ["ToyForCausalLM"], "vocab_size": 110, "width": 40, "eps": 1e-5,
+    "layers": [{"mixer": "latent", "rank": 12, "ff": 48},
+               {"mixer": "attention", "heads": 2, "kv_heads": 1, "head_dim": 16, "ff": 56},
+               {"mixer": "latent", "rank": 20, "window": 70, "ff": 40}],
+    # the first latent layer runs a second time reading the rows of its first run
+    "order": [{"block": 0, "cache": 0}, {"block": 1, "cache": 1}, {"block": 2, "cache": 2},
+              {"block": 0, "cache": 0, "writes": False}],
 }
 
 
@@ -450,6 +501,39 @@ def test_windows_shared_cache_and_a_layer_that_runs_twice(dtype):
     assert held[0] == 5 and held[50] <= 2 and held[70] <= 3
     eng.free_slot(s)
     assert all(eng.cache.held_pages(i) == 0 for i in range(3))
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_toy_mixer_that_caches_rows_of_its_own_shape(dtype):
+    """A mixer that keeps a compressed row per token instead of keys and values of heads, defined
+    above in this file: its `cache_spec` names the row's shape and a window, the cache gives it
+    pages of such rows in groups of their own beside the attention layer's keys and values, a
+    second run of the layer reads the first run's rows, and the windowed group gives pages back."""
+    from sonicboom_amd.engine import StepEntry
+    cfg, ref, model, eng = build_toy(TOY_LATENT, dtype)
+    needs = sorted((g.row_shape, g.kv_heads, g.head_dim, g.window, g.entries) for g in model.groups)
+    assert needs == [((), 1, 16, 0, (1,)), ((12,), 0, 0, 0, (0,)), ((20,), 0, 0, 70, (2,))]
+    rng = np.random.default_rng(5)
+    a, b = ([int(t) for t in rng.integers(0, 110, size=n)] for n in (230, 90))
+    want_a, want_b = plain_toy(cfg, ref, a), plain_toy(cfg, ref, b)
+    sa, sb = eng.alloc_slot(), eng.alloc_slot()
+    out = eng.step([StepEntry(sa, a[:130], range(130)), StepEntry(sb, b[:50], range(50))])
+    close(out[:130], want_a[:130], dtype, "latent a prompt")
+    close(out[130:], want_b[:50], dtype, "latent b prompt")
+    out = eng.step([StepEntry(sa, a[130:200], range(70))])                  # more rows on top of the cache
+    close(out, want_a[130:200], dtype, "latent a, second piece")
+    for i in range(30):
+        out = eng.step([StepEntry(sa, [a[200 + i]], [0]), StepEntry(sb, [b[50 + i]], [0])])
+        close(out[:1], want_a[200 + i:201 + i], dtype, f"latent a token {i}")
+        close(out[1:], want_b[50 + i:51 + i], dtype, f"latent b token {i}")
+    held = {g.row_shape: eng.cache.held_pages(i) for i, g in enumerate(eng.cache.groups)}
+    assert held[(12,)] == 4 + 2 and held[(20,)] <= 3 + 2          # a: 230 tokens, b: 80
+    eng.free_slot(sa)
+    eng.free_slot(sb)
+    assert all(eng.cache.held_pages(i) == 0 for i in range(3))
+    s = eng.alloc_slot()                                          # used pages, used slot
+    close(eng.step([StepEntry(s, b, range(len(b)))]), want_b, dtype, "latent b whole, on a used slot")
+    eng.free_slot(s)
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
