@@ -173,7 +173,10 @@ int sb_gemm_skinny_partial_bf16(float *partial, const void *x, const void *w, in
 int sb_gemm_stream_max_rows(void);                       /* up to 128 rows, waves split the features */
 /* `hint` (0: the launcher chooses; for tests and measurements): bits 0..7 waves per block (4..8),
  * bits 8..15 the K slices the partial form aims at (1..8).  `tile_shape`: -1 the launcher
- * chooses, 0 / 1 / 2 tiles of 128 x 128, 256 x 128, 256 x 256 outputs. */
+ * chooses; else bits 0..3 the tile, 0 / 1 / 2 / 3 for 128 x 128, 256 x 128, 256 x 256, 128 x 256
+ * outputs, and bits 4..5 the kernel: 0 the launcher's choice, 1 the one that stages tiles
+ * through registers, 2 the one that loads them straight into LDS (packed weights, n_in a multiple
+ * of 64; the only one with the 128 x 256 tile), 3 the same with a block for every tile. */
 int sb_gemm_stream_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,
                         int bias_dtype, const float *resid, int n_rows, int n_out, int n_in, int gated,
                         int hint, void *stream);
