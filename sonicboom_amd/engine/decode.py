@@ -16,6 +16,7 @@ position, replay the captured step, read the token).
 """
 from __future__ import annotations
 
+import gc
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
@@ -194,11 +195,22 @@ class DecodeLoop:
         """Record the launches of a step of this shape.  Capture runs nothing; replays read the
         ids, positions and page tables that ``refresh`` puts into the fixed buffers."""
         torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            logits = self.engine.forward(ctx)
-            if choose:
-                ops.argmax(logits, out=ctx.next_ids)
+        # Python's collector must not run inside the capture: what it finalizes (the pinned
+        # buffers of earlier steps' contexts, graphs of loops long gone, anything that waited in
+        # a reference cycle) calls into the HIP runtime, which refuses such calls on a capturing
+        # stream, and the process aborts.  So it runs now, and not again until the capture ends.
+        gc.collect()
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                logits = self.engine.forward(ctx)
+                if choose:
+                    ops.argmax(logits, out=ctx.next_ids)
+        finally:
+            if collecting:
+                gc.enable()
         while len(self._graphs) >= MAX_GRAPHS:
             oldest = next(iter(self._graphs))
             del self._graphs[oldest]            # its memory pool goes with it

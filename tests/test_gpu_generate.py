@@ -136,6 +136,32 @@ def test_graph_replay_gives_the_same_tokens(model_folders):
     assert s == without.generate(prompts, temperature=0.7, seed=3, max_tokens=40, stop_tokens=())
 
 
+def test_the_collector_stays_out_of_graph_captures(model_folders):
+    """While a decode step is being recorded Python's garbage collector is switched off (what it
+    finalizes may call into the HIP runtime, which a capturing stream refuses), and it has run
+    just before; afterwards it is on again."""
+    import gc
+    import torch
+    folder = model_folders["A"]
+    session = model_for(folder, "bfloat16").session(max_tokens=64 * 4)
+    eng = session.engine
+    seen = []
+    forward = eng.forward
+
+    def watched(ctx):
+        if torch.cuda.is_current_stream_capturing():
+            seen.append(gc.isenabled())
+        return forward(ctx)
+    eng.forward = watched
+    try:
+        assert gc.isenabled()
+        session.generate(prompts_for("A", [5, 11], seed=2), max_tokens=8, stop_tokens=())
+    finally:
+        eng.forward = forward
+    assert seen and not any(seen)            # at least one step was recorded, none with the collector on
+    assert gc.isenabled()
+
+
 def test_batches_run_in_buckets_with_rows_that_do_nothing(model_folders):
     """The decode loop runs a batch of more than eight sequences at the next bucket's size (12,
     16, 24, ...): the rows it adds have no pages, store nothing and see no key.  A batch of 21
