@@ -190,10 +190,11 @@ def kernel_rates(m, totals, rows, kv_tokens, prefill_lengths=None):
                 item["frac"] = round(item["GB/s"] / PEAK_HBM_GBS, 3)
         else:
             if label in weights:
-                item["TFLOP/s"] = round(2 * rows * weights[label] * calls / us / 1e6, 1)
+                # per layer, not per call: a long prompt runs in portions, several calls a layer
+                item["TFLOP/s"] = round(2 * rows * weights[label] * L / us / 1e6, 1)
             elif label == "attention":
                 flops = sum(4 * (n * (n + 1) // 2) * m["hq"] * m["hd"] for n in prefill_lengths)
-                item["TFLOP/s"] = round(flops * calls / us / 1e6, 1)
+                item["TFLOP/s"] = round(flops * L / us / 1e6, 1)
             if "TFLOP/s" in item:
                 item["frac"] = round(item["TFLOP/s"] * 1e12 / PEAK_FLOPS["bf16"], 3)
         out[label] = item
