@@ -187,8 +187,7 @@ __device__ __forceinline__ void attend_half(WaveState<NC> &st, const bf16x8_t (&
       sc[e] = vis ? v : -__builtin_inff();
       mx = fmaxf(mx, sc[e]);
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx = max_over_lane_groups(mx);
     const float m_new = fmaxf(st.m[c], mx);
     // a column that has seen no key yet keeps m = -inf: give it a finite stand-in
     const float m_use = m_new == -__builtin_inff() ? 0.f : m_new;
@@ -373,8 +372,7 @@ __device__ __forceinline__ void attend_page64(WaveState<NC> &st, const bf16x8_t 
         sc[8 * h + e] = v;
         mx = fmaxf(mx, v);
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx = max_over_lane_groups(mx);
     mx *= scale_log2;                                              // the scale is positive
     const float m_old = st.m[c];
     const bool move = mx > m_old + kMaxSlack;                      // also the first key of a column
@@ -399,13 +397,23 @@ __device__ __forceinline__ void attend_page64(WaveState<NC> &st, const bf16x8_t 
   }
   // the old sums shrink by alpha; once the maxima have settled no column of the wave moves
   if (__any(rescale)) {
+    // (two waves a SIMD: in place, so that the sums stay in their registers on the way that does not
+    // come through here; a wave that has its SIMD to itself has registers to spare, and tying them
+    // made its two-head form spill)
 #pragma unroll
     for (int c = 0; c < NC; ++c)
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        st.o[c][dt][0] *= alpha[c]; st.o[c][dt][1] *= alpha[c];
-        st.o[c][dt][2] *= alpha[c]; st.o[c][dt][3] *= alpha[c];
-      }
+      for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (PIN) {
+            st.o[c][dt][e] *= alpha[c];
+          } else {
+            float v = st.o[c][dt][e];
+            asm volatile("v_mul_f32 %0, %0, %1" : "+v"(v) : "v"(alpha[c]));
+            st.o[c][dt][e] = v;
+          }
+        }
   }
   if (PIN) __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -1437,11 +1445,18 @@ extern "C" int sb_attn_prefill_bf16(void *out, const void *q, const void *k_cach
         max_pages, n_pages_total, row_pos, tiles, n_tiles, heads_q, heads_kv, head_tiles, y_per_kv,      \
         scale * kLog2e, window);                                                                         \
   } while (0)
-  if (waves == 8) SB_GO(1, 8);
-  else if (nc == 4) SB_GO(4, 4);
-  else if (nc == 3) SB_GO(3, 4);
-  else if (nc == 2) SB_GO(2, 4);
-  else SB_GO(1, 4);
+  // (forms that nc_max rules out for this head size are not compiled)
+  if (waves == 8) {
+    if constexpr (HD <= 128) SB_GO(1, 8);
+  } else if (nc == 4) {
+    if constexpr (DT <= 4) SB_GO(4, 4);
+  } else if (nc == 3) {
+    if constexpr (DT <= 4) SB_GO(3, 4);
+  } else if (nc == 2) {
+    if constexpr (DT <= 12) SB_GO(2, 4);
+  } else {
+    SB_GO(1, 4);
+  }
 #undef SB_GO
   return sb::check_launch("sb_attn_prefill_bf16");
 }

@@ -36,3 +36,20 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
   const bf16x2_t v = {(__bf16)lo, (__bf16)hi};
   return __builtin_bit_cast(uint32_t, v);
 }
+
+// The maximum over the four lanes l % 16, l % 16 + 16, + 32, + 48 (the four lane groups that hold
+// one column of an MFMA result), in every one of them.  Two lane swaps inside the vector unit
+// (v_permlane32_swap, v_permlane16_swap: halves of the wave, then odd against even rows of 16)
+// where a shuffle would go through LDS and make the wave wait for everything it has asked of it.
+// Both operands of a swap are the same value, and the halves it returns are taken apart into
+// variables first: written as max(p[0], p[1]) the compiler drops the maximum.
+__device__ __forceinline__ float max_over_lane_groups(float v) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const auto p = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const uint32_t p0 = p[0], p1 = p[1];
+  const float a = fmaxf(__builtin_bit_cast(float, p0), __builtin_bit_cast(float, p1));
+  const uint32_t ua = __builtin_bit_cast(uint32_t, a);
+  const auto q = __builtin_amdgcn_permlane16_swap(ua, ua, false, false);
+  const uint32_t q0 = q[0], q1 = q[1];
+  return fmaxf(__builtin_bit_cast(float, q0), __builtin_bit_cast(float, q1));
+}
