@@ -265,6 +265,107 @@ top_candidates_kernel(int32_t *__restrict__ cand_id, float *__restrict__ cand_z,
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// The filters and the draw over a row's candidates (/root/reference/core/src/nn/sampling.cpp:157-203,
+// :287-312): window of 30 below the best z, top-k, min-p, the shortest prefix whose probability
+// reaches top_p (running sums in float64, in order), then Gumbel-max: the candidate with the
+// largest z + g, g = -ln(-ln u), u = (w + 0.5) / 2^32 for word 0 of Philox4x32-10 of counter
+// (position low, position high, id, 0) under the 64-bit seed; ties to the lower id.  One wave
+// per row; the candidates are ordered (z descending, id ascending), so what every filter keeps
+// is a prefix and a count stands for it.
+__device__ __forceinline__ uint32_t philox_word0(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint64_t key) {
+  uint32_t k0 = uint32_t(key), k1 = uint32_t(key >> 32);
+#pragma unroll
+  for (int round = 0; round < 10; ++round) {
+    const uint64_t p0 = uint64_t(0xD2511F53u) * c0, p1 = uint64_t(0xCD9E8D57u) * c2;
+    const uint32_t n0 = uint32_t(p1 >> 32) ^ c1 ^ k0, n1 = uint32_t(p1), n2 = uint32_t(p0 >> 32) ^ c3 ^ k1,
+                   n3 = uint32_t(p0);
+    c0 = n0, c1 = n1, c2 = n2, c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  return c0;
+}
+
+constexpr int kDrawPerLane = kMaxCand / 64;
+
+__global__ void __launch_bounds__(64)
+draw_kernel(int32_t *__restrict__ token, const int32_t *__restrict__ cand_id, const float *__restrict__ cand_z,
+            const int64_t *__restrict__ position, int k, int top_k, int use_min_p, float log_min_p,
+            int use_top_p, double top_p, uint64_t seed) {
+  __shared__ double e_of[kMaxCand];
+  __shared__ int n_keep_sh;
+  const int row = blockIdx.x, lane = threadIdx.x;
+  const int32_t *ids = cand_id + size_t(row) * k;
+  const float *zs = cand_z + size_t(row) * k;
+  const float m = zs[0];
+  const float floor_z = m - 30.0f;
+  const float cutoff = m + log_min_p;
+  float z[kDrawPerLane];
+  int id[kDrawPerLane];
+  int keep = 0;            // candidates inside the window, then after top-k and min-p: a prefix
+#pragma unroll
+  for (int j = 0; j < kDrawPerLane; ++j) {
+    const int c = lane + 64 * j;
+    z[j] = c < k ? zs[c] : -__builtin_inff();
+    id[j] = c < k ? ids[c] : -1;
+    keep += int(__popcll(__ballot(c < k && id[j] >= 0 && z[j] >= floor_z)));
+  }
+  if (top_k > 0) keep = min(keep, top_k);
+  if (use_min_p) {
+    int kept = 0;
+#pragma unroll
+    for (int j = 0; j < kDrawPerLane; ++j) kept += int(__popcll(__ballot(lane + 64 * j < keep && !(z[j] < cutoff))));
+    keep = kept;
+  }
+  if (use_top_p && keep > 0) {
+#pragma unroll
+    for (int j = 0; j < kDrawPerLane; ++j) {
+      const int c = lane + 64 * j;
+      if (c < keep) e_of[c] = exp(double(z[j]) - double(m));
+    }
+    __syncthreads();
+    if (lane == 0) {
+      double total = 0.0;
+      for (int c = 0; c < keep; ++c) total += e_of[c];
+      int n = keep;
+      if (total > 0.0) {
+        double acc = 0.0;
+        for (int c = 0; c < keep; ++c) {
+          acc += e_of[c];
+          if (acc / total >= top_p) {
+            n = c + 1;
+            break;
+          }
+        }
+      }
+      n_keep_sh = n;
+    }
+    __syncthreads();
+    keep = n_keep_sh;
+  }
+  double best = -__builtin_inf();
+  int best_id = 0x7fffffff;
+  const uint64_t pos = uint64_t(position[row]);
+#pragma unroll
+  for (int j = 0; j < kDrawPerLane; ++j) {
+    const int c = lane + 64 * j;
+    if (c >= keep) continue;
+    const uint32_t w = philox_word0(uint32_t(pos), uint32_t(pos >> 32), uint32_t(id[j]), 0u, seed);
+    const double u = (double(w) + 0.5) / 4294967296.0;
+    const double score = double(z[j]) - log(-log(u));
+    if (score > best || (score == best && id[j] < best_id)) best = score, best_id = id[j];
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const double other = __shfl_xor(best, off, 64);
+    const int other_id = __shfl_xor(best_id, off, 64);
+    if (other > best || (other == best && other_id < best_id)) best = other, best_id = other_id;
+  }
+  if (lane == 0) token[row] = keep > 0 ? best_id : -1;
+}
+
 }  // namespace
 
 // Parts a row is cut into for the first stage (the second size of the partial buffers).
@@ -412,4 +513,20 @@ extern "C" int sb_top_candidates(int32_t *cand_id, float *cand_z, const float *l
   top_candidates_kernel<true><<<n_rows, kSelThreads, 0, s>>>(cand_id, cand_z, logits, scratch, parts * kMaxCand,
                                                              vocab, k, temperature);
   return sb::check_launch("sb_top_candidates");
+}
+
+// One token per row from its candidates (what sb_top_candidates wrote: k <= 256 per row, ordered
+// (z descending, id ascending), id -1 past a short row's end): window, top-k (0: off), min-p
+// (log_min_p = ln of it as a float; use_min_p 0: off), top-p (use_top_p 0: off), Gumbel-max under
+// (seed, position[row], id).  token int32 [n_rows]: -1 for a row that keeps no candidate.
+extern "C" int sb_draw(int32_t *token, const int32_t *cand_id, const float *cand_z, const int64_t *position,
+                       int n_rows, int k, int top_k, int use_min_p, float log_min_p, int use_top_p, double top_p,
+                       uint64_t seed, void *stream) {
+  SB_REQUIRE(token && cand_id && cand_z && position, "sb_draw: null pointer");
+  SB_REQUIRE(n_rows >= 0 && top_k >= 0, "sb_draw: bad sizes rows=%d top_k=%d", n_rows, top_k);
+  SB_SUPPORT(k >= 1 && k <= kMaxCand, "sb_draw: %d candidates a row, at most %d", k, kMaxCand);
+  if (n_rows == 0) return SB_OK;
+  draw_kernel<<<n_rows, 64, 0, (hipStream_t)stream>>>(token, cand_id, cand_z, position, k, top_k, use_min_p,
+                                                      log_min_p, use_top_p, top_p, seed);
+  return sb::check_launch("sb_draw");
 }

@@ -152,6 +152,17 @@ size_t sb_top_candidates_scratch(int n_rows, int vocab);
 int sb_top_candidates(int32_t *cand_id, float *cand_z, const float *logits, int n_rows, int vocab,
                       int k, float temperature, uint64_t *scratch, void *stream);
 
+/* One token per row from its candidates as sb_top_candidates wrote them (k <= 256
+ * per row): the window of 30 below the best z, top-k (0: off), min-p
+ * (log_min_p = ln(min_p) as a float; use_min_p 0: off), top-p (use_top_p 0: off;
+ * running sums in float64, in order) and the Gumbel-max draw with word 0 of
+ * Philox4x32-10 of counter (position, id, 0) under `seed`; ties to the lower id.
+ * position int64 [n_rows]: the absolute position of each row's new token.
+ * token int32 [n_rows]: -1 for a row that keeps no candidate. */
+int sb_draw(int32_t *token, const int32_t *cand_id, const float *cand_z, const int64_t *position,
+            int n_rows, int k, int top_k, int use_min_p, float log_min_p, int use_top_p, double top_p,
+            uint64_t seed, void *stream);
+
 /* ---- bf16 products on the matrix cores ----------------------------------
  * X bf16 [n_rows, n_in] row-major, n_in a multiple of 8, operands 16-byte
  * aligned.  W bf16 [n_out, n_in] row-major, or (packed != 0, or always for the

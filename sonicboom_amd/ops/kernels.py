@@ -304,6 +304,31 @@ def top_candidates(logits: torch.Tensor, temperature: float, k: int = MAX_CANDID
     return ids, z
 
 
+def draw(cand_ids: torch.Tensor, cand_z: torch.Tensor, positions, top_k: int, log_min_p: Optional[float],
+         top_p: Optional[float], seed: int) -> torch.Tensor:
+    """One token per row (int32 [n]; -1 where no candidate is kept) from the candidates that
+    :func:`top_candidates` wrote: the window of 30 below the best z, top-k (0: off), min-p
+    (``log_min_p`` = ln(min_p) rounded to float32, None: off), top-p (a float64, None: off) and
+    the Gumbel-max draw under (seed, position of the row's new token, candidate id).
+    ``positions``: one absolute position per row, a sequence or an int64 tensor on the device."""
+    _dev(cand_ids, cand_z)
+    if cand_ids.dtype != torch.int32 or cand_z.dtype != torch.float32 or cand_ids.dim() != 2 \
+            or tuple(cand_ids.shape) != tuple(cand_z.shape):
+        raise KernelLibraryError("candidates must be int32 ids and float32 z of one shape [rows, k]")
+    n, k = cand_ids.shape
+    if not torch.is_tensor(positions):
+        positions = torch.tensor([int(q) for q in positions], dtype=torch.int64).to(cand_ids.device)
+    _dev(positions)
+    if positions.dtype != torch.int64 or positions.numel() != n:
+        raise KernelLibraryError("positions must be int64, one per row")
+    out = torch.empty((n,), dtype=torch.int32, device=cand_ids.device)
+    check(library.core().sb_draw(_p(out), _p(cand_ids.contiguous()), _p(cand_z.contiguous()), _p(positions.contiguous()),
+                                 n, k, int(top_k), 0 if log_min_p is None else 1,
+                                 0.0 if log_min_p is None else float(log_min_p), 0 if top_p is None else 1,
+                                 0.0 if top_p is None else float(top_p), int(seed) & 0xFFFFFFFFFFFFFFFF, _stream()))
+    return out
+
+
 def read_bandwidth(n_bytes: int = 1 << 30, blocks: int = 512, repeats: int = 5, device="cuda:0") -> float:
     """Bytes a second that a plain streaming read of ``n_bytes`` reaches on this GPU (the best of
     ``repeats`` passes over a buffer that the caches do not hold): what "achievable" means beside

@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 import threading
-from ctypes import c_char_p, c_float, c_int, c_size_t, c_void_p
+from ctypes import c_char_p, c_double, c_float, c_int, c_size_t, c_uint64, c_void_p
 
 from ..csrc import build
 
@@ -34,6 +34,7 @@ _CORE_SIGNATURES = {
     "sb_argmax_parts": [_I],
     "sb_penalize": [_P, _I, _P, _P, _P, _I, _F, _F, _F, _I, _P],
     "sb_top_candidates": [_P, _P, _P, _I, _I, _I, _F, _P, _P],
+    "sb_draw": [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I, c_double, c_uint64, _P],
 }
 # Entry points of later kernels; declared when the library has them.
 _OPTIONAL_SIGNATURES = {

@@ -6,10 +6,14 @@ last ``repeat_last_n`` tokens of the history, then either the argmax
 (temperature 0, ties to the lowest id) or: the 256 best candidates by
 z = logit / temperature, a window of 30 below the best, top-k, min-p, top-p,
 and a Gumbel-max draw with a Philox4x32-10 word keyed by (seed, position of
-the token being produced, candidate id).  Penalties, argmax and the candidate
-selection run on the device over the whole batch; the filters and the draw
-work on 256 numbers per sequence and run on the host in float64 (all rows of a
-step in one pass of array arithmetic), as the reference's do (/root/reference/core/src/nn/sampling.cpp:157-203, :287-312).
+the token being produced, candidate id).  All of it runs on the device over the
+whole batch: penalties, argmax, the candidate selection, and the filters and the
+draw over each row's 256 candidates (a wave a row, the running sums of top-p and
+the Gumbel scores in float64, /root/reference/core/src/nn/sampling.cpp:157-203,
+:287-312); a step's tokens come back in one small copy.  The same filters and draw
+on the host, row by row and for all rows at once in array arithmetic, are
+:func:`filter_candidates`, :func:`gumbel_draw` and :func:`draw_rows`: what the
+tests hold the device kernel to, beside the plain sampler.
 Every sequence draws from its own (seed, position) stream, so its tokens do
 not depend on what else is in the batch.
 """
@@ -146,4 +150,7 @@ class Sampler:
             return ops.argmax(logits).tolist()
         k = min(CANDIDATES, vocab)
         ids_d, z_d = ops.top_candidates(logits, p.temperature, k)
-        return draw_rows(ids_d.cpu().numpy(), z_d.cpu().numpy(), positions, p)
+        # the cut-offs as the host form rounds them: ln(min_p) in float32, top_p through float32
+        log_min_p = float(np.log(np.float32(p.min_p))) if p.min_p > 0.0 else None
+        top_p = float(np.float64(np.float32(p.top_p))) if 0.0 < p.top_p < 1.0 else None
+        return ops.draw(ids_d, z_d, positions, p.top_k, log_min_p, top_p, p.seed).tolist()

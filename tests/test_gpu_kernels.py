@@ -987,6 +987,53 @@ def test_top_candidates(vocab, temperature):
         assert np.array_equal(np.array([c[1] for c in want], dtype=np.float32), z[r]), f"row {r}"
 
 
+@pytest.mark.parametrize("params", [
+    dict(temperature=0.8), dict(temperature=1.3, top_k=5), dict(temperature=0.5, top_p=0.7),
+    dict(temperature=1.0, min_p=0.2), dict(temperature=0.9, top_k=40, top_p=0.9, min_p=0.01),
+    dict(temperature=0.05, top_p=0.5), dict(temperature=2.0, top_k=1), dict(temperature=1.0, top_p=1e-9, min_p=1.0),
+    dict(temperature=1.0, top_k=300, top_p=0.999),
+])
+@pytest.mark.parametrize("vocab", [40, 400, 5000])
+def test_draw_equals_the_plain_sampler(params, vocab):
+    """Filters and Gumbel draw on the device, a wave a row: every row gets the token that the
+    plain sampler draws for it alone (flat and peaked rows, ties among the best, one candidate far
+    above the window, positions past 2^32, a 64-bit seed, fewer logits than candidates)."""
+    from sonicboom_amd import ops
+    SP = sampling_plain
+    r = np.random.default_rng(vocab)
+    rows = []
+    for i in range(96):
+        logits = (r.standard_normal(vocab) * (0.2 if i % 5 == 0 else 3.0)).astype(np.float32)
+        if i % 7 == 3:
+            logits[10:20] = logits[5]
+        if i % 6 == 1:
+            logits[3] = 80.0
+        rows.append(logits)
+    positions = [int(q) for q in r.integers(0, 5000, size=len(rows))]
+    positions[0], positions[1] = 0, 2 ** 33 + 5
+    seed = 0x9E3779B97F4A7C15
+    t = params["temperature"]
+    k = min(ops.MAX_CANDIDATES, vocab)
+    ids, z = ops.top_candidates(torch.tensor(np.stack(rows), device=DEV), t, k)
+    log_min_p = float(np.log(np.float32(params["min_p"]))) if params.get("min_p", 0.0) > 0.0 else None
+    top_p = float(np.float64(np.float32(params["top_p"]))) if 0.0 < params.get("top_p", 1.0) < 1.0 else None
+    got = ops.draw(ids, z, positions, params.get("top_k", 0), log_min_p, top_p, seed).tolist()
+    for i, logits in enumerate(rows):
+        kept = SP.filter_candidates(SP.select_candidates(logits, t), params.get("top_k", 0),
+                                    params.get("top_p", 1.0), params.get("min_p", 0.0))
+        assert got[i] == SP.draw(kept, seed, positions[i]), f"row {i}"
+
+
+def test_draw_keeps_no_candidate_of_an_empty_row():
+    """A row whose candidates all lie outside (ids of -1, as a row shorter than k is filled)
+    gives -1; its neighbours are not disturbed."""
+    from sonicboom_amd import ops
+    ids = torch.tensor([[3, 1, -1, -1], [-1, -1, -1, -1]], dtype=torch.int32, device=DEV)
+    z = torch.tensor([[2.0, 1.0, 0.0, 0.0], [0.0, 0.0, 0.0, 0.0]], dtype=torch.float32, device=DEV)
+    got = ops.draw(ids, z, [5, 6], 0, None, None, 1).tolist()
+    assert got[0] in (3, 1) and got[1] == -1
+
+
 @pytest.mark.parametrize("exact", [False, True])
 def test_penalize(exact):
     from sonicboom_amd import ops
