@@ -15,10 +15,12 @@
 // /root/reference/core/src/nn/attention.cpp:26-105, activation
 // /root/reference/core/src/nn/activation.cpp:41-50, first maximum
 // /root/reference/core/src/nn/sampling.cpp:238-244.
+#include <algorithm>
 #include <cmath>
 #include <cstddef>
 #include <cstdint>
 #include <limits>
+#include <utility>
 #include <vector>
 
 namespace {
@@ -224,6 +226,109 @@ int sbp_argmax(int32_t *ids, const float *logits, int n_rows, int vocab) {
     for (int i = 1; i < vocab; ++i)
       if (logits[size_t(r) * vocab + i] > logits[size_t(r) * vocab + best]) best = i;
     ids[r] = best;
+  }
+  return 0;
+}
+
+// Sampling penalties in place for (row, token, count) triples
+// (/root/reference/core/src/nn/sampling.cpp:43-70 and, exact, :77-104): v = v > 0 ? v / rp : v * rp when rp != 1,
+// then v -= freq * count + presence; exact: with one rounding where the sampled path has one.
+int sbp_penalize(float *logits, int vocab, const int32_t *item_row, const int32_t *item_token,
+                 const int32_t *item_count, int n_items, float rp, float presence, float freq, int exact) {
+  if (!logits || vocab <= 0 || n_items < 0 || (n_items && (!item_row || !item_token || !item_count))) return 1;
+  for (int it = 0; it < n_items; ++it) {
+    const int tok = item_token[it];
+    if (tok < 0 || tok >= vocab) continue;
+    float &v = logits[size_t(item_row[it]) * vocab + tok];
+    const float c = float(item_count[it]);
+    if (rp != 1.0f) v = v > 0.0f ? v / rp : v * rp;
+    if (exact) {
+      v = std::fma(-1.0f, std::fma(freq, c, presence), v);
+    } else {
+      const float fc = freq * c;
+      const float adjust = fc + presence;
+      v = v - adjust;
+    }
+  }
+  return 0;
+}
+
+// The k best of every row by z = logit / temperature (one float32 division), ordered
+// (z descending, id ascending); id -1 and z 0 past a short row's end
+// (/root/reference/core/src/nn/sampling.cpp:257-285).
+int sbp_top_candidates(int32_t *cand_id, float *cand_z, const float *logits, int n_rows, int vocab, int k,
+                       float temperature) {
+  if (!cand_id || !cand_z || !logits || n_rows < 0 || vocab <= 0 || k < 1 || !(temperature > 0.0f)) return 1;
+  std::vector<std::pair<float, int>> row(static_cast<size_t>(vocab));
+  for (int r = 0; r < n_rows; ++r) {
+    for (int i = 0; i < vocab; ++i) row[i] = {logits[size_t(r) * vocab + i] / temperature + 0.0f, i};
+    std::sort(row.begin(), row.end(), [](const std::pair<float, int> &a, const std::pair<float, int> &b) {
+      return a.first != b.first ? a.first > b.first : a.second < b.second;
+    });
+    for (int i = 0; i < k; ++i) {
+      cand_id[size_t(r) * k + i] = i < vocab ? row[i].second : -1;
+      cand_z[size_t(r) * k + i] = i < vocab ? row[i].first : 0.0f;
+    }
+  }
+  return 0;
+}
+
+namespace {
+uint32_t philox_word0(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint64_t key) {
+  uint32_t k0 = uint32_t(key), k1 = uint32_t(key >> 32);
+  for (int round = 0; round < 10; ++round) {
+    const uint64_t p0 = uint64_t(0xD2511F53u) * c0, p1 = uint64_t(0xCD9E8D57u) * c2;
+    const uint32_t n0 = uint32_t(p1 >> 32) ^ c1 ^ k0, n1 = uint32_t(p1), n2 = uint32_t(p0 >> 32) ^ c3 ^ k1,
+                   n3 = uint32_t(p0);
+    c0 = n0, c1 = n1, c2 = n2, c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  return c0;
+}
+}  // namespace
+
+// One token per row from its ordered candidates: window 30, top-k, min-p, top-p, Gumbel-max
+// (/root/reference/core/src/nn/sampling.cpp:157-203, :287-312); the arguments of sb_draw.
+int sbp_draw(int32_t *token, const int32_t *cand_id, const float *cand_z, const int64_t *position, int n_rows,
+             int k, int top_k, int use_min_p, float log_min_p, int use_top_p, double top_p, uint64_t seed) {
+  if (!token || !cand_id || !cand_z || !position || n_rows < 0 || k < 1 || top_k < 0) return 1;
+  for (int r = 0; r < n_rows; ++r) {
+    const int32_t *id = cand_id + size_t(r) * k;
+    const float *z = cand_z + size_t(r) * k;
+    const float m = z[0], floor_z = m - 30.0f, cutoff = m + log_min_p;
+    int keep = 0;
+    for (int c = 0; c < k; ++c) keep += id[c] >= 0 && z[c] >= floor_z;
+    if (top_k > 0 && keep > top_k) keep = top_k;
+    if (use_min_p) {
+      int kept = 0;
+      for (int c = 0; c < keep; ++c) kept += !(z[c] < cutoff);
+      keep = kept;
+    }
+    if (use_top_p && keep > 0) {
+      double total = 0.0;
+      for (int c = 0; c < keep; ++c) total += std::exp(double(z[c]) - double(m));
+      if (total > 0.0) {
+        double acc = 0.0;
+        for (int c = 0; c < keep; ++c) {
+          acc += std::exp(double(z[c]) - double(m));
+          if (acc / total >= top_p) {
+            keep = c + 1;
+            break;
+          }
+        }
+      }
+    }
+    int best = -1;
+    double best_score = 0.0;
+    const uint64_t pos = uint64_t(position[r]);
+    for (int c = 0; c < keep; ++c) {
+      const uint32_t w = philox_word0(uint32_t(pos), uint32_t(pos >> 32), uint32_t(id[c]), 0u, seed);
+      const double u = (double(w) + 0.5) / 4294967296.0;
+      const double score = double(z[c]) - std::log(-std::log(u));
+      if (best < 0 || score > best_score || (score == best_score && id[c] < best)) best = id[c], best_score = score;
+    }
+    token[r] = best;
   }
   return 0;
 }

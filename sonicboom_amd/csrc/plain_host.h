@@ -30,6 +30,13 @@ int sbp_attention(float *out, const float *q, int q_stride, const float *k_cache
                   const int32_t *row_seq, int n_rows, int heads_q, int heads_kv, int head_dim, float scale,
                   int window);
 int sbp_argmax(int32_t *ids, const float *logits, int n_rows, int vocab);
+int sbp_penalize(float *logits, int vocab, const int32_t *item_row, const int32_t *item_token,
+                 const int32_t *item_count, int n_items, float repeat_penalty, float presence_penalty,
+                 float frequency_penalty, int exact);
+int sbp_top_candidates(int32_t *cand_id, float *cand_z, const float *logits, int n_rows, int vocab, int k,
+                       float temperature);
+int sbp_draw(int32_t *token, const int32_t *cand_id, const float *cand_z, const int64_t *position, int n_rows,
+             int k, int top_k, int use_min_p, float log_min_p, int use_top_p, double top_p, uint64_t seed);
 
 #ifdef __cplusplus
 }

@@ -9,6 +9,7 @@ import pytest
 import torch
 
 from plain import qwen2_plain as P
+from plain import sampling_plain as SP
 
 F32, BF16 = torch.float32, torch.bfloat16
 DEV = "cuda:0"
@@ -18,7 +19,8 @@ def twins():
     from sonicboom_amd.csrc import build
     lib = ctypes.CDLL(build.ensure_plain_host())
     for name in ("sbp_embed", "sbp_rmsnorm", "sbp_reduce_resid_norm", "sbp_gemm", "sbp_silu_mul", "sbp_add_into",
-                 "sbp_rope_kv_store", "sbp_attention", "sbp_argmax"):
+                 "sbp_rope_kv_store", "sbp_attention", "sbp_argmax", "sbp_penalize", "sbp_top_candidates",
+                 "sbp_draw"):
         getattr(lib, name).restype = ctypes.c_int
     return lib
 
@@ -115,6 +117,71 @@ def test_host_twins_agree_with_the_plain_implementation():
     assert lib.sbp_argmax(ptr(ids), ptr(logits), C(3), C(3)) == 0 and ids.tolist() == [0, 1, 0]
 
 
+def host_penalize(lib, logits, rows, toks, counts, rp, pp, fp, exact):
+    out = np.array(logits, np.float32, copy=True)
+    assert lib.sbp_penalize(ptr(out), C(out.shape[1]), ptr(i32(rows)), ptr(i32(toks)), ptr(i32(counts)), C(len(rows)),
+                            ctypes.c_float(rp), ctypes.c_float(pp), ctypes.c_float(fp), C(int(exact))) == 0
+    return out
+
+
+def host_candidates(lib, logits, k, temperature):
+    ids, z = np.empty((logits.shape[0], k), np.int32), np.empty((logits.shape[0], k), np.float32)
+    assert lib.sbp_top_candidates(ptr(ids), ptr(z), ptr(logits), C(logits.shape[0]), C(logits.shape[1]), C(k),
+                                  ctypes.c_float(temperature)) == 0
+    return ids, z
+
+
+def host_draw(lib, ids, z, positions, top_k, min_p, top_p, seed):
+    out = np.empty(ids.shape[0], np.int32)
+    pos = np.ascontiguousarray(positions, dtype=np.int64)
+    log_min_p = float(np.log(np.float32(min_p))) if min_p > 0.0 else 0.0
+    assert lib.sbp_draw(ptr(out), ptr(ids), ptr(z), ptr(pos), C(ids.shape[0]), C(ids.shape[1]), C(top_k),
+                        C(int(min_p > 0.0)), ctypes.c_float(log_min_p), C(int(0.0 < top_p < 1.0)),
+                        ctypes.c_double(float(np.float32(top_p))), ctypes.c_uint64(seed)) == 0
+    return out
+
+
+def sampling_rows(vocab, n=24, seed=11):
+    r = np.random.default_rng(seed)
+    rows = (r.standard_normal((n, vocab)) * 3.0).astype(np.float32)
+    rows[::5] *= 0.07                      # flat rows
+    rows[3, 10:20] = rows[3, 5]            # ties among the best
+    rows[1, 3] = 80.0                      # one candidate far above the window
+    positions = [int(q) for q in r.integers(0, 5000, size=n)]
+    positions[0], positions[1] = 0, 2 ** 33 + 5
+    return rows, positions
+
+
+SAMPLING_CASES = [dict(temperature=0.8), dict(temperature=1.3, top_k=5), dict(temperature=0.5, top_p=0.7),
+                  dict(temperature=1.0, min_p=0.2), dict(temperature=0.9, top_k=40, top_p=0.9, min_p=0.01),
+                  dict(temperature=1.0, top_p=1e-9, min_p=1.0)]
+
+
+def test_sampling_twins_agree_with_the_plain_sampler():
+    lib = twins()
+    rows, positions = sampling_rows(400)
+    # penalties, both arithmetic forms
+    history = [5, 9, 5, 399, 5, 17]
+    for exact in (False, True):
+        want = SP.penalize(rows[0], exact, repeat_penalty=1.3, repeat_last_n=64, presence_penalty=0.25,
+                           frequency_penalty=0.125, history=history)
+        got = host_penalize(lib, rows[:1], [0, 0, 0, 0], [5, 9, 399, 17], [3, 1, 1, 1], 1.3, 0.25, 0.125, exact)
+        assert np.array_equal(got[0], want)
+    seed = 0x9E3779B97F4A7C15
+    for case in SAMPLING_CASES:
+        t = case["temperature"]
+        ids, z = host_candidates(lib, rows, 256, t)
+        got = host_draw(lib, ids, z, positions, case.get("top_k", 0), case.get("min_p", 0.0), case.get("top_p", 1.0), seed)
+        for i in range(rows.shape[0]):
+            cands = SP.select_candidates(rows[i], t)
+            assert ids[i].tolist() == [c[0] for c in cands] and z[i].tolist() == [float(c[1]) for c in cands]
+            kept = SP.filter_candidates(cands, case.get("top_k", 0), case.get("top_p", 1.0), case.get("min_p", 0.0))
+            assert got[i] == SP.draw(kept, seed, positions[i]), (case, i)
+    # a row shorter than the candidates asked for is filled with id -1
+    ids, z = host_candidates(lib, rows[:2, :40], 64, 1.0)
+    assert (ids[:, 40:] == -1).all() and (ids[:, :40] >= 0).all()
+
+
 # ---- kernels against twins ---------------------------------------------------------------------
 @pytest.mark.gpu
 def test_kernels_equal_their_host_twins():
@@ -186,3 +253,23 @@ def test_kernels_equal_their_host_twins():
     ids = np.empty(4, np.int32)
     lib.sbp_argmax(ptr(ids), ptr(logits), C(4), C(20001))
     assert ops.argmax(dev(logits)).cpu().numpy().tolist() == ids.tolist() and ids[1] == 7
+    # penalties, candidates, filters and draw
+    rows, positions = sampling_rows(5000, n=16, seed=21)
+    item_rows, item_toks, item_counts = [0, 0, 3, 15], [7, 4999, 0, 123], [2, 1, 4, 1]
+    for exact in (False, True):
+        want = host_penalize(lib, rows, item_rows, item_toks, item_counts, 1.3, 0.25, 0.125, exact)
+        got = dev(rows).clone()
+        ops.penalize(got, dev(i32(item_rows)), dev(i32(item_toks)), dev(i32(item_counts)), 1.3, 0.25, 0.125, exact=exact)
+        assert np.array_equal(got.cpu().numpy(), want)
+    seed = 0x9E3779B97F4A7C15
+    for case in SAMPLING_CASES:
+        t = case["temperature"]
+        ids_h, z_h = host_candidates(lib, rows, 256, t)
+        ids_d, z_d = ops.top_candidates(dev(rows), t, 256)
+        assert np.array_equal(ids_d.cpu().numpy(), ids_h) and np.array_equal(z_d.cpu().numpy(), z_h)
+        min_p, top_p = case.get("min_p", 0.0), case.get("top_p", 1.0)
+        want = host_draw(lib, ids_h, z_h, positions, case.get("top_k", 0), min_p, top_p, seed)
+        got = ops.draw(ids_d, z_d, positions, case.get("top_k", 0),
+                       float(np.log(np.float32(min_p))) if min_p > 0.0 else None,
+                       float(np.float32(top_p)) if 0.0 < top_p < 1.0 else None, seed)
+        assert got.cpu().numpy().tolist() == want.tolist(), case
