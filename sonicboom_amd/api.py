@@ -75,9 +75,12 @@ class Session:
                  top_k: int = 0, seed: int = 0, max_tokens: int = 16, min_p: float = 0.0,
                  repeat_penalty: float = 1.0, repeat_last_n: int = 64, presence_penalty: float = 0.0,
                  frequency_penalty: float = 0.0, stop_tokens: Optional[Iterable[int]] = None,
-                 max_batch: int = 64, callback: Optional[Callable] = None) -> List[List[int]]:
+                 max_batch: int = 64, callback: Optional[Callable] = None,
+                 allowed: Optional[Callable] = None) -> List[List[int]]:
+        """``allowed(i, history)`` returns the bitmap of the ids request i may choose next (bit
+        i & 7 of byte i >> 3 for id i; None: any): the mask of constrained decoding."""
         params = SamplingParams(temperature=temperature, top_p=top_p, top_k=top_k, seed=seed,
                                 max_tokens=max_tokens, min_p=min_p, repeat_penalty=repeat_penalty,
                                 repeat_last_n=repeat_last_n, presence_penalty=presence_penalty,
                                 frequency_penalty=frequency_penalty)
-        return generate(self.engine, prompts, params, stop_tokens, max_batch, callback)
+        return generate(self.engine, prompts, params, stop_tokens, max_batch, callback, allowed=allowed)

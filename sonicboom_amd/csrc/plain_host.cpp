@@ -253,6 +253,19 @@ int sbp_penalize(float *logits, int vocab, const int32_t *item_row, const int32_
   return 0;
 }
 
+// The mask of constrained decoding in place (/root/reference/core/src/nn/sampling.cpp:266-274): -inf
+// wherever bit i & 7 of byte i >> 3 of the row's bitmap is clear or the bitmap ends before it.
+int sbp_mask_logits(float *logits, int n_rows, int vocab, const uint8_t *bitmaps, int n_bytes) {
+  if (!logits || !bitmaps || n_rows < 0 || vocab <= 0 || n_bytes <= 0) return 1;
+  for (int r = 0; r < n_rows; ++r)
+    for (int i = 0; i < vocab; ++i) {
+      const int byte = i >> 3;
+      const bool allowed = byte < n_bytes && ((bitmaps[size_t(r) * n_bytes + byte] >> (i & 7)) & 1u);
+      if (!allowed) logits[size_t(r) * vocab + i] = -std::numeric_limits<float>::infinity();
+    }
+  return 0;
+}
+
 // The k best of every row by z = logit / temperature (one float32 division), ordered
 // (z descending, id ascending); id -1 and z 0 past a short row's end
 // (/root/reference/core/src/nn/sampling.cpp:257-285).

@@ -33,6 +33,7 @@ int sbp_argmax(int32_t *ids, const float *logits, int n_rows, int vocab);
 int sbp_penalize(float *logits, int vocab, const int32_t *item_row, const int32_t *item_token,
                  const int32_t *item_count, int n_items, float repeat_penalty, float presence_penalty,
                  float frequency_penalty, int exact);
+int sbp_mask_logits(float *logits, int n_rows, int vocab, const uint8_t *bitmaps, int n_bytes);
 int sbp_top_candidates(int32_t *cand_id, float *cand_z, const float *logits, int n_rows, int vocab, int k,
                        float temperature);
 int sbp_draw(int32_t *token, const int32_t *cand_id, const float *cand_z, const int64_t *position, int n_rows,

@@ -102,6 +102,19 @@ __global__ void penalize_kernel(float *__restrict__ logits, int vocab,
   *p = v;
 }
 
+// The mask of constrained decoding (/root/reference/core/src/nn/sampling.cpp:266-274, :334-339): bit
+// i & 7 of byte i >> 3 of a row's bitmap says whether id i may be chosen; an id past the bitmap
+// may not.  What may not be chosen gets -inf, which neither the argmax nor the candidates' window
+// ever takes while one id is allowed.
+__global__ void mask_logits_kernel(float *__restrict__ logits, int vocab, const uint8_t *__restrict__ bitmaps,
+                                   int n_bytes) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x, row = blockIdx.y;
+  if (i >= vocab) return;
+  const int byte = i >> 3;
+  const bool allowed = byte < n_bytes && ((bitmaps[size_t(row) * n_bytes + byte] >> (i & 7)) & 1u);
+  if (!allowed) logits[size_t(row) * vocab + i] = -__builtin_inff();
+}
+
 // Order-preserving map of a float to an unsigned key (larger float, larger key).
 __device__ __forceinline__ uint32_t float_key(float z) {
   z = z + 0.0f;  // -0 and +0 are one value
@@ -475,6 +488,20 @@ extern "C" int sb_penalize(float *logits, int vocab, const int32_t *item_row, co
       logits, vocab, item_row, item_token, item_count, n_items, repeat_penalty, presence_penalty,
       frequency_penalty, exact);
   return sb::check_launch("sb_penalize");
+}
+
+// logits [n_rows, vocab] in place: -inf wherever the row's bitmap (bitmaps uint8 [n_rows, n_bytes],
+// bit i & 7 of byte i >> 3 for id i; ids past it are not allowed) does not allow the id.
+extern "C" int sb_mask_logits(float *logits, int n_rows, int vocab, const uint8_t *bitmaps, int n_bytes,
+                              void *stream) {
+  SB_REQUIRE(logits && bitmaps, "sb_mask_logits: null pointer");
+  SB_REQUIRE(n_rows >= 0 && vocab > 0 && n_bytes > 0, "sb_mask_logits: bad sizes rows=%d vocab=%d bytes=%d", n_rows,
+             vocab, n_bytes);
+  SB_SUPPORT(n_rows <= 65535, "sb_mask_logits: more than 65535 rows");
+  if (n_rows == 0) return SB_OK;
+  mask_logits_kernel<<<dim3((vocab + 255) / 256, n_rows), 256, 0, (hipStream_t)stream>>>(logits, vocab, bitmaps,
+                                                                                        n_bytes);
+  return sb::check_launch("sb_mask_logits");
 }
 
 // 64-bit words of scratch sb_top_candidates needs for rows of this length (0: none).  Rows of

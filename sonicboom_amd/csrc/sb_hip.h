@@ -143,6 +143,11 @@ int sb_penalize(float *logits, int vocab, const int32_t *item_row, const int32_t
                 const int32_t *item_count, int n_items, float repeat_penalty,
                 float presence_penalty, float frequency_penalty, int exact, void *stream);
 
+/* The mask of constrained decoding on logits [n_rows, vocab] in place: -inf wherever
+ * a row's bitmap (uint8 [n_rows, n_bytes]; bit i & 7 of byte i >> 3 for id i; ids past
+ * the bitmap are not allowed) does not allow the id. */
+int sb_mask_logits(float *logits, int n_rows, int vocab, const uint8_t *bitmaps, int n_bytes, void *stream);
+
 /* The `k` (<= 256) candidates with the largest z = logit / temperature of every
  * row (ties toward the lower id), ordered by (z descending, id ascending).
  * cand_id int32 [n_rows,k], cand_z f32 [n_rows,k]; rows with vocab < k are

@@ -66,7 +66,8 @@ def plan_batches(prompt_lens: Sequence[int], max_new: int, n_pages: int, max_bat
 def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = SamplingParams(),
              stop_tokens: Optional[Iterable[int]] = None, max_batch: int = 64,
              callback: Optional[Callable[[int, int], Optional[bool]]] = None,
-             sampler=None) -> List[List[int]]:
+             sampler=None,
+             allowed: Optional[Callable[[int, Sequence[int]], Optional[bytes]]] = None) -> List[List[int]]:
     """Continue every prompt; returns the produced tokens per prompt.
 
     ``engine`` has ``alloc_slot()``, ``free_slot(slot)``, ``step(entries) ->
@@ -78,7 +79,11 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = 
     return value ends that request before that token, which is not part of the
     output (/root/reference/capi/src/capi.cpp:2892-2898: an abort at a token
     returns the tokens before it).  ``sampler`` has ``pick(logits, positions, histories)``
-    and defaults to the device sampler for ``params``.
+    and defaults to the device sampler for ``params``.  ``allowed(i, history)``, asked before
+    every choice of request i, returns the bitmap of the ids it may choose from (bit i & 7 of
+    byte i >> 3 for id i; None: any), the mask of constrained decoding; the sampler's ``pick``
+    then gets the bitmaps as ``masks=``.  A request that may choose nothing ends there, as it
+    does in the reference (/root/reference/capi/src/capi.cpp:2820).
     """
     params = params.validated()
     own_sampler = sampler is None
@@ -100,19 +105,27 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = 
     batches = plan_batches([len(p) for p in prompts], params.max_tokens, engine.cache.n_pages, max_batch,
                            engine.cache.max_slots)
     loop = engine.decode_loop() if hasattr(engine, "decode_loop") else None
-    on_device = loop is not None and own_sampler and not params.temperature > 0.0 and not params.has_penalties
+    on_device = loop is not None and own_sampler and not params.temperature > 0.0 and not params.has_penalties \
+        and allowed is None
+
+    def pick(logits, live):
+        more = {} if allowed is None else {"masks": [allowed(s.index, s.history) for s in live]}
+        return sampler.pick(logits, [len(s.history) for s in live], [s.history for s in live], **more)
+
     for batch in batches:
         live = [_Live(i, engine.alloc_slot(), list(prompts[i]), len(prompts[i])) for i in batch]
         try:
             # The prompts in one step; logits of every last row.
             logits = engine.step([StepEntry(s.slot, prompts[s.index], (s.prompt_len - 1,)) for s in live])
-            tokens = sampler.pick(logits, [len(s.history) for s in live], [s.history for s in live])
+            tokens = pick(logits, live)
             started = False
             while True:
                 flags = []
                 for s, t in zip(live, tokens):
                     t = int(t)
-                    if callback is not None and callback(s.index, t):
+                    if t < 0:
+                        ended = True                     # nothing could be chosen
+                    elif callback is not None and callback(s.index, t):
                         ended = True                     # aborted at this token: it is not reported
                     else:
                         s.out.append(t)
@@ -131,7 +144,7 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = 
                 # every live sequence goes on by the token it has just produced
                 if loop is None:
                     logits = engine.step([StepEntry(s.slot, (t,), (0,)) for s, t in zip(live, fed)])
-                    tokens = sampler.pick(logits, [len(s.history) for s in live], [s.history for s in live])
+                    tokens = pick(logits, live)
                     continue
                 if not started or not all(flags):
                     loop.start([s.slot for s in live], fed)
@@ -140,7 +153,7 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = 
                     tokens = loop.step()             # greedy choice on the device, fed back by the loop
                 else:
                     logits = loop.step_logits(fed)
-                    tokens = sampler.pick(logits, [len(s.history) for s in live], [s.history for s in live])
+                    tokens = pick(logits, live)
         finally:
             for s in live:
                 if s.slot >= 0:

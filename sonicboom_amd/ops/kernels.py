@@ -304,6 +304,20 @@ def top_candidates(logits: torch.Tensor, temperature: float, k: int = MAX_CANDID
     return ids, z
 
 
+def mask_logits(logits: torch.Tensor, bitmaps: torch.Tensor) -> None:
+    """The mask of constrained decoding, in place: float32 ``logits`` [rows, vocab] become -inf
+    wherever the row's bitmap (uint8 [rows, bytes]: bit i & 7 of byte i >> 3 for id i; ids past the
+    bitmap are not allowed) does not allow the id."""
+    _dev(logits, bitmaps)
+    if logits.dtype != torch.float32 or logits.dim() != 2 or not logits.is_contiguous():
+        raise KernelLibraryError("logits must be contiguous float32 [rows, vocab]")
+    if bitmaps.dtype != torch.uint8 or bitmaps.dim() != 2 or bitmaps.shape[0] != logits.shape[0] \
+            or bitmaps.shape[1] == 0 or not bitmaps.is_contiguous():
+        raise KernelLibraryError("bitmaps must be contiguous uint8 [rows, bytes], a row for every row of logits")
+    check(library.core().sb_mask_logits(_p(logits), logits.shape[0], logits.shape[1], _p(bitmaps),
+                                        bitmaps.shape[1], _stream()))
+
+
 def draw(cand_ids: torch.Tensor, cand_z: torch.Tensor, positions, top_k: int, log_min_p: Optional[float],
          top_p: Optional[float], seed: int) -> torch.Tensor:
     """One token per row (int32 [n]; -1 where no candidate is kept) from the candidates that

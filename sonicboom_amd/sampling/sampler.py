@@ -2,7 +2,8 @@
 
 The order of stages is the reference's
 (/root/reference/core/include/sonicboom/nn/sampling.h:93-98): penalties over the
-last ``repeat_last_n`` tokens of the history, then either the argmax
+last ``repeat_last_n`` tokens of the history, the mask of constrained decoding (a
+bitmap of the ids a row may choose from, when the caller brings one), then either the argmax
 (temperature 0, ties to the lowest id) or: the 256 best candidates by
 z = logit / temperature, a window of 30 below the best, top-k, min-p, top-p,
 and a Gumbel-max draw with a Philox4x32-10 word keyed by (seed, position of
@@ -19,7 +20,7 @@ not depend on what else is in the batch.
 """
 from __future__ import annotations
 
-from typing import List, Sequence
+from typing import List, Optional, Sequence
 
 import numpy as np
 import torch
@@ -132,10 +133,15 @@ class Sampler:
     def __init__(self, params: SamplingParams):
         self.params = params.validated()
 
-    def pick(self, logits: torch.Tensor, positions: Sequence[int], histories: Sequence[Sequence[int]]) -> List[int]:
+    def pick(self, logits: torch.Tensor, positions: Sequence[int], histories: Sequence[Sequence[int]],
+             masks: Optional[Sequence[Optional[bytes]]] = None) -> List[int]:
         """One token per row of float32 ``logits`` [rows, vocab] (modified in place when
-        penalties apply).  ``positions[r]`` is the absolute position the new token of row r
-        will take; ``histories[r]`` its prompt and generated tokens so far."""
+        penalties or masks apply).  ``positions[r]`` is the absolute position the new token of
+        row r will take; ``histories[r]`` its prompt and generated tokens so far; ``masks[r]``
+        the bitmap of the ids row r may choose from (bit i & 7 of byte i >> 3 for id i, ids past
+        the bitmap not allowed; None or empty: no constraint), applied after the penalties
+        (/root/reference/core/src/nn/sampling.cpp:266-274, :334-339).  -1 for a row that may
+        choose nothing."""
         p = self.params
         n, vocab = logits.shape
         sampled = p.temperature > 0.0
@@ -146,11 +152,27 @@ class Sampler:
                 items = torch.tensor([rows, toks, counts], dtype=torch.int32).to(dev)
                 ops.penalize(logits, items[0].contiguous(), items[1].contiguous(), items[2].contiguous(),
                              p.repeat_penalty, p.presence_penalty, p.frequency_penalty, exact=sampled)
+        nothing_allowed = [False] * n
+        if masks is not None and any(masks):
+            n_bytes = (vocab + 7) // 8
+            bitmaps = np.zeros((n, n_bytes), dtype=np.uint8)
+            for r, mask in enumerate(masks):
+                if not mask:
+                    bitmaps[r] = 0xFF
+                    continue
+                row = np.frombuffer(bytes(mask), dtype=np.uint8)[:n_bytes]
+                bitmaps[r, :row.size] = row
+                if vocab % 8:
+                    bitmaps[r, -1] &= (1 << (vocab % 8)) - 1
+                nothing_allowed[r] = not bitmaps[r].any()
+            ops.mask_logits(logits, torch.from_numpy(bitmaps).to(logits.device))
         if not sampled:
-            return ops.argmax(logits).tolist()
+            tokens = ops.argmax(logits).tolist()
+            return [-1 if none else t for t, none in zip(tokens, nothing_allowed)]
         k = min(CANDIDATES, vocab)
         ids_d, z_d = ops.top_candidates(logits, p.temperature, k)
         # the cut-offs as the host form rounds them: ln(min_p) in float32, top_p through float32
         log_min_p = float(np.log(np.float32(p.min_p))) if p.min_p > 0.0 else None
         top_p = float(np.float64(np.float32(p.top_p))) if 0.0 < p.top_p < 1.0 else None
-        return ops.draw(ids_d, z_d, positions, p.top_k, log_min_p, top_p, p.seed).tolist()
+        tokens = ops.draw(ids_d, z_d, positions, p.top_k, log_min_p, top_p, p.seed).tolist()
+        return [-1 if none else t for t, none in zip(tokens, nothing_allowed)]

@@ -65,13 +65,22 @@ def penalize(logits, temperature_path: bool, repeat_penalty=1.0, repeat_last_n=6
     return adv
 
 
-def select_candidates(logits, temperature, history=(), **pen):
-    """core/src/nn/sampling.cpp:257-285: z = l_adj / T as one float32 division,
-    the 256 largest z (ties to the lower id), ordered (z descending, id
-    ascending)."""
+def allowed_by(mask, i: int) -> bool:
+    """core/src/nn/sampling.cpp:266-274: bit i & 7 of byte i >> 3; an id past the
+    bitmap is not allowed; an empty mask allows everything."""
+    if not mask:
+        return True
+    byte = i >> 3
+    return byte < len(mask) and bool((mask[byte] >> (i & 7)) & 1)
+
+
+def select_candidates(logits, temperature, history=(), mask=None, **pen):
+    """core/src/nn/sampling.cpp:257-285: z = l_adj / T as one float32 division
+    over the ids the mask allows, the 256 largest z (ties to the lower id),
+    ordered (z descending, id ascending)."""
     adv = penalize(logits, True, history=history, **pen)
     T = F32(temperature)
-    cands = [(i, F32(adv[i] / T)) for i in range(adv.shape[0])]
+    cands = [(i, F32(adv[i] / T)) for i in range(adv.shape[0]) if allowed_by(mask, i)]
     cands.sort(key=lambda c: (-float(c[1]), c[0]))
     return cands[:K_CANDIDATES]
 
@@ -121,18 +130,19 @@ def draw(cands, seed: int, position: int) -> int:
 
 def sample_token(logits, position: int, temperature=0.0, seed=0, top_k=0, top_p=1.0,
                  min_p=0.0, repeat_penalty=1.0, repeat_last_n=64, presence_penalty=0.0,
-                 frequency_penalty=0.0, history=()) -> int:
-    """core/src/nn/sampling.cpp:314-352 without the grammar mask."""
+                 frequency_penalty=0.0, history=(), mask=None) -> int:
+    """core/src/nn/sampling.cpp:314-352 (the mask as a filter over the ids, not
+    through the compacted list, which selects the same)."""
     pen = dict(repeat_penalty=repeat_penalty, repeat_last_n=repeat_last_n,
                presence_penalty=presence_penalty, frequency_penalty=frequency_penalty)
     if not temperature > 0.0:
         adv = penalize(logits, False, history=history, **pen)
-        best = 0
-        for i in range(1, adv.shape[0]):
-            if adv[i] > adv[best]:
+        best = -1
+        for i in range(adv.shape[0]):
+            if allowed_by(mask, i) and (best < 0 or adv[i] > adv[best]):
                 best = i
         return best
-    cands = select_candidates(logits, temperature, history=history, **pen)
+    cands = select_candidates(logits, temperature, history=history, mask=mask, **pen)
     kept = filter_candidates(cands, top_k=top_k, top_p=top_p, min_p=min_p)
     return draw(kept, seed, position)
 

@@ -78,6 +78,46 @@ def test_temperature_sampling_tiny_b(model_folders):
             assert t == want, (len(p), i)
 
 
+@pytest.mark.parametrize("temperature", [0.0, 0.9])
+def test_masks_of_constrained_decoding(model_folders, temperature):
+    """A bitmap of allowed ids per request and step: the engine's tokens are the plain sampler's
+    under the same masks (after the penalties), a request without a mask is not constrained, and a
+    request that may choose nothing ends there."""
+    folder = model_folders["A"]
+    prompts = prompts_for("A", [6, 11, 9], seed=8)
+    session = model_for(folder, "float32").session(max_tokens=64 * 4)
+    vocab = session.model.vocab_size
+    n_bytes = (vocab + 7) // 8
+
+    def allowed(i, history):
+        if i == 1:
+            return None                                   # unconstrained
+        if i == 2 and len(history) >= len(prompts[2]) + 4:
+            return bytes(n_bytes)                         # nothing may follow the fourth token
+        rng = np.random.default_rng(1000 * i + len(history))
+        bits = rng.integers(0, 256, size=n_bytes if i == 0 else n_bytes // 2, dtype=np.uint8)   # a short bitmap too
+        return bytes(bits)
+
+    kw = dict(temperature=temperature, seed=21, top_k=30, repeat_penalty=1.2, presence_penalty=0.1,
+              max_tokens=8, stop_tokens=())
+    outs = session.generate(prompts, allowed=allowed, **kw)
+    assert [len(o) for o in outs] == [8, 8, 4]
+    for r, (p, out) in enumerate(zip(prompts, outs)):
+        logits = plain_logits(folder, p + out)
+        hist = list(p)
+        for i, t in enumerate(out):
+            mask = allowed(r, hist)
+            want = sampling_plain.sample_token(logits[len(p) - 1 + i], len(p) + i, temperature=temperature, seed=21,
+                                               top_k=30, repeat_penalty=1.2, presence_penalty=0.1, history=hist,
+                                               mask=mask)
+            assert t == want, (r, i)
+            if mask:
+                assert (mask[t >> 3] >> (t & 7)) & 1
+            hist.append(t)
+    # alone or in the batch, the same tokens
+    assert [session.generate([p], allowed=lambda i, h, r=r: allowed(r, h), **kw)[0] for r, p in enumerate(prompts)] == outs
+
+
 def test_sampling_filters_and_penalties_run_on_the_device(model_folders):
     folder = model_folders["A"]
     prompts = prompts_for("A", [6, 11], seed=5)

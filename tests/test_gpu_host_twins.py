@@ -19,8 +19,8 @@ def twins():
     from sonicboom_amd.csrc import build
     lib = ctypes.CDLL(build.ensure_plain_host())
     for name in ("sbp_embed", "sbp_rmsnorm", "sbp_reduce_resid_norm", "sbp_gemm", "sbp_silu_mul", "sbp_add_into",
-                 "sbp_rope_kv_store", "sbp_attention", "sbp_argmax", "sbp_penalize", "sbp_top_candidates",
-                 "sbp_draw"):
+                 "sbp_rope_kv_store", "sbp_attention", "sbp_argmax", "sbp_penalize", "sbp_mask_logits",
+                 "sbp_top_candidates", "sbp_draw"):
         getattr(lib, name).restype = ctypes.c_int
     return lib
 
@@ -124,6 +124,12 @@ def host_penalize(lib, logits, rows, toks, counts, rp, pp, fp, exact):
     return out
 
 
+def host_mask(lib, logits, bitmaps):
+    out = np.array(logits, np.float32, copy=True)
+    assert lib.sbp_mask_logits(ptr(out), C(out.shape[0]), C(out.shape[1]), ptr(bitmaps), C(bitmaps.shape[1])) == 0
+    return out
+
+
 def host_candidates(lib, logits, k, temperature):
     ids, z = np.empty((logits.shape[0], k), np.int32), np.empty((logits.shape[0], k), np.float32)
     assert lib.sbp_top_candidates(ptr(ids), ptr(z), ptr(logits), C(logits.shape[0]), C(logits.shape[1]), C(k),
@@ -180,6 +186,17 @@ def test_sampling_twins_agree_with_the_plain_sampler():
     # a row shorter than the candidates asked for is filled with id -1
     ids, z = host_candidates(lib, rows[:2, :40], 64, 1.0)
     assert (ids[:, 40:] == -1).all() and (ids[:, :40] >= 0).all()
+    # the mask: the candidates of the masked row are the plain sampler's under the same mask
+    bitmaps = np.zeros((2, 12), np.uint8)            # 96 ids of 400: the rest is past the bitmap
+    bitmaps[0, [0, 3, 11]] = [0b00001001, 0xFF, 0x80]
+    bitmaps[1, :] = 0xFF
+    masked = host_mask(lib, rows[:2], bitmaps)
+    allowed0 = [0, 3] + list(range(24, 32)) + [95]
+    assert np.isneginf(np.delete(masked[0], allowed0)).all() and np.array_equal(masked[0, allowed0], rows[0, allowed0])
+    assert np.array_equal(masked[1, :96], rows[1, :96]) and np.isneginf(masked[1, 96:]).all()
+    ids, z = host_candidates(lib, masked, 256, 0.8)
+    want = SP.select_candidates(rows[0], 0.8, mask=bytes(bitmaps[0]))
+    assert ids[0, :len(want)].tolist() == [c[0] for c in want] and np.isneginf(z[0, len(want):]).all()
 
 
 # ---- kernels against twins ---------------------------------------------------------------------
@@ -261,6 +278,10 @@ def test_kernels_equal_their_host_twins():
         got = dev(rows).clone()
         ops.penalize(got, dev(i32(item_rows)), dev(i32(item_toks)), dev(i32(item_counts)), 1.3, 0.25, 0.125, exact=exact)
         assert np.array_equal(got.cpu().numpy(), want)
+    bitmaps = np.random.default_rng(5).integers(0, 256, size=(rows.shape[0], 500), dtype=np.uint8)   # 4,000 ids of 5,000
+    masked = dev(rows).clone()
+    ops.mask_logits(masked, dev(bitmaps))
+    assert np.array_equal(masked.cpu().numpy(), host_mask(lib, rows, bitmaps))
     seed = 0x9E3779B97F4A7C15
     for case in SAMPLING_CASES:
         t = case["temperature"]

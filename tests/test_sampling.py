@@ -147,6 +147,33 @@ def test_all_rows_at_once_equal_the_plain_sampler_row_by_row(params):
         assert one == [got[i]]
 
 
+def test_mask_of_constrained_decoding():
+    """The plain sampler's mask (/root/reference/core/src/nn/sampling.cpp:266-274, :334-339): bit i & 7
+    of byte i >> 3 allows id i, an id past the bitmap is not allowed, an empty mask allows all."""
+    logits = np.array([0.1, 5.0, 0.3, 4.0, -1.0, 4.5, 0.0, 0.2, 9.0, 3.0], dtype=F32)
+    only = lambda *ids: bytes(sum(1 << (i & 7) for i in ids if i >> 3 == b) for b in range(2))  # noqa: E731
+    assert SP.sample_token(logits, 0) == 8 and SP.sample_token(logits, 0, mask=b"") == 8
+    assert SP.sample_token(logits, 0, mask=only(3, 5, 9)) == 5           # the best of the allowed
+    assert SP.sample_token(logits, 0, mask=only(3, 5, 9)[:1]) == 5       # a bitmap of one byte: ids 0..7
+    assert SP.sample_token(logits, 0, mask=bytes([0xFF])) == 1           # 8 and 9 lie past it
+    assert SP.sample_token(logits, 0, mask=bytes(2)) == -1               # nothing allowed
+    assert SP.sample_token(logits, 0, temperature=0.7, seed=3, mask=bytes(2)) == -1
+    # penalties come first: the penalised best of the allowed loses to the next one
+    assert SP.sample_token(logits, 3, mask=only(3, 5), history=[5, 5, 5], frequency_penalty=1.0) == 3
+    # sampled: only allowed ids are ever drawn, every allowed id within the window is drawn sometimes
+    mask = only(0, 3, 5, 9)
+    drawn = {SP.sample_token(logits, pos, temperature=1.5, seed=11, mask=mask) for pos in range(300)}
+    assert drawn == {0, 3, 5, 9}
+    cands = SP.select_candidates(logits, 1.5, mask=mask)
+    assert [c[0] for c in cands] == [5, 3, 9, 0]
+    # an allowed id is drawn as it would be from the same candidates without a mask
+    sub = np.full(10, -np.inf, dtype=F32)
+    sub[[0, 3, 5, 9]] = logits[[0, 3, 5, 9]]
+    for pos in range(50):
+        assert SP.sample_token(logits, pos, temperature=1.5, seed=11, mask=mask) == \
+            SP.sample_token(sub, pos, temperature=1.5, seed=11)
+
+
 def test_params_validation():
     assert SamplingParams(repeat_penalty=0.0).validated().repeat_penalty == 1.0
     assert not SamplingParams().has_penalties and SamplingParams(presence_penalty=0.1).has_penalties
