@@ -161,3 +161,31 @@ def test_portions_of_a_long_step():
         assert flat == [(i, r) for i, n in enumerate(n_new) for r in range(n)]
     with pytest.raises(ValueError):
         portion_rows([3], 0)
+
+
+def test_masks_reach_the_sampler_and_a_request_that_may_choose_nothing_ends():
+    """``allowed`` is asked before every choice with the request's index and history; its bitmaps
+    go to the sampler as ``masks``; a sampler's -1 (nothing may be chosen) ends that request
+    without a token, frees its slot at once, and the others go on."""
+    asked = []
+
+    class MaskedSampler(HostSampler):
+        def pick(self, logits, positions, histories, masks=None):
+            assert masks is not None and len(masks) == len(positions)
+            picks = super().pick(logits, positions, histories)
+            return [-1 if m == b"\x00" else t for t, m in zip(picks, masks)]
+
+    def allowed(i, history):
+        asked.append((i, len(history)))
+        return b"\x00" if i == 1 and len(history) >= 9 + 3 else None
+
+    eng, smp = TableEngine(64 * 8), MaskedSampler()
+    prompts = [[1, 2, 3, 4, 5], [9] * 9, [4] * 13]
+    outs = generate(eng, prompts, SamplingParams(max_tokens=6), stop_tokens=(), sampler=smp, allowed=allowed)
+    assert outs == [expected(prompts[0], 6), expected(prompts[1], 3), expected(prompts[2], 6)]
+    assert asked[:3] == [(0, 5), (1, 9), (2, 13)] and (1, 12) in asked and (1, 13) not in asked
+    assert eng.steps[4] == [(0, 1), (2, 1)]                           # request 1 has left the batch
+    assert not eng.cache.live_slots and eng.cache.held_pages() == 0
+    # without ``allowed`` a sampler of the three-argument form is called as before
+    assert generate(TableEngine(64 * 8), prompts, SamplingParams(max_tokens=2), stop_tokens=(), sampler=HostSampler()) \
+        == [expected(p, 2) for p in prompts]
