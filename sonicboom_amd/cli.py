@@ -13,7 +13,7 @@ import argparse
 import json
 import sys
 
-USAGE = ("usage: sb-gen (-m MODEL_DIR | --random CONFIG.json [--seed S]) --tokens FILE [-n N] [--ctx N]\n"
+USAGE = ("sb-gen (-m MODEL_DIR | --random CONFIG.json [--seed S]) --tokens FILE [-n N] [--ctx N]\n"
          "              [--dtype bfloat16|float32] [--batch B] [--temperature T] [--top-k K] [--top-p P]\n"
          "              [--min-p P] [--sample-seed S] [--repeat-penalty R] [--repeat-last-n N]\n"
          "              [--presence-penalty X] [--frequency-penalty X] [--stop ID,ID,...]\n")
@@ -21,7 +21,7 @@ USAGE = ("usage: sb-gen (-m MODEL_DIR | --random CONFIG.json [--seed S]) --token
 
 class _Parser(argparse.ArgumentParser):
     def error(self, message):
-        sys.stderr.write(f"sb-gen: {message}\n{USAGE}")
+        sys.stderr.write(f"sb-gen: {message}\nusage: {USAGE}")
         raise SystemExit(2)
 
 
