@@ -121,7 +121,7 @@ class OpTimer:
     times are summed by (function, what it worked on)."""
 
     NAMES = ("embed", "rmsnorm", "gemm_bf16", "gemm_bf16_partial", "reduce_resid_norm", "rope_kv_store",
-             "attention", "argmax", "gemm_plain", "silu_mul", "add_into", "cast")
+             "attention", "attention_decode_rope", "argmax", "gemm_plain", "silu_mul", "add_into", "cast")
 
     def __init__(self, m):
         self.m, self.records, self._saved = m, [], {}
@@ -134,7 +134,9 @@ class OpTimer:
                 return "gate_up"
             return {(m["qw"] + 2 * m["kvw"], m["d"]): "qkv", (m["d"], m["qw"]): "out", (m["d"], m["ff"]): "down",
                     (m["v"], m["d"]): "head"}.get((n, k), f"product_{n}x{k}")
-        return {"reduce_resid_norm": "add_slices_norm", "rope_kv_store": "rotate_store"}.get(name, name)
+        # (a decode step's attention rotates and stores the new key and value itself)
+        return {"reduce_resid_norm": "add_slices_norm", "rope_kv_store": "rotate_store",
+                "attention_decode_rope": "attention"}.get(name, name)
 
     def __enter__(self):
         import torch
