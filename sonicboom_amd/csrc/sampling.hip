@@ -303,10 +303,11 @@ __device__ __forceinline__ uint32_t philox_word0(uint32_t c0, uint32_t c1, uint3
 
 constexpr int kDrawPerLane = kMaxCand / 64;
 
+template <typename POS>    // int64 positions, or int32 lengths to which position_offset is added
 __global__ void __launch_bounds__(64)
 draw_kernel(int32_t *__restrict__ token, const int32_t *__restrict__ cand_id, const float *__restrict__ cand_z,
-            const int64_t *__restrict__ position, int k, int top_k, int use_min_p, float log_min_p,
-            int use_top_p, double top_p, uint64_t seed) {
+            const POS *__restrict__ position, int64_t position_offset, int k, int top_k, int use_min_p,
+            float log_min_p, int use_top_p, double top_p, uint64_t seed) {
   __shared__ double e_of[kMaxCand];
   __shared__ int n_keep_sh;
   const int row = blockIdx.x, lane = threadIdx.x;
@@ -360,7 +361,7 @@ draw_kernel(int32_t *__restrict__ token, const int32_t *__restrict__ cand_id, co
   }
   double best = -__builtin_inf();
   int best_id = 0x7fffffff;
-  const uint64_t pos = uint64_t(position[row]);
+  const uint64_t pos = uint64_t(int64_t(position[row]) + position_offset);
 #pragma unroll
   for (int j = 0; j < kDrawPerLane; ++j) {
     const int c = lane + 64 * j;
@@ -553,7 +554,21 @@ extern "C" int sb_draw(int32_t *token, const int32_t *cand_id, const float *cand
   SB_REQUIRE(n_rows >= 0 && top_k >= 0, "sb_draw: bad sizes rows=%d top_k=%d", n_rows, top_k);
   SB_SUPPORT(k >= 1 && k <= kMaxCand, "sb_draw: %d candidates a row, at most %d", k, kMaxCand);
   if (n_rows == 0) return SB_OK;
-  draw_kernel<<<n_rows, 64, 0, (hipStream_t)stream>>>(token, cand_id, cand_z, position, k, top_k, use_min_p,
-                                                      log_min_p, use_top_p, top_p, seed);
+  draw_kernel<int64_t><<<n_rows, 64, 0, (hipStream_t)stream>>>(token, cand_id, cand_z, position, 0, k, top_k,
+                                                               use_min_p, log_min_p, use_top_p, top_p, seed);
   return sb::check_launch("sb_draw");
+}
+
+// The same for a decode step whose bookkeeping lives on the device: the position of row r's new
+// token is length_before[r] + 1 (the token it feeds sits at length_before[r]).
+extern "C" int sb_draw_after(int32_t *token, const int32_t *cand_id, const float *cand_z,
+                             const int32_t *length_before, int n_rows, int k, int top_k, int use_min_p,
+                             float log_min_p, int use_top_p, double top_p, uint64_t seed, void *stream) {
+  SB_REQUIRE(token && cand_id && cand_z && length_before, "sb_draw_after: null pointer");
+  SB_REQUIRE(n_rows >= 0 && top_k >= 0, "sb_draw_after: bad sizes rows=%d top_k=%d", n_rows, top_k);
+  SB_SUPPORT(k >= 1 && k <= kMaxCand, "sb_draw_after: %d candidates a row, at most %d", k, kMaxCand);
+  if (n_rows == 0) return SB_OK;
+  draw_kernel<int32_t><<<n_rows, 64, 0, (hipStream_t)stream>>>(token, cand_id, cand_z, length_before, 1, k, top_k,
+                                                               use_min_p, log_min_p, use_top_p, top_p, seed);
+  return sb::check_launch("sb_draw_after");
 }

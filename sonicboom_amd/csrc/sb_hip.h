@@ -167,6 +167,11 @@ int sb_top_candidates(int32_t *cand_id, float *cand_z, const float *logits, int 
 int sb_draw(int32_t *token, const int32_t *cand_id, const float *cand_z, const int64_t *position,
             int n_rows, int k, int top_k, int use_min_p, float log_min_p, int use_top_p, double top_p,
             uint64_t seed, void *stream);
+/* The same with the positions taken from a decode step's device bookkeeping:
+ * row r's new token takes position length_before[r] + 1. */
+int sb_draw_after(int32_t *token, const int32_t *cand_id, const float *cand_z, const int32_t *length_before,
+                  int n_rows, int k, int top_k, int use_min_p, float log_min_p, int use_top_p, double top_p,
+                  uint64_t seed, void *stream);
 
 /* ---- bf16 products on the matrix cores ----------------------------------
  * X bf16 [n_rows, n_in] row-major, n_in a multiple of 8, operands 16-byte

@@ -131,8 +131,8 @@ class DecodeLoop:
         # added rows would run a mixer's per-sequence state of some live slot: no padding then
         self.pad_batches = not engine.cache.state
         self._ctx: Dict[Tuple[int, int], _StaticContext] = {}
-        self._graphs: Dict[Tuple[int, int, bool], Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
-        self._uses: Dict[Tuple[int, int, bool], int] = {}
+        self._graphs: Dict[tuple, Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}    # (batch, width, choice)
+        self._uses: Dict[tuple, int] = {}
         self.slots: List[int] = []
         self.pending: List[int] = []
 
@@ -153,9 +153,21 @@ class DecodeLoop:
         batch = batch_bucket(len(self.slots)) if self.pad_batches else len(self.slots)
         return batch, ((need + WIDTH_STEP - 1) // WIDTH_STEP) * WIDTH_STEP
 
-    def _run(self, tokens: Sequence[int], choose: bool):
+    def _choose(self, logits: torch.Tensor, ctx, choose) -> None:
+        """The step's choice on the device, into ``ctx.next_ids``: the first maximum (``choose``
+        is True) or a draw (``choose`` = (temperature, candidates, top_k, ln min_p or None, top_p
+        or None, seed), what :meth:`Sampler.device_draw` gives) at the positions that follow from
+        the step's own lengths."""
+        if choose is True:
+            ops.argmax(logits, out=ctx.next_ids)
+        elif choose:
+            temperature, k, top_k, log_min_p, top_p, seed = choose
+            cand_ids, cand_z = ops.top_candidates(logits, temperature, k)
+            ops.draw(cand_ids, cand_z, ctx.len_before, top_k, log_min_p, top_p, seed, out=ctx.next_ids)
+
+    def _run(self, tokens: Sequence[int], choose):
         """One step of the live sequences feeding ``tokens``: the logits [B, vocab] and the
-        buffer that holds the greedy choice when ``choose``."""
+        buffer that holds the choice when ``choose`` asks for one (see :meth:`_choose`)."""
         eng = self.engine
         cache = eng.cache
         vocab = eng.model.vocab
@@ -182,8 +194,7 @@ class DecodeLoop:
             logits = entry[1]
         else:
             logits = eng.forward(ctx)
-            if choose:
-                ops.argmax(logits, out=ctx.next_ids)
+            self._choose(logits, ctx, choose)
             n = self._uses[gkey] = self._uses.get(gkey, 0) + 1
             if self.use_graph and n >= CAPTURE_AFTER:
                 self._capture(gkey, ctx, choose)
@@ -191,7 +202,7 @@ class DecodeLoop:
         live = len(self.slots)
         return logits[:live], ctx.next_ids[:live]
 
-    def _capture(self, gkey, ctx, choose: bool) -> None:
+    def _capture(self, gkey, ctx, choose) -> None:
         """Record the launches of a step of this shape.  Capture runs nothing; replays read the
         ids, positions and page tables that ``refresh`` puts into the fixed buffers."""
         torch.cuda.synchronize()
@@ -206,8 +217,7 @@ class DecodeLoop:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 logits = self.engine.forward(ctx)
-                if choose:
-                    ops.argmax(logits, out=ctx.next_ids)
+                self._choose(logits, ctx, choose)
         finally:
             if collecting:
                 gc.enable()
@@ -217,10 +227,11 @@ class DecodeLoop:
             self._uses.pop(oldest, None)
         self._graphs[gkey] = (graph, logits)
 
-    def step(self) -> List[int]:
-        """Feed the pending tokens and choose greedily; the new token of every sequence, which
-        is also what the next step feeds."""
-        _, ids = self._run(self.pending, choose=True)
+    def step(self, draw=None) -> List[int]:
+        """Feed the pending tokens and choose on the device, greedily or with ``draw`` (what
+        :meth:`Sampler.device_draw` gives); the new token of every sequence, which is also what
+        the next step feeds."""
+        _, ids = self._run(self.pending, choose=draw if draw else True)
         self.pending = ids.tolist()
         return self.pending
 

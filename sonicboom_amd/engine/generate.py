@@ -73,7 +73,8 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = 
     ``engine`` has ``alloc_slot()``, ``free_slot(slot)``, ``step(entries) ->
     logits`` and ``cache.n_pages`` / ``cache.max_slots``; when it also has
     ``decode_loop()`` the single-token steps go through that loop (fixed buffers,
-    HIP graph replay, greedy choice on the device).  ``stop_tokens``
+    HIP graph replay, the choice, greedy or drawn, on the device inside the replayed step unless
+    penalties or masks need the host).  ``stop_tokens``
     defaults to the model's own (its configuration's eos ids).  ``callback(i,
     token)`` is called for every produced token of request i in order; a true
     return value ends that request before that token, which is not part of the
@@ -105,8 +106,9 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = 
     batches = plan_batches([len(p) for p in prompts], params.max_tokens, engine.cache.n_pages, max_batch,
                            engine.cache.max_slots)
     loop = engine.decode_loop() if hasattr(engine, "decode_loop") else None
-    on_device = loop is not None and own_sampler and not params.temperature > 0.0 and not params.has_penalties \
-        and allowed is None
+    # the choice inside the loop's recorded step: greedy, or a draw that needs nothing of the host
+    on_device = loop is not None and own_sampler and not params.has_penalties and allowed is None
+    draw = sampler.device_draw(engine.model.vocab) if on_device else None
 
     def pick(logits, live):
         more = {} if allowed is None else {"masks": [allowed(s.index, s.history) for s in live]}
@@ -150,7 +152,7 @@ def generate(engine, prompts: Sequence[Sequence[int]], params: SamplingParams = 
                     loop.start([s.slot for s in live], fed)
                     started = True
                 if on_device:
-                    tokens = loop.step()             # greedy choice on the device, fed back by the loop
+                    tokens = loop.step(draw)         # the choice on the device, fed back by the loop
                 else:
                     logits = loop.step_logits(fed)
                     tokens = pick(logits, live)

@@ -319,12 +319,14 @@ def mask_logits(logits: torch.Tensor, bitmaps: torch.Tensor) -> None:
 
 
 def draw(cand_ids: torch.Tensor, cand_z: torch.Tensor, positions, top_k: int, log_min_p: Optional[float],
-         top_p: Optional[float], seed: int) -> torch.Tensor:
+         top_p: Optional[float], seed: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """One token per row (int32 [n]; -1 where no candidate is kept) from the candidates that
     :func:`top_candidates` wrote: the window of 30 below the best z, top-k (0: off), min-p
     (``log_min_p`` = ln(min_p) rounded to float32, None: off), top-p (a float64, None: off) and
     the Gumbel-max draw under (seed, position of the row's new token, candidate id).
-    ``positions``: one absolute position per row, a sequence or an int64 tensor on the device."""
+    ``positions``: one absolute position per row, a sequence or an int64 tensor on the device; or
+    an int32 tensor on the device of each row's cached length before the step, whose new token then
+    takes position length + 1 (a decode step's own bookkeeping: nothing comes from the host)."""
     _dev(cand_ids, cand_z)
     if cand_ids.dtype != torch.int32 or cand_z.dtype != torch.float32 or cand_ids.dim() != 2 \
             or tuple(cand_ids.shape) != tuple(cand_z.shape):
@@ -332,14 +334,19 @@ def draw(cand_ids: torch.Tensor, cand_z: torch.Tensor, positions, top_k: int, lo
     n, k = cand_ids.shape
     if not torch.is_tensor(positions):
         positions = torch.tensor([int(q) for q in positions], dtype=torch.int64).to(cand_ids.device)
-    _dev(positions)
-    if positions.dtype != torch.int64 or positions.numel() != n:
-        raise KernelLibraryError("positions must be int64, one per row")
-    out = torch.empty((n,), dtype=torch.int32, device=cand_ids.device)
-    check(library.core().sb_draw(_p(out), _p(cand_ids.contiguous()), _p(cand_z.contiguous()), _p(positions.contiguous()),
-                                 n, k, int(top_k), 0 if log_min_p is None else 1,
-                                 0.0 if log_min_p is None else float(log_min_p), 0 if top_p is None else 1,
-                                 0.0 if top_p is None else float(top_p), int(seed) & 0xFFFFFFFFFFFFFFFF, _stream()))
+    _dev(positions, out)
+    if positions.dtype not in (torch.int64, torch.int32) or positions.numel() != n or not positions.is_contiguous():
+        raise KernelLibraryError("positions must be int64 (or int32 lengths), contiguous, one per row")
+    if out is None:
+        out = torch.empty((n,), dtype=torch.int32, device=cand_ids.device)
+    elif out.dtype != torch.int32 or out.numel() != n or not out.is_contiguous():
+        raise KernelLibraryError("the tokens' buffer must be contiguous int32, one per row")
+    lib = library.core()
+    entry = lib.sb_draw if positions.dtype == torch.int64 else lib.sb_draw_after
+    check(entry(_p(out), _p(cand_ids.contiguous()), _p(cand_z.contiguous()), _p(positions),
+                n, k, int(top_k), 0 if log_min_p is None else 1,
+                0.0 if log_min_p is None else float(log_min_p), 0 if top_p is None else 1,
+                0.0 if top_p is None else float(top_p), int(seed) & 0xFFFFFFFFFFFFFFFF, _stream()))
     return out
 
 

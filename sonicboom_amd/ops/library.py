@@ -36,6 +36,7 @@ _CORE_SIGNATURES = {
     "sb_top_candidates": [_P, _P, _P, _I, _I, _I, _F, _P, _P],
     "sb_mask_logits": [_P, _I, _I, _P, _I, _P],
     "sb_draw": [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I, c_double, c_uint64, _P],
+    "sb_draw_after": [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I, c_double, c_uint64, _P],
 }
 # Entry points of later kernels; declared when the library has them.
 _OPTIONAL_SIGNATURES = {

@@ -133,6 +133,23 @@ class Sampler:
     def __init__(self, params: SamplingParams):
         self.params = params.validated()
 
+    def device_draw(self, vocab: int):
+        """What a decode loop needs to draw on the device inside its own recorded step
+        (temperature, candidates, top_k, ln min_p or None, top_p or None, seed): None when the
+        choice is greedy or needs the host (penalties over the histories)."""
+        p = self.params
+        if not p.temperature > 0.0 or p.has_penalties:
+            return None
+        return (float(p.temperature), min(CANDIDATES, vocab), int(p.top_k), self._log_min_p(), self._top_p(),
+                int(p.seed))
+
+    # the cut-offs as the host form rounds them: ln(min_p) in float32, top_p through float32
+    def _log_min_p(self) -> Optional[float]:
+        return float(np.log(np.float32(self.params.min_p))) if self.params.min_p > 0.0 else None
+
+    def _top_p(self) -> Optional[float]:
+        return float(np.float64(np.float32(self.params.top_p))) if 0.0 < self.params.top_p < 1.0 else None
+
     def pick(self, logits: torch.Tensor, positions: Sequence[int], histories: Sequence[Sequence[int]],
              masks: Optional[Sequence[Optional[bytes]]] = None) -> List[int]:
         """One token per row of float32 ``logits`` [rows, vocab] (modified in place when
@@ -171,8 +188,5 @@ class Sampler:
             return [-1 if none else t for t, none in zip(tokens, nothing_allowed)]
         k = min(CANDIDATES, vocab)
         ids_d, z_d = ops.top_candidates(logits, p.temperature, k)
-        # the cut-offs as the host form rounds them: ln(min_p) in float32, top_p through float32
-        log_min_p = float(np.log(np.float32(p.min_p))) if p.min_p > 0.0 else None
-        top_p = float(np.float64(np.float32(p.top_p))) if 0.0 < p.top_p < 1.0 else None
-        tokens = ops.draw(ids_d, z_d, positions, p.top_k, log_min_p, top_p, p.seed).tolist()
+        tokens = ops.draw(ids_d, z_d, positions, p.top_k, self._log_min_p(), self._top_p(), p.seed).tolist()
         return [-1 if none else t for t, none in zip(tokens, nothing_allowed)]
