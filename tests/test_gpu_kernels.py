@@ -1024,6 +1024,21 @@ def test_draw_equals_the_plain_sampler(params, vocab):
         assert got[i] == SP.draw(kept, seed, positions[i]), f"row {i}"
 
 
+def test_draw_at_the_positions_after_device_side_lengths():
+    """Lengths as a decode step keeps them on the device (int32): the new token's position is
+    length + 1, and the tokens are those of the same positions brought from the host."""
+    from sonicboom_amd import ops
+    r = np.random.default_rng(3)
+    logits = torch.tensor((r.standard_normal((40, 3000)) * 2.0).astype(np.float32), device=DEV)
+    ids, z = ops.top_candidates(logits, 0.9, ops.MAX_CANDIDATES)
+    lengths = [int(q) for q in r.integers(0, 4000, size=40)]
+    want = ops.draw(ids, z, [n + 1 for n in lengths], 50, None, 0.9, 12345).tolist()
+    out = torch.full((40,), -7, dtype=torch.int32, device=DEV)
+    got = ops.draw(ids, z, torch.tensor(lengths, dtype=torch.int32, device=DEV), 50, None, 0.9, 12345, out=out)
+    assert got is out and out.tolist() == want
+    assert ops.draw(ids, z, lengths, 50, None, 0.9, 12345).tolist() != want       # other positions, other draws
+
+
 def test_draw_keeps_no_candidate_of_an_empty_row():
     """A row whose candidates all lie outside (ids of -1, as a row shorter than k is filled)
     gives -1; its neighbours are not disturbed."""
