@@ -4,7 +4,8 @@ vocabularies that are no power of two and no multiple of a tile, one to three la
 untied heads, head_dim given or left to follow from the width.  Each is drawn from a seed,
 written as a model folder with random weights, and run in float32 and bfloat16 against the plain
 implementation: every request whole, with its tail token by token, and in a batch of unequal
-prompts; no page may be left held afterwards."""
+prompts; no page may be left held afterwards.  Widths of 2,048 and more are held to the bfloat16
+bounds of real layer sizes (rows that long round as those do), the others to the tiny models'."""
 import numpy as np
 import pytest
 
@@ -64,17 +65,19 @@ def test_odd_sizes_whole_tail_and_batch(tmp_path, seed):
     write_random_model(folder, dict(cfg), seed=100 + seed, dtype="bfloat16")
     requests = [[int(t) for t in rng.integers(0, cfg["vocab_size"], size=n)] for n in lengths]
     prompt_lengths = [max(1, n // 2) for n in lengths]
+    kind = "wide" if cfg["hidden_size"] >= 2048 else False
     try:
         for dtype in ("float32", "bfloat16"):
             engine = Engine(DecoderModel.from_folder(folder, dtype), 64 * 24)
             for tokens in requests:
                 want = plain_logits(folder, tokens)
-                assert_logits_close(run_whole(engine, tokens), want, dtype, f"{dtype} whole")
-                assert_logits_close(run_tail_one_by_one(engine, tokens), want, dtype, f"{dtype} tail")
+                assert_logits_close(run_whole(engine, tokens), want, dtype, f"{dtype} whole", kind)
+                assert_logits_close(run_tail_one_by_one(engine, tokens), want, dtype, f"{dtype} tail", kind)
             got = run_batch(engine, requests, prompt_lengths)
             for tokens, p, g in zip(requests, prompt_lengths, got):
                 want = plain_logits(folder, tokens)
-                assert_logits_close(g, want[p - 1:] if g.shape[0] != len(tokens) else want, dtype, f"{dtype} batch")
+                assert_logits_close(g, want[p - 1:] if g.shape[0] != len(tokens) else want, dtype, f"{dtype} batch",
+                                    kind)
             assert engine.cache.held_pages() == 0
             del engine
     finally:
