@@ -100,6 +100,16 @@ struct HalfPage {
   uint4 v[DT];
 };
 
+constexpr int CPRK = HD / 8;                       // 16-byte chunks in a row of keys
+constexpr int kPageChunks = SB_PAGE * HD / 8;      // 16-byte chunks of a page of keys (= of values)
+
+// Where chunk `chunk` (8 elements) of key row `key` of a page lies, in chunks from the page's
+// start: the cache's own order (sb_key_index), in which the sixteen rows a fragment read touches at
+// once (key bits 0, 1, 3, 4) land in distinct LDS banks; a page is copied into LDS as it lies.
+__device__ __forceinline__ int k_slot(int key, int chunk) { return key * CPRK + (chunk ^ sb_key_swizzle(key, HD)); }
+// ... and of chunk `chunk` (8 keys) of value row d (sb_value_index).
+__device__ __forceinline__ int v_slot(int d, int chunk) { return d * 8 + (chunk ^ ((d >> 1) & 7)); }
+
 __device__ __forceinline__ void load_half(HalfPage &hp, const bf16_t *__restrict__ kp,
                                           const bf16_t *__restrict__ vp, int half, int lane) {
   const int r = lane & 15, g = lane >> 4;
@@ -107,15 +117,14 @@ __device__ __forceinline__ void load_half(HalfPage &hp, const bf16_t *__restrict
   for (int t = 0; t < 2; ++t) {
     // A row r = 4 gg + i of score tile t is key 8 gg + 4 t + i of the 32
     const int key = 32 * half + 8 * (r >> 2) + 4 * t + (r & 3);
-    const bf16_t *krow = kp + size_t(key) * HD;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d = ks * 32 + g * 8;
-      hp.k[t][ks] = ld16(krow + d, d < HD);
+      hp.k[t][ks] = ld16(kp + size_t(k_slot(key, d < HD ? ks * 4 + g : 0)) * 8, d < HD);
     }
   }
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) hp.v[dt] = ld16(vp + size_t(dt * 16 + r) * SB_PAGE + 32 * half + 8 * g, true);
+  for (int dt = 0; dt < DT; ++dt) hp.v[dt] = ld16(vp + size_t(v_slot(dt * 16 + r, 4 * half + g)) * 8, true);
 }
 
 // The same without a branch around any load (a branch makes the compiler wait for every load in
@@ -127,21 +136,20 @@ __device__ __forceinline__ void load_half_straight(HalfPage &hp, const bf16_t *_
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     const int key = 32 * half + 8 * (r >> 2) + 4 * t + (r & 3);
-    const bf16_t *krow = kp + size_t(key) * HD;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d = ks * 32 + g * 8;
       if ((ks + 1) * 32 <= HD) {
-        hp.k[t][ks] = *reinterpret_cast<const uint4 *>(krow + d);
+        hp.k[t][ks] = *reinterpret_cast<const uint4 *>(kp + size_t(k_slot(key, ks * 4 + g)) * 8);
       } else {
-        const uint4 v = *reinterpret_cast<const uint4 *>(krow + (d < HD ? d : 0));
+        const uint4 v = *reinterpret_cast<const uint4 *>(kp + size_t(k_slot(key, d < HD ? ks * 4 + g : 0)) * 8);
         hp.k[t][ks] = d < HD ? v : make_uint4(0u, 0u, 0u, 0u);
       }
     }
   }
 #pragma unroll
   for (int dt = 0; dt < DT; ++dt)
-    hp.v[dt] = *reinterpret_cast<const uint4 *>(vp + size_t(dt * 16 + r) * SB_PAGE + 32 * half + 8 * g);
+    hp.v[dt] = *reinterpret_cast<const uint4 *>(vp + size_t(v_slot(dt * 16 + r, 4 * half + g)) * 8);
 }
 
 // 32 keys at absolute positions base .. base+31, their fragments in hp, for the wave's NC groups
@@ -260,18 +268,6 @@ __device__ __forceinline__ void load_q(bf16x8_t (&qf)[KS], const bf16_t *qrow, b
 // tiles: int32 [n_tiles][4] = (first row, rows, sequence, unused).  Grid: one dimension, the
 // block number counting (kv head, group of four head tiles) fastest and row tiles from the last
 // one down: the heavy (late) tiles of all heads start first and the short ones fill the gaps.
-constexpr int CPRK = HD / 8;                       // 16-byte chunks in a row of keys
-constexpr int kSwzK = CPRK % 16 == 0 ? 16 : (CPRK % 8 == 0 ? 8 : (CPRK % 4 == 0 ? 4 : 2));
-constexpr int kPageChunks = SB_PAGE * HD / 8;      // 16-byte chunks of a page of keys (= of values)
-
-// LDS position (in chunks) of chunk `chunk` of key row `key`: the sixteen rows a fragment read
-// touches at once (key bits 0, 1, 3, 4) land in distinct banks.
-__device__ __forceinline__ int k_slot(int key, int chunk) {
-  const int f = ((key & 3) | (((key >> 3) & 3) << 2)) & (kSwzK - 1);
-  return key * CPRK + (chunk ^ f);
-}
-// ... and of chunk `chunk` (8 keys) of value row d.
-__device__ __forceinline__ int v_slot(int d, int chunk) { return d * 8 + (chunk ^ ((d >> 1) & 7)); }
 
 __device__ __forceinline__ void load_half_lds(HalfPage &hp, const uint4 *kl, const uint4 *vl, int half, int lane) {
   const int r = lane & 15, g = lane >> 4;
@@ -518,8 +514,8 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
     for (int j = 0; j < kStageLoads; ++j) {
       const int id = tid + kThreads * j;
       if (kPageChunks % kThreads == 0 || id < kPageChunks) {
-        kl[k_slot(id / CPRK, id % CPRK)] = stage_k[set][j];
-        vl[v_slot(id / 8, id % 8)] = stage_v[set][j];
+        kl[id] = stage_k[set][j];      // the cache keeps a page in the order LDS wants it
+        vl[id] = stage_v[set][j];
       }
     }
   };
@@ -917,13 +913,13 @@ __device__ __forceinline__ void rope_store(RopeShared &sh, const RopeItem &first
     if (it < n_q + kPerHead) {
       const uint4 packed = pack8(y);
       sh.k[d0 / 8] = packed;
-      *reinterpret_cast<uint4 *>(k_cache + base + size_t(pos % SB_PAGE) * HD + d0) = packed;
+      *reinterpret_cast<uint4 *>(k_cache + base + size_t(k_slot(pos % SB_PAGE, d0 / 8)) * 8) = packed;
     } else {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const bf16_t b = f32_to_bf16(y[i]);
         sh.v[d0 + i] = b;
-        v_cache[base + size_t(d0 + i) * SB_PAGE + pos % SB_PAGE] = b;
+        v_cache[base + sb_value_index(d0 + i, pos % SB_PAGE)] = b;
       }
     }
   }

@@ -52,9 +52,8 @@ attention_plain_kernel(TA *__restrict__ out, const TA *__restrict__ q, int q_str
     const bool visible = j >= lo && j <= pos;
     float s = neg_inf;
     if (visible) {
-      const TC *kr = kp + size_t(lane) * head_dim;
       float dot = 0.0f;
-      for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], ld_f(kr, d), dot);
+      for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], ld_f(kp, sb_key_index(lane, d, head_dim)), dot);
       s = dot * scale;
     }
     const float cm = wave_max(s);
@@ -70,7 +69,7 @@ attention_plain_kernel(TA *__restrict__ out, const TA *__restrict__ q, int q_str
       const int d = lane + 64 * i;
       if (d < head_dim) {
         float acc = o[i] * alpha;
-        for (int jj = j0; jj <= j1; ++jj) acc = fmaf(ps[jj], ld_f(vp, size_t(d) * SB_PAGE + jj), acc);
+        for (int jj = j0; jj <= j1; ++jj) acc = fmaf(ps[jj], ld_f(vp, sb_value_index(d, jj)), acc);
         o[i] = acc;
       }
     }

@@ -187,7 +187,7 @@ def ensure_plain_host(force: bool = False) -> str:
     lib, stamp = os.path.join(out_dir, "libsbplain.so"), os.path.join(out_dir, "libsbplain.so.stamp")
     src, header = os.path.join(HERE, "plain_host.cpp"), os.path.join(HERE, "plain_host.h")
     h = hashlib.sha256()
-    for path in (src, header):
+    for path in (src, header, os.path.join(HERE, "sb_hip.h")):
         with open(path, "rb") as f:
             h.update(f.read())
     want = h.hexdigest()

@@ -23,6 +23,8 @@
 #include <utility>
 #include <vector>
 
+#include "sb_hip.h"   // the cache's element order (sb_key_index, sb_value_index)
+
 namespace {
 constexpr int kPage = 64;   // SB_PAGE
 }
@@ -151,8 +153,8 @@ int sbp_rope_kv_store(float *q_out, const float *qkv, int row_stride, const floa
         const int kh = is_k ? h - heads_q : h - heads_q - heads_kv;
         const size_t base = (size_t(page) * heads_kv + kh) * kPage * head_dim;
         for (int d = 0; d < head_dim; ++d) {
-          if (is_k) k_cache[base + size_t(pos % kPage) * head_dim + d] = head[d];
-          else v_cache[base + size_t(d) * kPage + pos % kPage] = head[d];
+          if (is_k) k_cache[base + sb_key_index(pos % kPage, d, head_dim)] = head[d];
+          else v_cache[base + sb_value_index(d, pos % kPage)] = head[d];
         }
       }
     }
@@ -184,9 +186,9 @@ int sbp_attention(float *out, const float *q, int q_stride, const float *k_cache
         const int lp = j / kPage;
         const int page = lp < max_pages ? page_table[size_t(seq) * max_pages + lp] : -1;
         if (page < 0 || page >= n_pages_total) continue;
-        const float *kr = k_cache + ((size_t(page) * heads_kv + kh) * kPage + j % kPage) * head_dim;
+        const float *kp = k_cache + (size_t(page) * heads_kv + kh) * kPage * head_dim;
         double dot = 0.0;
-        for (int d = 0; d < head_dim; ++d) dot += double(qh[d]) * double(kr[d]);
+        for (int d = 0; d < head_dim; ++d) dot += double(qh[d]) * double(kp[sb_key_index(j % kPage, d, head_dim)]);
         score.push_back(float(dot) * scale);
         key.push_back(j);
       }
@@ -209,7 +211,7 @@ int sbp_attention(float *out, const float *q, int q_stride, const float *k_cache
           const int j = key[i];
           const int page = page_table[size_t(seq) * max_pages + j / kPage];
           acc += double(score[i] * inv) *
-                 double(v_cache[((size_t(page) * heads_kv + kh) * head_dim + d) * kPage + j % kPage]);
+                 double(v_cache[(size_t(page) * heads_kv + kh) * head_dim * kPage + sb_value_index(d, j % kPage)]);
         }
         o[d] = float(acc);
       }

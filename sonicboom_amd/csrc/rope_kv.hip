@@ -87,8 +87,7 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
   }
   const size_t head_step = size_t(SB_PAGE) * head_dim;  // from one kv head to the next within a page
   const size_t page_base = size_t(page_of_row) * heads_kv * head_step;
-  const size_t k_base = page_base + size_t(pos % SB_PAGE) * head_dim;   // keys   [position][d]
-  const size_t v_base = page_base + size_t(pos % SB_PAGE);              // values [d][position]
+  const int slot = pos % SB_PAGE;      // keys [slot][d], values [d][slot], in the cache's order of groups
 
   // The angle of pair i is the same for every head of the row: cosine and sine once per block,
   // the cosines by one half of the threads that take part, the sines by the other.
@@ -113,7 +112,7 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
       const int kh = head - heads_q - heads_kv;
 #pragma unroll 1
       for (int d = w; d < head_dim; d += per_head)
-        st_f(v_cache, v_base + kh * head_step + size_t(d) * SB_PAGE,
+        st_f(v_cache, page_base + kh * head_step + sb_value_index(d, slot),
              qkv_at<SLICES>(r, hoff + d, n_slices, slice_stride, bias));
       continue;
     }
@@ -132,14 +131,14 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
         st_f(qo, hoff + i, y0);
         st_f(qo, hoff + i + half, y1);
       } else {
-        st_f(k_cache, k_base + kh * head_step + i, y0);
-        st_f(k_cache, k_base + kh * head_step + i + half, y1);
+        st_f(k_cache, page_base + kh * head_step + sb_key_index(slot, i, head_dim), y0);
+        st_f(k_cache, page_base + kh * head_step + sb_key_index(slot, i + half, head_dim), y1);
       }
     } else {
       const int d = first_plain + (w - (rotate ? half : 0));
       const float v = qkv_at<SLICES>(r, hoff + d, n_slices, slice_stride, bias);
       if (is_q) st_f(qo, hoff + d, v);
-      else st_f(k_cache, k_base + kh * head_step + d, v);
+      else st_f(k_cache, page_base + kh * head_step + sb_key_index(slot, d, head_dim), v);
     }
   }
 }
@@ -187,8 +186,7 @@ rope_kv_rows_kernel(bf16_t *__restrict__ q_out, const TI *__restrict__ qkv, int 
   }
   const size_t head_step = size_t(SB_PAGE) * head_dim;
   const size_t page_base = size_t(page_of_row) * heads_kv * head_step;
-  const size_t k_base = page_base + size_t(pos % SB_PAGE) * head_dim;
-  const size_t v_base = page_base + size_t(pos % SB_PAGE);
+  const int slot = pos % SB_PAGE;
   __shared__ float cs[kMaxPairs], sn[kMaxPairs];
   for (int j = threadIdx.x; j < 2 * half; j += blockDim.x) {
     const int i = j < half ? j : j - half;
@@ -210,7 +208,11 @@ rope_kv_rows_kernel(bf16_t *__restrict__ q_out, const TI *__restrict__ qkv, int 
   for (int it = threadIdx.x; it < n_qk; it += blockDim.x) {
     const int head = it / per_head, w = it % per_head;
     const TI *src = r + size_t(head) * head_dim;
-    bf16_t *dst = head < heads_q ? qo + size_t(head) * head_dim : k_cache + k_base + size_t(head - heads_q) * head_step;
+    // a group of eight (d0 a multiple of 8) goes to the query row as it is, into the cache at the
+    // group's place in the cache's order
+    const bool is_q = head < heads_q;
+    bf16_t *dst = is_q ? qo + size_t(head) * head_dim : k_cache + page_base + size_t(head - heads_q) * head_step;
+    auto at = [&](int d0) { return is_q ? size_t(d0) : sb_key_index(slot, d0, head_dim); };
     if (w < pair_groups) {
       const int i0 = w * 8;
       float lo[8], hi[8], y0[8], y1[8];
@@ -218,13 +220,13 @@ rope_kv_rows_kernel(bf16_t *__restrict__ q_out, const TI *__restrict__ qkv, int 
       load_eight(hi, src + i0 + half);
 #pragma unroll
       for (int e = 0; e < 8; ++e) rotate_pair(lo[e], hi[e], cs[i0 + e], sn[i0 + e], y0[e], y1[e]);
-      *reinterpret_cast<uint4 *>(dst + i0) = pack(y0);
-      *reinterpret_cast<uint4 *>(dst + i0 + half) = pack(y1);
+      *reinterpret_cast<uint4 *>(dst + at(i0)) = pack(y0);
+      *reinterpret_cast<uint4 *>(dst + at(i0 + half)) = pack(y1);
     } else {
       const int d0 = 2 * half + (w - pair_groups) * 8;
       float v[8];
       load_eight(v, src + d0);
-      *reinterpret_cast<uint4 *>(dst + d0) = pack(v);
+      *reinterpret_cast<uint4 *>(dst + at(d0)) = pack(v);
     }
   }
   // values: eight elements a time, each to its own row of the transposed page
@@ -235,7 +237,7 @@ rope_kv_rows_kernel(bf16_t *__restrict__ q_out, const TI *__restrict__ qkv, int 
     float v[8];
     load_eight(v, r + size_t(heads_q + heads_kv + kh) * head_dim + d0);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) v_cache[v_base + kh * head_step + size_t(d0 + e) * SB_PAGE] = f32_to_bf16(v[e]);
+    for (int e = 0; e < 8; ++e) v_cache[page_base + kh * head_step + sb_value_index(d0 + e, slot)] = f32_to_bf16(v[e]);
   }
 }
 

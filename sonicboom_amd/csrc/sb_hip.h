@@ -14,7 +14,12 @@
  * [pages][kv_heads][SB_PAGE][head_dim], its values transposed,
  * [pages][kv_heads][head_dim][SB_PAGE]; `page_table` is int32 [batch][max_pages]
  * and maps the logical page (position / SB_PAGE) of a sequence to a physical
- * page, -1 for none.
+ * page, -1 for none.  Within a row of keys (one slot of a page) and within a row
+ * of values (one dimension over the page's slots) the groups of eight elements
+ * are kept in a permuted order: sb_key_index and sb_value_index below say where
+ * an element lies.  It is the order in which the matrix-core attention reads a
+ * page from LDS without bank conflicts, so a page goes from the cache into LDS
+ * as it lies.
  */
 #ifndef SONICBOOM_AMD_SB_HIP_H
 #define SONICBOOM_AMD_SB_HIP_H
@@ -27,6 +32,33 @@ extern "C" {
 #endif
 
 #define SB_PAGE 64
+
+#if defined(__HIPCC__)
+#define SB_INLINE static inline __host__ __device__
+#else
+#define SB_INLINE static inline
+#endif
+
+/* Offset (in elements) of element d of the key at slot `slot` (0..SB_PAGE-1)
+ * within a page's [SB_PAGE][head_dim] block of one head: group d / 8 of the row
+ * lies at group (d / 8) ^ s, s made of bits 0, 1, 3 and 4 of the slot, cut to the
+ * largest power of two (up to 16) that divides the row's number of groups.
+ * Head sizes that are no multiple of 16 keep the plain order. */
+SB_INLINE int sb_key_swizzle(int slot, int head_dim) {
+  if (head_dim % 16) return 0;
+  const int groups = head_dim / 8;
+  const int mask = groups % 16 == 0 ? 15 : (groups % 8 == 0 ? 7 : (groups % 4 == 0 ? 3 : 1));
+  return ((slot & 3) | (((slot >> 3) & 3) << 2)) & mask;
+}
+SB_INLINE size_t sb_key_index(int slot, int d, int head_dim) {
+  return (size_t)slot * (size_t)head_dim + (size_t)((((d >> 3) ^ sb_key_swizzle(slot, head_dim)) << 3) | (d & 7));
+}
+/* Offset of the value of dimension d at slot `slot` within a page's
+ * [head_dim][SB_PAGE] block of one head: group slot / 8 of the row lies at group
+ * (slot / 8) ^ ((d / 2) % 8). */
+SB_INLINE size_t sb_value_index(int d, int slot) {
+  return (size_t)d * SB_PAGE + (size_t)((((slot >> 3) ^ ((d >> 1) & 7)) << 3) | (slot & 7));
+}
 
 typedef enum sb_status {
   SB_OK = 0,

@@ -159,3 +159,28 @@ def test_groups_of_rows_beside_keys_and_values():
     assert [c.held_pages(i) for i in range(4)] == [4, 4, 2, 4]      # the window of 70 has let two pages go
     c.free_slot(s)
     assert [c.held_pages(i) for i in range(4)] == [0, 0, 0, 0]
+
+
+def test_the_caches_order_of_elements_is_a_permutation_of_every_row():
+    """cache.layout (the Python face of sb_key_index / sb_value_index): within a row the groups
+    of eight elements are permuted, nothing is lost or doubled, elements keep their place within
+    a group, head sizes that are no multiple of 16 keep the plain order, and the sixteen keys that
+    a matrix-core fragment read touches at once get sixteen different group offsets when the row
+    has that many groups."""
+    from sonicboom_amd.cache import layout
+    for hd in (8, 16, 24, 32, 48, 64, 80, 96, 112, 128, 144, 160, 192, 240, 256):
+        kp, vp = layout.key_positions(hd), layout.value_positions(hd)
+        assert kp.shape == (64, hd) and vp.shape == (hd, 64)
+        for j in range(64):
+            assert sorted(kp[j].tolist()) == list(range(hd))
+            assert (kp[j] % 8 == np.arange(hd) % 8).all()
+        for d in range(hd):
+            assert sorted(vp[d].tolist()) == list(range(64))
+            assert (vp[d] % 8 == np.arange(64) % 8).all()
+        if hd % 16:
+            assert (kp == np.arange(hd)[None, :]).all()
+    kp = layout.key_positions(128)
+    keys = [8 * a + i for a in range(4) for i in range(4)]                      # one score tile's rows
+    assert len({int(kp[j, 0]) // 8 for j in keys}) == 16
+    vp = layout.value_positions(128)
+    assert len({(int(vp[d, 0]) // 8, d % 2) for d in range(16)}) == 16           # sixteen rows: 8 offsets x 2 rows of 128 bytes

@@ -10,6 +10,7 @@ import torch
 
 from plain import qwen2_plain as P
 from plain import sampling_plain as SP
+from sonicboom_amd.cache import layout
 
 F32, BF16 = torch.float32, torch.bfloat16
 DEV = "cuda:0"
@@ -101,7 +102,21 @@ def test_host_twins_agree_with_the_plain_implementation():
     assert np.allclose(q, P.rope_neox(full[:, :hq * hd], pos, hd, 1e4), atol=1e-6)
     k_want = P.rope_neox(full[:, hq * hd:(hq + hkv) * hd], pos, hd, 1e4).reshape(5, hkv, hd)
     assert np.allclose(kc[2, :, 1, :], k_want[1], atol=1e-6) and np.allclose(kc[0, :, 6, :], k_want[3], atol=1e-6)
-    assert np.array_equal(vc[1, :, :, 0], full[4, (hq + hkv) * hd:].reshape(hkv, hd))
+    # (head size 8: rows of keys keep the plain order; rows of values never do)
+    assert np.array_equal(vc[1][:, np.arange(hd), layout.value_positions(hd)[:, 0]], full[4, (hq + hkv) * hd:].reshape(hkv, hd))
+    # a head size whose rows are kept in the cache's own order: what the twin (the C functions of
+    # sb_hip.h) stores is found where cache.layout (their Python face) says
+    hq2, hkv2, hd2 = 2, 2, 32
+    inv2 = np.exp(-2.0 * np.arange(hd2 // 2, dtype=np.float32) / hd2 * np.log(np.float32(1e4))).astype(np.float32)
+    qkv2 = f32(3, (hq2 + 2 * hkv2) * hd2, seed=18)
+    pos2, seq2, table2 = i32([5, 27, 64 + 40]), i32([0, 0, 0]), i32([[1, 0]])
+    _, kc2, vc2 = host_paged(lib, qkv2, None, inv2, None, hd2, pos2, seq2, table2, 2, hq2, hkv2, hd2)
+    k2 = P.rope_neox(qkv2[:, hq2 * hd2:(hq2 + hkv2) * hd2], pos2, hd2, 1e4).reshape(3, hkv2, hd2)
+    v2 = qkv2[:, (hq2 + hkv2) * hd2:].reshape(3, hkv2, hd2)
+    for r, (page, slot) in enumerate([(1, 5), (1, 27), (0, 40)]):
+        assert np.allclose(kc2[page, :, slot][:, layout.key_positions(hd2)[slot]], k2[r], atol=1e-6)
+        assert np.array_equal(vc2[page][:, np.arange(hd2), layout.value_positions(hd2)[:, slot]], v2[r])
+    assert not np.allclose(kc2[1, :, 27], k2[1], atol=1e-6)          # slot 27's groups are not in the plain order
     y = np.array([[1.0, 0.0, 2.0, 3.0] * 3], np.float32)
     quarter = np.full(2, math.pi / 2, np.float32)
     qq, _, _ = host_paged(lib, y, None, quarter, None, 4, i32([1]), i32([0]), i32([[0]]), 1, 1, 1, 4)

@@ -9,6 +9,7 @@ import torch
 
 from plain import qwen2_plain as plain
 from plain import sampling_plain
+from sonicboom_amd.cache import layout
 
 pytestmark = pytest.mark.gpu
 
@@ -394,7 +395,8 @@ def test_silu_mul_add_cast(dtype):
 
 def make_cache(n_pages, heads_kv, head_dim, dtype, fill=float("nan")):
     """Keys [pages, heads, 64, d] and values [pages, heads, d, 64], filled with NaN: whatever a
-    kernel reads beyond what was stored shows in its result."""
+    kernel reads beyond what was stored shows in its result.  Within a row the cache keeps its own
+    order of elements; the tests read and write through sonicboom_amd.cache.layout."""
     k = torch.full((n_pages, heads_kv, 64, head_dim), fill, dtype=dtype, device=DEV)
     v = torch.full((n_pages, heads_kv, head_dim, 64), fill, dtype=dtype, device=DEV)
     return k, v
@@ -429,8 +431,8 @@ def test_rope_kv_store(hq, hkv, hd, rot, dtype):
     close(q, want_q, what="q", **tol)
     for r in range(n):
         page = table[seq[r], pos[r] // 64]
-        got_k = kc[page, :, pos[r] % 64, :].reshape(-1)
-        got_v = vc[page, :, :, pos[r] % 64].reshape(-1)
+        got_k = layout.get_key(kc, int(page), int(pos[r]) % 64).reshape(-1)
+        got_v = layout.get_value(vc, int(page), int(pos[r]) % 64).reshape(-1)
         close(got_k, want_k[r], what=f"k row {r}", **tol)
         close(got_v, qkv[r, qw + kvw:].to(dtype).float(), atol=0, rtol=0, what=f"v row {r}")
     # nothing else was written
@@ -524,8 +526,8 @@ def fill_cache_from(keys, values, table, dtype):
     for s, (k, v) in enumerate(zip(keys, values)):
         for p in range(k.shape[0]):
             page = table[s, p // 64]
-            kc[page, :, p % 64, :] = k[p].to(dtype)
-            vc[page, :, :, p % 64] = v[p].to(dtype)
+            layout.put_key(kc, int(page), p % 64, k[p])
+            layout.put_value(vc, int(page), p % 64, v[p])
     return kc, vc
 
 
@@ -577,8 +579,8 @@ def attention_case(hq, hkv, hd, lens, rows_per_seq, window, seed=0):
     for s_, (k, v) in enumerate(zip(keys, vals)):
         for p in range(k.shape[0]):
             page = table[s_, p // 64]
-            kc[page, :, p % 64, :] = k[p].to(BF16)
-            vc[page, :, :, p % 64] = v[p].to(BF16)
+            layout.put_key(kc, int(page), p % 64, k[p])
+            layout.put_value(vc, int(page), p % 64, v[p])
     rows = [(s_, p) for s_, ps in enumerate(rows_per_seq) for p in ps]
     q = randn(len(rows), hq * hd, seed=seed + 7).to(BF16)
     scale = 1.0 / math.sqrt(hd)
@@ -817,10 +819,11 @@ def test_attention_decode_one_dominant_key_in_each_chunk(pages):
     with ops.attention_decode_pages_per_wave(hd, pages):
         for far in spots:
             page, slot = int(table[0, far // 64]), far % 64
-            before = kc[page, :, slot, 0].clone()
-            kc[page, :, slot, 0] = rise
+            at = int(layout.key_positions(hd)[slot, 0])          # where element 0 of that key lies
+            before = kc[page, :, slot, at].clone()
+            kc[page, :, slot, at] = rise
             got = ops.attention_decode_mfma(q.to(DEV), kc, vc, table.to(DEV), pos, hq, hkv, hd, scale, 0)
-            kc[page, :, slot, 0] = before
+            kc[page, :, slot, at] = before
             want = vals[far].repeat_interleave(group, dim=0).reshape(1, -1)
             close(got, want.numpy(), atol=2e-2, rtol=1e-2, what=f"dominant key at {far}, {pages} pages per wave")
 
