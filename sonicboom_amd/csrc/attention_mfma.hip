@@ -110,21 +110,33 @@ __device__ __forceinline__ int k_slot(int key, int chunk) { return key * CPRK + 
 // ... and of chunk `chunk` (8 keys) of value row d (sb_value_index).
 __device__ __forceinline__ int v_slot(int d, int chunk) { return d * 8 + (chunk ^ ((d >> 1) & 7)); }
 
+// The same for the fragments of a lane (row r = lane % 16, lane group g = lane / 16), written so
+// that few registers hold addresses.  The keys a lane reads are 32 half + 8 (r / 4) + 4 t + r % 4:
+// bits 0, 1, 3, 4 of every one of them are r's bits, so the permutation of its rows' chunks is
+// the same for all of them, and a key's chunk 4 ks + g lies at
+//   key_chunk(r, g, ks) + (32 half + 4 t) CPRK      (the second term a constant of the call).
+// Likewise the value rows 16 dt + r of a lane share (d / 2) % 8 = (r / 2) % 8:
+//   value_chunk(r, g, half) + 128 dt.
+__device__ __forceinline__ int key_chunk(int r, int g, int ks) {
+  const int key = 8 * (r >> 2) + (r & 3);            // the lane's key of half 0, score tile 0
+  return key * CPRK + ((4 * ks + g) ^ sb_key_swizzle(key, HD));
+}
+__device__ __forceinline__ int value_chunk(int r, int g, int half) { return r * 8 + ((4 * half + g) ^ ((r >> 1) & 7)); }
+
 __device__ __forceinline__ void load_half(HalfPage &hp, const bf16_t *__restrict__ kp,
                                           const bf16_t *__restrict__ vp, int half, int lane) {
   const int r = lane & 15, g = lane >> 4;
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    // A row r = 4 gg + i of score tile t is key 8 gg + 4 t + i of the 32
-    const int key = 32 * half + 8 * (r >> 2) + 4 * t + (r & 3);
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d = ks * 32 + g * 8;
+    const int at = key_chunk(r, g, d < HD ? ks : 0);
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int d = ks * 32 + g * 8;
-      hp.k[t][ks] = ld16(kp + size_t(k_slot(key, d < HD ? ks * 4 + g : 0)) * 8, d < HD);
-    }
+    for (int t = 0; t < 2; ++t)   // A row r = 4 gg + i of score tile t is key 8 gg + 4 t + i of the 32
+      hp.k[t][ks] = ld16(kp + size_t(at + (32 * half + 4 * t) * CPRK) * 8, d < HD);
   }
+  const int vat = value_chunk(r, g, half);
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) hp.v[dt] = ld16(vp + size_t(v_slot(dt * 16 + r, 4 * half + g)) * 8, true);
+  for (int dt = 0; dt < DT; ++dt) hp.v[dt] = ld16(vp + size_t(vat + 128 * dt) * 8, true);
 }
 
 // The same without a branch around any load (a branch makes the compiler wait for every load in
@@ -134,22 +146,18 @@ __device__ __forceinline__ void load_half_straight(HalfPage &hp, const bf16_t *_
                                                    const bf16_t *__restrict__ vp, int half, int lane) {
   const int r = lane & 15, g = lane >> 4;
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    const int key = 32 * half + 8 * (r >> 2) + 4 * t + (r & 3);
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d = ks * 32 + g * 8;
+    const int at = key_chunk(r, g, d < HD ? ks : 0);
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int d = ks * 32 + g * 8;
-      if ((ks + 1) * 32 <= HD) {
-        hp.k[t][ks] = *reinterpret_cast<const uint4 *>(kp + size_t(k_slot(key, ks * 4 + g)) * 8);
-      } else {
-        const uint4 v = *reinterpret_cast<const uint4 *>(kp + size_t(k_slot(key, d < HD ? ks * 4 + g : 0)) * 8);
-        hp.k[t][ks] = d < HD ? v : make_uint4(0u, 0u, 0u, 0u);
-      }
+    for (int t = 0; t < 2; ++t) {
+      const uint4 v = *reinterpret_cast<const uint4 *>(kp + size_t(at + (32 * half + 4 * t) * CPRK) * 8);
+      hp.k[t][ks] = ((ks + 1) * 32 <= HD || d < HD) ? v : make_uint4(0u, 0u, 0u, 0u);
     }
   }
+  const int vat = value_chunk(r, g, half);
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt)
-    hp.v[dt] = *reinterpret_cast<const uint4 *>(vp + size_t(v_slot(dt * 16 + r, 4 * half + g)) * 8);
+  for (int dt = 0; dt < DT; ++dt) hp.v[dt] = *reinterpret_cast<const uint4 *>(vp + size_t(vat + 128 * dt) * 8);
 }
 
 // 32 keys at absolute positions base .. base+31, their fragments in hp, for the wave's NC groups
@@ -272,16 +280,16 @@ __device__ __forceinline__ void load_q(bf16x8_t (&qf)[KS], const bf16_t *qrow, b
 __device__ __forceinline__ void load_half_lds(HalfPage &hp, const uint4 *kl, const uint4 *vl, int half, int lane) {
   const int r = lane & 15, g = lane >> 4;
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    const int key = 32 * half + 8 * (r >> 2) + 4 * t + (r & 3);
+  for (int ks = 0; ks < KS; ++ks) {
+    const int d = ks * 32 + g * 8;
+    const int at = key_chunk(r, g, d < HD ? ks : 0);
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const int d = ks * 32 + g * 8;
-      hp.k[t][ks] = d < HD ? kl[k_slot(key, ks * 4 + g)] : make_uint4(0u, 0u, 0u, 0u);
-    }
+    for (int t = 0; t < 2; ++t)
+      hp.k[t][ks] = d < HD ? kl[at + (32 * half + 4 * t) * CPRK] : make_uint4(0u, 0u, 0u, 0u);
   }
+  const int vat = value_chunk(r, g, half);
 #pragma unroll
-  for (int dt = 0; dt < DT; ++dt) hp.v[dt] = vl[v_slot(dt * 16 + r, 4 * half + g)];
+  for (int dt = 0; dt < DT; ++dt) hp.v[dt] = vl[vat + 128 * dt];
 }
 
 // One page (64 keys at page_pos ..) out of LDS for the wave's NC groups of 16 columns, the softmax
@@ -297,14 +305,12 @@ __device__ __forceinline__ void attend_page64(WaveState<NC> &st, const bf16x8_t 
   const int r = lane & 15, g = lane >> 4;
   auto read_k = [&](uint4 (&kf)[2][KS], int h) {
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      // A row r = 4 gg + i of score tile t is key 8 gg + 4 t + i of the 32
-      const int key = 32 * h + 8 * (r >> 2) + 4 * t + (r & 3);
+    for (int ks = 0; ks < KS; ++ks) {
+      const int d = ks * 32 + g * 8;
+      const int at = key_chunk(r, g, d < HD ? ks : 0);
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int d = ks * 32 + g * 8;
-        kf[t][ks] = d < HD ? kl[k_slot(key, ks * 4 + g)] : make_uint4(0u, 0u, 0u, 0u);
-      }
+      for (int t = 0; t < 2; ++t)   // A row r = 4 gg + i of score tile t is key 8 gg + 4 t + i of the 32
+        kf[t][ks] = d < HD ? kl[at + (32 * h + 4 * t) * CPRK] : make_uint4(0u, 0u, 0u, 0u);
     }
   };
   floatx4_t s[NC][2][2];      // [group][half][score tile]
@@ -334,7 +340,7 @@ __device__ __forceinline__ void attend_page64(WaveState<NC> &st, const bf16x8_t 
 #pragma unroll
     for (int dt = 0; dt < (PIN ? DT : 1); ++dt)
 #pragma unroll
-      for (int h = 0; h < 2; ++h) vf[dt][h] = vl[v_slot(dt * 16 + r, 4 * h + g)];
+      for (int h = 0; h < 2; ++h) vf[dt][h] = vl[value_chunk(r, g, h) + 128 * dt];
     __builtin_amdgcn_sched_barrier(0);
   } else {
 #pragma unroll
@@ -417,7 +423,7 @@ __device__ __forceinline__ void attend_page64(WaveState<NC> &st, const bf16x8_t 
     uint4 va[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
-      uint4 a = PIN ? vf[PIN ? dt : 0][h] : vl[v_slot(dt * 16 + r, 4 * h + g)];
+      uint4 a = PIN ? vf[PIN ? dt : 0][h] : vl[value_chunk(r, g, h) + 128 * dt];
       if (MASKED) {
         // values of keys outside [key_lo, key_hi] may be stale or never written: 0 * garbage must
         // not reach the accumulator
@@ -444,7 +450,8 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
   constexpr int kThreads = 64 * WAVES;
   constexpr int kStageLoads = (kPageChunks + kThreads - 1) / kThreads;
   extern __shared__ uint4 lds_pages[];               // [2 buffers][keys | values][kPageChunks]
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n_y = heads_kv * y_per_kv;
   const int tile = n_tiles - 1 - int(blockIdx.x) / n_y, by = int(blockIdx.x) % n_y;
   const int group = heads_q / heads_kv;
@@ -521,8 +528,74 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
   };
   using Set0 = std::integral_constant<int, 0>;
   using Set1 = std::integral_constant<int, 1>;
+  // Page pg out of LDS buffer buf, for a wave that has a head.
+  auto attend = [&](int pg, int buf) __attribute__((always_inline)) {
+    const uint4 *kl = lds_pages + buf * 2 * kPageChunks, *vl = kl + kPageChunks;
+    const int page_pos = pg * SB_PAGE;
+    if (HD > 128) {
+      // too many fragments for the registers at once: half a page at a time
+      HalfPage h;
+      if (!(page_pos > key_hi || page_pos + 31 < key_lo)) {
+        load_half_lds(h, kl, vl, 0, lane);
+        attend_half<NC>(st, qf, h, page_pos, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
+      }
+      if (!(page_pos + 32 > key_hi || page_pos + 63 < key_lo)) {
+        load_half_lds(h, kl, vl, 1, lane);
+        attend_half<NC>(st, qf, h, page_pos + 32, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
+      }
+    } else if (page_pos + SB_PAGE - 1 <= pos_first && page_pos >= lo_last) {
+      attend_page64<NC, false, WAVES == 4 && NC != 1>(st, qf, kl, vl, page_pos, col_pos, col_lo, key_lo, key_hi,
+                                                      scale_log2, lane);
+    } else {
+      attend_page64<NC, true, WAVES == 4 && NC != 1>(st, qf, kl, vl, page_pos, col_pos, col_lo, key_lo, key_hi,
+                                                     scale_log2, lane);
+    }
+  };
 
   int pg = next_valid(key_lo / SB_PAGE);                      // the page being multiplied
+  // Waves without a head (the block's last ones, when the kv head's group does not fill it) bring
+  // the pages in alone, straight into LDS (a load of 64 lanes x 16 bytes lands in 1 KB of
+  // consecutive LDS, and a page lies in the cache as LDS wants it): the waves that multiply then
+  // issue nothing for it, and a page comes through no registers.  While page p is multiplied out
+  // of one buffer, page p + 1 arrives in the other.
+  const int n_busy = min(head_tiles - yb * WAVES, WAVES), n_stagers = WAVES - n_busy;
+  if (n_stagers > 0) {
+    typedef __attribute__((address_space(3))) uint4 *lds_ptr_t;
+    constexpr int kWaveLoads = kPageChunks / 64;       // per page of keys, and of values
+    auto bring = [&](int pg_in, int buf_in) __attribute__((always_inline)) {
+      if (wave < n_busy) return;
+      const size_t off = (size_t(pt[pg_in]) * heads_kv + kvh) * SB_PAGE * HD;
+      const __amdgpu_buffer_rsrc_t rsrc_k = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<bf16_t *>(k_cache + off), 0, uint32_t(kPageChunks * 16), 0x00020000);
+      const __amdgpu_buffer_rsrc_t rsrc_v = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<bf16_t *>(v_cache + off), 0, uint32_t(kPageChunks * 16), 0x00020000);
+      for (int i = wave - n_busy; i < kWaveLoads; i += n_stagers) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_k, (lds_ptr_t)(lds_pages) + buf_in * 2 * kPageChunks + i * 64,
+                                                 16, lane * 16, i * 1024, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(
+            rsrc_v, (lds_ptr_t)(lds_pages) + buf_in * 2 * kPageChunks + kPageChunks + i * 64, 16, lane * 16, i * 1024,
+            0, 0);
+      }
+    };
+    // a wave's own loads have landed, and after the barrier everybody's (a bare barrier between
+    // two fences for the compiler: __syncthreads() says more than is needed)
+    auto landed = [&]() __attribute__((always_inline)) {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+    };
+    if (pg <= pg_hi) bring(pg, 0);
+    landed();
+    int buf = 0;
+    while (pg <= pg_hi) {
+      const int pg_next = next_valid(pg + 1);
+      if (pg_next <= pg_hi) bring(pg_next, buf ^ 1);
+      if (active) attend(pg, buf);
+      landed();
+      pg = pg_next;
+      buf ^= 1;
+    }
+  } else {
   int pg1 = pg <= pg_hi ? next_valid(pg + 1) : pg;            // the page after it
   if (pg <= pg_hi) issue(Set0{}, pg);
   if (pg1 <= pg_hi) issue(Set1{}, pg1);
@@ -536,28 +609,7 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
     using SetHeld = std::integral_constant<int, free_set ^ 1>;
     const int pg2 = pg1 <= pg_hi ? next_valid(pg1 + 1) : pg1;
     if (pg2 <= pg_hi) issue(SetFree{}, pg2);
-    if (active) {
-      const uint4 *kl = lds_pages + buf * 2 * kPageChunks, *vl = kl + kPageChunks;
-      const int page_pos = pg * SB_PAGE;
-      if (HD > 128) {
-        // too many fragments for the registers at once: half a page at a time
-        HalfPage h;
-        if (!(page_pos > key_hi || page_pos + 31 < key_lo)) {
-          load_half_lds(h, kl, vl, 0, lane);
-          attend_half<NC>(st, qf, h, page_pos, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
-        }
-        if (!(page_pos + 32 > key_hi || page_pos + 63 < key_lo)) {
-          load_half_lds(h, kl, vl, 1, lane);
-          attend_half<NC>(st, qf, h, page_pos + 32, col_pos, col_lo, key_lo, key_hi, scale_log2, lane);
-        }
-      } else if (page_pos + SB_PAGE - 1 <= pos_first && page_pos >= lo_last) {
-        attend_page64<NC, false, WAVES == 4 && NC != 1>(st, qf, kl, vl, page_pos, col_pos, col_lo, key_lo, key_hi,
-                                             scale_log2, lane);
-      } else {
-        attend_page64<NC, true, WAVES == 4 && NC != 1>(st, qf, kl, vl, page_pos, col_pos, col_lo, key_lo, key_hi,
-                                            scale_log2, lane);
-      }
-    }
+    if (active) attend(pg, buf);
     if (pg1 <= pg_hi) store(SetHeld{}, buf ^ 1);
     __syncthreads();
     pg = pg1;
@@ -568,6 +620,7 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
     step(Set0{});
     if (pg > pg_hi) break;
     step(Set1{});
+  }
   }
 #pragma unroll
   for (int c = 0; c < NC; ++c) {
