@@ -130,10 +130,14 @@ __device__ __forceinline__ uint64_t cand_key(float logit, float temperature, int
 }
 
 // The key of rank `want` (1 = largest) among the keys a block's threads hold in registers, PER per
-// thread: eight radix passes from the top byte down, each a histogram of the keys that share the
-// bytes found so far (one histogram per wave, then added up), and a look for the bucket that
-// holds the rank.  A key of 0 stands for "nothing" and lies below every real key; `want` must not
-// exceed the number of real keys.  Every thread of the block calls it and gets the same key.
+// thread: up to eight radix passes from the top byte down, each a histogram of the keys that share
+// the bytes found so far (one histogram per wave, then added up), and a look for the bucket that
+// holds the rank.  When that bucket holds exactly the keys still wanted, its lowest possible key
+// cuts as the key of the rank would, and the passes end there: with keys that differ in their
+// upper half (z) this is after four passes or fewer; the lower half (the id) only matters among
+// equal z at the cut.  A key of 0 stands for "nothing" and lies below every real key; `want` must
+// not exceed the number of real keys.  Every thread of the block calls it and gets the same key:
+// exactly `want` of the real keys are greater or equal.
 struct SelectShared {
   uint32_t hist[kSelWaves][256];
   uint32_t wave_total[4];
@@ -154,6 +158,7 @@ __device__ __forceinline__ uint64_t select_kth(const uint64_t (&mine)[PER], int 
     __syncthreads();
     const uint64_t prefix = sh.prefix;
     const uint32_t remaining = uint32_t(sh.remaining);
+    if (remaining == 0) break;          // (uniform) the cut is found
 #pragma unroll
     for (int j = 0; j < PER; ++j) {
       const uint64_t key = mine[j];
@@ -179,7 +184,8 @@ __device__ __forceinline__ uint64_t select_kth(const uint64_t (&mine)[PER], int 
       uint32_t above = suffix - mine_n;
       for (int wv = wave + 1; wv < 4; ++wv) above += sh.wave_total[wv];
       if (above < remaining && above + mine_n >= remaining) {
-        sh.remaining = int(remaining - above);
+        // the whole bucket is wanted: its lowest key cuts where the key of the rank would
+        sh.remaining = above + mine_n == remaining ? 0 : int(remaining - above);
         sh.prefix = prefix | (uint64_t(tid) << shift);
       }
     }
