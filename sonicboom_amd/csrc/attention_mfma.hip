@@ -557,19 +557,26 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
   // the pages in alone, straight into LDS (a load of 64 lanes x 16 bytes lands in 1 KB of
   // consecutive LDS, and a page lies in the cache as LDS wants it): the waves that multiply then
   // issue nothing for it, and a page comes through no registers.  While page p is multiplied out
-  // of one buffer, page p + 1 arrives in the other.
+  // of one buffer, page p + 1 arrives in the other.  Where every wave has a head, blocks of four
+  // waves with one head per wave, or with heads of more than 128, share these loads among all
+  // waves (measured against the path through registers below, 8,192 tokens, groups of 4: head
+  // size 64 5 % faster, 96 22 %, 128 10 %, 144 12 %, 192 2.4 times, 256 7 times, whose two sets of
+  // staging registers no longer fit; two and more heads per wave at head sizes up to 128, and eight
+  // waves, are 5 to 11 % slower with them and keep the registers).
+  constexpr bool kAllBring = WAVES == 4 && (NC == 1 || HD > 128);
   const int n_busy = min(head_tiles - yb * WAVES, WAVES), n_stagers = WAVES - n_busy;
-  if (n_stagers > 0) {
+  if (n_stagers > 0 || kAllBring) {
     typedef __attribute__((address_space(3))) uint4 *lds_ptr_t;
     constexpr int kWaveLoads = kPageChunks / 64;       // per page of keys, and of values
     auto bring = [&](int pg_in, int buf_in) __attribute__((always_inline)) {
-      if (wave < n_busy) return;
+      if (n_stagers > 0 && wave < n_busy) return;
+      const int first_load = n_stagers > 0 ? wave - n_busy : wave, step_load = n_stagers > 0 ? n_stagers : WAVES;
       const size_t off = (size_t(pt[pg_in]) * heads_kv + kvh) * SB_PAGE * HD;
       const __amdgpu_buffer_rsrc_t rsrc_k = __builtin_amdgcn_make_buffer_rsrc(
           const_cast<bf16_t *>(k_cache + off), 0, uint32_t(kPageChunks * 16), 0x00020000);
       const __amdgpu_buffer_rsrc_t rsrc_v = __builtin_amdgcn_make_buffer_rsrc(
           const_cast<bf16_t *>(v_cache + off), 0, uint32_t(kPageChunks * 16), 0x00020000);
-      for (int i = wave - n_busy; i < kWaveLoads; i += n_stagers) {
+      for (int i = first_load; i < kWaveLoads; i += step_load) {
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_k, (lds_ptr_t)(lds_pages) + buf_in * 2 * kPageChunks + i * 64,
                                                  16, lane * 16, i * 1024, 0, 0);
         __builtin_amdgcn_raw_ptr_buffer_load_lds(
@@ -1373,8 +1380,11 @@ int decode_launch(const char *who, void *out, const void *q, const RopeArgs &ra,
   (bf16_t *)out, part_o, part_ml, (const bf16_t *)q, ra, (const bf16_t *)k_cache, (const bf16_t *)v_cache, \
       page_table, max_pages, n_pages_total, row_pos, heads_q, heads_kv, n_chunks, scale *kLog2e, window
   if (ppw > 1) {
-    if (fused) attn_decode_long_kernel<true><<<grid, 256, 0, s>>>(SB_ARGS, ppw, n_seqs);
-    else attn_decode_long_kernel<false><<<grid, 256, 0, s>>>(SB_ARGS, ppw, n_seqs);
+    // (only head sizes up to 128 get here, and only they hold this kernel)
+    if constexpr (HD <= 128) {
+      if (fused) attn_decode_long_kernel<true><<<grid, 256, 0, s>>>(SB_ARGS, ppw, n_seqs);
+      else attn_decode_long_kernel<false><<<grid, 256, 0, s>>>(SB_ARGS, ppw, n_seqs);
+    }
   } else if ((long long)n_chunks * per_chunk <= 1536) {
     if (fused) attn_decode_kernel<true, true><<<grid, 256, 0, s>>>(SB_ARGS, n_seqs);
     else attn_decode_kernel<true, false><<<grid, 256, 0, s>>>(SB_ARGS, n_seqs);
