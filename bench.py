@@ -2,7 +2,7 @@
 MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
-                    [--sizes 7b|14b|72b] [--prompt T] [--context C] [--workload steady|mixed]
+                    [--sizes 0.5b|1.5b|3b|7b|14b|32b|72b] [--prompt T] [--context C] [--workload steady|mixed]
 
 A "step" is one decode step: every sequence of the batch goes on by one token (step function,
 greedy choice on the device, the token fed back).
@@ -40,9 +40,18 @@ CONFIG_14B = dict(CONFIG_7B, num_hidden_layers=48, hidden_size=5120, num_attenti
                   num_key_value_heads=8, intermediate_size=13824)
 CONFIG_72B = dict(CONFIG_7B, num_hidden_layers=80, hidden_size=8192, num_attention_heads=64,
                   num_key_value_heads=8, intermediate_size=29568)
-SIZES = {"7b": ("Qwen2.5-7B", CONFIG_7B), "14b": ("Qwen2.5-14B", CONFIG_14B), "72b": ("Qwen2.5-72B", CONFIG_72B)}
+CONFIG_32B = dict(CONFIG_14B, num_hidden_layers=64, intermediate_size=27648)
+# the family's small members: tied head, a vocabulary of 151,936
+CONFIG_05B = dict(CONFIG_7B, num_hidden_layers=24, hidden_size=896, num_attention_heads=14, num_key_value_heads=2,
+                  intermediate_size=4864, vocab_size=151936, tie_word_embeddings=True)
+CONFIG_15B = dict(CONFIG_05B, num_hidden_layers=28, hidden_size=1536, num_attention_heads=12, intermediate_size=8960)
+CONFIG_3B = dict(CONFIG_05B, num_hidden_layers=36, hidden_size=2048, num_attention_heads=16, intermediate_size=11008)
+SIZES = {"7b": ("Qwen2.5-7B", CONFIG_7B), "14b": ("Qwen2.5-14B", CONFIG_14B), "72b": ("Qwen2.5-72B", CONFIG_72B),
+         "32b": ("Qwen2.5-32B", CONFIG_32B), "0.5b": ("Qwen2.5-0.5B", CONFIG_05B), "1.5b": ("Qwen2.5-1.5B", CONFIG_15B),
+         "3b": ("Qwen2.5-3B", CONFIG_3B)}
 # the mixed workloads: prompts, shortest, longest, greedy steps, cache tokens a sequence
-MIXED = {"14b": (16, 256, 4096, 256, 8192), "72b": (8, 512, 2048, 128, 4096), "7b": (16, 256, 4096, 256, 8192)}
+MIXED = {"72b": (8, 512, 2048, 128, 4096), "32b": (8, 512, 2048, 128, 4096)}
+MIXED_DEFAULT = (16, 256, 4096, 256, 8192)
 CONTEXT = 4096
 PROMPT = 2048
 
@@ -255,7 +264,7 @@ def main() -> int:
             "layers_of_configuration": full_layers, "hidden_size": m["d"], "num_attention_heads": m["hq"],
             "num_key_value_heads": m["hkv"], "head_dim": m["hd"], "intermediate_size": m["ff"],
             "vocab_size": m["v"], "rope_theta": cfg["rope_theta"], "rms_norm_eps": cfg["rms_norm_eps"],
-            "tie_word_embeddings": False, "parallelism": "single GPU", "decode_graph": not a.no_graph,
+            "tie_word_embeddings": bool(cfg["tie_word_embeddings"]), "parallelism": "single GPU", "decode_graph": not a.no_graph,
         }
         c.update(more)
         return c
@@ -272,7 +281,7 @@ def main() -> int:
 
     # ------------------------------------------------------------------------------------------
     if a.workload == "mixed":
-        n_prompts, shortest, longest, n_steps, per_seq = MIXED[a.sizes]
+        n_prompts, shortest, longest, n_steps, per_seq = MIXED.get(a.sizes, MIXED_DEFAULT)
         lengths = [int(n) for n in rng.integers(shortest, longest + 1, size=n_prompts)]
         prompts = random_prompts(lengths)
         engine = Engine(model, max_tokens=per_seq * n_prompts)
