@@ -726,23 +726,26 @@ int launch_direct(const Args &a, long long blocks, int round_blocks, hipStream_t
 
 // Tile shapes the launcher chooses from: rows x columns of Y per block.
 struct Shape { int bm, bn; };
-constexpr Shape kShapes[4] = {{128, 128}, {256, 128}, {256, 256}, {128, 256}};
+constexpr Shape kShapes[5] = {{128, 128}, {256, 128}, {256, 256}, {128, 256}, {192, 256}};
 
 // The tile shape for a problem: the one with the best product of three factors.  How fast the
 // shape's kernel runs on a full grid, relative to 128 x 128 (measured on MI355X at 2,048 to 16,384
 // rows of Qwen2.5-7B's four products: the 256 x 256 kernel, which loads straight into LDS, reaches
-// 1.19 to 1.31 PFLOP/s where the 128 x 128 one reaches 0.73 to 0.98); the share of the tiles' rows
+// 1.19 to 1.31 PFLOP/s where the 128 x 128 one reaches 0.73 to 0.98; the same kernel with tiles of
+// 192 rows takes 0.84 of the time for 0.75 of the outputs); the share of the tiles' rows
 // that are rows of Y; and the share of the last round of tiles over the CUs that is filled.
 // Some of what this decides at 2,048 rows: the output product (3,584 x 3,584) takes 256 x 128
-// (224 tiles, one round: 65 us against 92 with 112 tiles of 256 x 256), the QKV product 256 x 256
-// (144 tiles: 86 us against 92 with 128 x 128), the down product 256 x 128 (274 against 403 us);
-// from 4,096 rows on nearly everything takes 256 x 256.
-int pick_shape(int n_rows, int n_out, int n_in, int gated) {
+// (224 tiles, one round: 65 us against 92 with 112 tiles of 256 x 256), the QKV product 192 x 256
+// (198 tiles: 63 us against 73 with 144 of 256 x 256), the down product 256 x 128 (274 against 403 us);
+// from 4,096 rows on nearly everything takes 256 x 256.  `direct_ok`: the kernel that loads
+// straight into LDS takes these operands (the 192 x 256 shape has no other).
+int pick_shape(int n_rows, int n_out, int n_in, int gated, bool direct_ok) {
   (void)n_in;
-  const double speed[3] = {1.0, gated ? 1.0 : 1.05, gated ? 1.25 : 1.35};
+  const double speed[5] = {1.0, gated ? 1.0 : 1.05, gated ? 1.25 : 1.35, 0.0, (gated ? 1.25 : 1.35) * 0.89};
   double best = 0;
   int pick = 0;
-  for (int v = 0; v < 3; ++v) {
+  for (int v = 0; v < 5; ++v) {
+    if (v == 3 || (v == 4 && !direct_ok)) continue;
     const int bm = kShapes[v].bm, bn = gated ? kShapes[v].bn / 2 : kShapes[v].bn;
     const long long tiles_m = (n_rows + bm - 1) / bm, tiles_n = (n_out + bn - 1) / bn;
     const long long tiles = tiles_m * tiles_n, rounds = (tiles + kCus - 1) / kCus;
@@ -777,12 +780,13 @@ extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void
   a.n_rows = n_rows; a.n_out = n_out; a.n_in = n_in; a.gated = gated;
   a.partial = nullptr; a.stages_per_slice = 0;
   a.vec4 = n_out % 4 == 0 && (reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(resid)) % 16 == 0;
-  int variant = pick_shape(n_rows, n_out, n_in, a.gated);
+  const bool direct_ok = packed && n_in % 64 == 0;
+  int variant = pick_shape(n_rows, n_out, n_in, a.gated, direct_ok);
   // a test's or a measurement's choice: the shape (0..3) + 16 * the path (0: the launcher's, 1:
   // through registers, 2: straight into LDS)
   int path = 0;
   if (tile_shape >= 0) {
-    SB_REQUIRE((tile_shape & 15) < 4 && (tile_shape >> 4) < 4, "sb_gemm_mfma_bf16: unknown tile shape %d", tile_shape);
+    SB_REQUIRE((tile_shape & 15) < 5 && (tile_shape >> 4) < 4, "sb_gemm_mfma_bf16: unknown tile shape %d", tile_shape);
     variant = tile_shape & 15;
     path = tile_shape >> 4;
   }
@@ -804,20 +808,20 @@ extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void
   a.w_tiles = (n_out + 15) / 16;
   a.w_steps = (n_in + 31) / 32;
   int rc;
-  const bool direct_ok = packed && n_in % 64 == 0;
   SB_SUPPORT(path < 2 || direct_ok, "sb_gemm_mfma_bf16: the direct path takes packed weights and an inner size in 64s");
   // left to itself only the 256 x 256 shape goes straight into LDS: the smaller tiles' stages are too
   // short for loads that run one stage ahead, and the register path, which runs two ahead, is
   // faster there (128 x 128, QKV product at 2,048 rows: 92 against 128 us)
-  const bool direct = path >= 2 || (path == 0 && direct_ok && variant == 2);
-  SB_SUPPORT(variant != 3 || direct, "sb_gemm_mfma_bf16: the 128 x 256 shape exists on the direct path only");
+  const bool direct = path >= 2 || (path == 0 && direct_ok && (variant == 2 || variant == 4));
+  SB_SUPPORT(variant < 3 || direct, "sb_gemm_mfma_bf16: the shapes 128 x 256 and 192 x 256 exist on the direct path only");
   if (direct) {
     // path 3 (a measurement's): the 256 x 256 shape with a block for every tile
     if (variant == 0) rc = launch_direct<4, 2, 64, 2, false>(a, blocks, 0, s);
     else if (variant == 1) rc = launch_direct<8, 2, 64, 2, false>(a, blocks, 0, s);
     else if (variant == 2 && path == 3) rc = launch_direct<8, 4, 64, 2, false>(a, blocks, 0, s);
     else if (variant == 2) rc = launch_direct<8, 4, 64, 2, true>(a, blocks, kCus, s);     // 128 KB of LDS: a block a CU
-    else rc = launch_direct<4, 4, 64, 2, false>(a, blocks, 0, s);
+    else if (variant == 3) rc = launch_direct<4, 4, 64, 2, false>(a, blocks, 0, s);
+    else rc = launch_direct<6, 4, 64, 2, true>(a, blocks, kCus, s);
   } else {
     if (variant == 0) rc = launch<2, 2, 64, 2, true>(a, blocks, packed, s);
     else if (variant == 1) rc = launch<4, 2, 64, 2, false>(a, blocks, packed, s);

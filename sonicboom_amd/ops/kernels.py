@@ -527,10 +527,10 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], re
 @contextlib.contextmanager
 def gemm_tile_shape(shape: Optional[int], path: Optional[str] = None):
     """For tests and measurements: inside the block the tiled products of this thread use tile
-    shape ``shape`` (0: 128 x 128, 1: 256 x 128, 2: 256 x 256, 3: 128 x 256 outputs per block)
-    instead of choosing one, and with ``path`` the kernel that stages tiles through "registers"
-    or the one that loads them "direct" into LDS (packed weights, inner size in 64s; the only one
-    with shape 3)."""
+    shape ``shape`` (0: 128 x 128, 1: 256 x 128, 2: 256 x 256, 3: 128 x 256, 4: 192 x 256 outputs per
+    block) instead of choosing one, and with ``path`` the kernel that stages tiles through
+    "registers" or the one that loads them "direct" into LDS (packed weights, inner size in 64s;
+    the only one with shapes 3 and 4)."""
     paths = {None: 0, "registers": 1, "direct": 2, "direct, a block a tile": 3}
     if path not in paths:
         raise ValueError(f"unknown path {path!r}")

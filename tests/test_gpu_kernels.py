@@ -216,7 +216,7 @@ def test_gemm_bf16_every_tile_shape(shape, packed, t, n, k):
         close(got, g / (1.0 + torch.exp(-g)) * u, atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"gated shape {shape}")
 
 
-@pytest.mark.parametrize("shape, path", [(0, "direct"), (1, "direct"), (2, "direct"), (3, "direct"),
+@pytest.mark.parametrize("shape, path", [(0, "direct"), (1, "direct"), (2, "direct"), (3, "direct"), (4, "direct"),
                                          (2, "direct, a block a tile"), (0, "registers"), (2, "registers")])
 @pytest.mark.parametrize("t, n, k", [(65, 100, 64), (300, 226, 192), (520, 264, 128), (257, 1001, 448), (130, 72, 2368)])
 def test_gemm_bf16_every_path(shape, path, t, n, k):
@@ -252,15 +252,16 @@ def test_gemm_bf16_blocks_that_go_from_tile_to_tile():
     x, w = randn(t, k, dtype=BF16), randn(n, k, dtype=BF16, scale=0.05)
     want = ref_gemm(x, w, None, None)
     wd = w.to(DEV)
-    for path in ("direct", "direct, a block a tile"):
-        with ops.gemm_tile_shape(2, path):
+    # (tiles of 192 rows: 23 x 17 = 391)
+    for shape, path in ((2, "direct"), (2, "direct, a block a tile"), (4, "direct")):
+        with ops.gemm_tile_shape(shape, path):
             got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(wd), None, None, F32, packed_shape=(n, k))
-            close(got, want, atol=3e-5 * math.sqrt(k), rtol=1e-5, what=path)
+            close(got, want, atol=3e-5 * math.sqrt(k), rtol=1e-5, what=f"{shape} {path}")
             inner = n // 2
             g, u = want[:, :inner].double(), want[:, inner:2 * inner].double()
             got = ops.gemm_bf16(x.to(DEV), ops.pack_weight(wd[:2 * inner].contiguous(), True), None, None, F32,
                                 gated=True, packed_shape=(2 * inner, k))
-            close(got, g / (1.0 + torch.exp(-g)) * u, atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"gated {path}")
+            close(got, g / (1.0 + torch.exp(-g)) * u, atol=1e-4 * math.sqrt(k), rtol=1e-4, what=f"gated {shape} {path}")
 
 
 def test_gemm_bf16_direct_path_refuses_what_it_cannot_take():
