@@ -217,6 +217,7 @@ extern "C" int sb_reduce_resid_norm(void *y, int y_dtype, float *x, const float 
 #define SB_GO(TO, KEEP)                          \
   do {                                           \
     if (n_slices == 1) SB_GO2(TO, KEEP, 1);      \
+    else if (n_slices == 2) SB_GO2(TO, KEEP, 2); \
     else if (n_slices <= 4) SB_GO2(TO, KEEP, 4); \
     else if (n_slices == 5) SB_GO2(TO, KEEP, 5); \
     else SB_GO2(TO, KEEP, kMaxSlices);           \

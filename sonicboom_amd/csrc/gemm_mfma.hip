@@ -739,7 +739,7 @@ constexpr Shape kShapes[5] = {{128, 128}, {256, 128}, {256, 256}, {128, 256}, {1
 // (198 tiles: 63 us against 73 with 144 of 256 x 256), the down product 256 x 128 (274 against 403 us);
 // from 4,096 rows on nearly everything takes 256 x 256.  `direct_ok`: the kernel that loads
 // straight into LDS takes these operands (the 192 x 256 shape has no other).
-int pick_shape(int n_rows, int n_out, int n_in, int gated, bool direct_ok) {
+int pick_shape(int n_rows, int n_out, int n_in, int gated, bool direct_ok, double *score_out = nullptr) {
   (void)n_in;
   const double speed[5] = {1.0, gated ? 1.0 : 1.05, gated ? 1.25 : 1.35, 0.0, (gated ? 1.25 : 1.35) * 0.89};
   double best = 0;
@@ -752,6 +752,7 @@ int pick_shape(int n_rows, int n_out, int n_in, int gated, bool direct_ok) {
     const double score = speed[v] * (double(n_rows) / double(tiles_m * bm)) * (double(tiles) / double(rounds * kCus));
     if (score > best) { best = score; pick = v; }
   }
+  if (score_out) *score_out = best;
   return pick;
 }
 
@@ -832,26 +833,70 @@ extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void
 }
 
 namespace {
-// K slices of the partial form: enough blocks for the GPU (one 128 x 128 tile per CU and slice),
-// every slice at least four stages of 64 long, at most the eight that the consumers add.
-int partial_slices(int n_rows, int n_out, int n_in) {
+// K slices of the partial form, and the tiles that multiply them.  Few rows: enough blocks for
+// the GPU (one 128 x 128 tile per CU and slice), every slice at least four stages of 64 long, at
+// most the eight that the consumers add.  Where that gives one slice, a problem with few tiles
+// of 256 x 256 (a prompt of one or two thousand rows against a matrix a few thousand wide) may
+// still be faster with those tiles, loaded straight into LDS, and K cut so that the tiles and
+// slices together make one round over the CUs.  Both ways are priced in microseconds from
+// what was measured on MI355X with the 7B products at 768 to 2,304 rows: a shape's tile takes
+// 2 bm bn K flops at its kernel's rate on a full GPU (pick_shape's speeds, 1 standing for 0.93
+// PFLOP/s over 256 CUs); a round that leaves CUs idle runs faster (0.72 of the time with up to 170
+// blocks, rising to 1 at 256: the chip's clock follows its load); a whole product costs 14 us
+// beside its tiles and a cut one 6; the consumer's pass over the additional slices moves
+// (2 slices - 2) x the result's bytes at 4 TB/s.  The cut is taken when it comes out under 0.92 of
+// the best whole product.  Measured, whole + norm against cut + the pass that adds the slices, the
+// residual and the norm: down (3,584 x 18,944) at 1,280 rows 237 against 152 us, at 2,048 rows 272
+// against 247; output (3,584 x 3,584) at 1,280 rows 69 against 52.
+struct PartialPlan { int slices; bool big; };
+double load_factor(long long blocks) { return blocks <= 170 ? 0.72 : 0.72 + 0.28 * double(blocks - 170) / 86.0; }
+PartialPlan partial_plan(int n_rows, int n_out, int n_in, bool direct_ok) {
   const long long tiles = (long long)((n_rows + 127) / 128) * ((n_out + 127) / 128);
   const int n_k = (n_in + 63) / 64;
   long long s = (224 + tiles - 1) / tiles;
   if (s > n_k / 4) s = n_k / 4;
   if (s > 8) s = 8;
   if (s < 1) s = 1;
+  const long long big = (long long)((n_rows + 255) / 256) * ((n_out + 255) / 256);
+  const long long big_grid = (big + kXcds - 1) / kXcds * kXcds;       // the grid is padded to whole eights
+  if (s == 1 && direct_ok && 2 * big_grid <= kCus) {
+    const double per_cu = 0.93e9 / kCus;                               // flops per microsecond at speed 1
+    const double speed[5] = {1.0, 1.05, 1.35, 0.0, 1.35 * 0.89};
+    double t_whole = 0;
+    for (int v = 0; v < 5; ++v) {
+      if (v == 3) continue;
+      const int bm = kShapes[v].bm, bn = kShapes[v].bn;
+      const long long n_tiles = (long long)((n_rows + bm - 1) / bm) * ((n_out + bn - 1) / bn);
+      const long long rounds = (n_tiles + kCus - 1) / kCus, last = n_tiles - (rounds - 1) * kCus;
+      const double t = 2.0 * bm * bn * double(n_in) / (speed[v] * per_cu) * (double(rounds - 1) + load_factor(last)) + 14.0;
+      if (v == 0 || t < t_whole) t_whole = t;
+    }
+    double t_best = 0;
+    long long s_best = 0;
+    for (long long s2 = 2; s2 <= 8 && s2 * big_grid <= kCus && s2 <= n_k / 4; ++s2) {
+      const int per = int((n_k + s2 - 1) / s2);
+      const double t = 2.0 * 256 * 256 * (64.0 * per) / (speed[2] * per_cu) * load_factor(s2 * big_grid) + 6.0 +
+                       (2.0 * s2 - 2.0) * n_rows * double(n_out) * 4.0 / 4e6;
+      if (s_best == 0 || t < t_best) t_best = t, s_best = s2;
+    }
+    if (s_best && t_best < 0.92 * t_whole) {
+      const int per = int((n_k + s_best - 1) / s_best);
+      return {(n_k + per - 1) / per, true};
+    }
+  }
   const int per = int((n_k + s - 1) / s);
-  return (n_k + per - 1) / per;
+  return {(n_k + per - 1) / per, false};
 }
 }  // namespace
 
 // Slices sb_gemm_mfma_partial_bf16 writes for these sizes.
-extern "C" int sb_gemm_mfma_slices(int n_rows, int n_out, int n_in) { return partial_slices(n_rows, n_out, n_in); }
+extern "C" int sb_gemm_mfma_slices(int n_rows, int n_out, int n_in, int packed) {
+  return partial_plan(n_rows, n_out, n_in, packed && n_in % 64 == 0).slices;
+}
 
 // The raw product X W^T in K slices: partial float [slices][n_rows][n_out], for a consumer that
 // adds the slices itself.  For few rows against a narrow, long matrix, where one slice would not
-// give the GPU enough tiles.  128 x 128 tiles.
+// give the GPU enough tiles.  128 x 128 tiles, or 256 x 256 (see partial_plan).
 extern "C" int sb_gemm_mfma_partial_bf16(float *partial, const void *x, const void *w, int n_rows, int n_out,
                                          int n_in, int packed, void *stream) {
   SB_REQUIRE(partial && x && w, "sb_gemm_mfma_partial_bf16: null pointer");
@@ -865,8 +910,10 @@ extern "C" int sb_gemm_mfma_partial_bf16(float *partial, const void *x, const vo
   a.y = nullptr; a.y_dtype = SB_F32; a.x = (const bf16_t *)x; a.w = (const bf16_t *)w;
   a.bias = nullptr; a.bias_dtype = 0; a.resid = nullptr;
   a.n_rows = n_rows; a.n_out = n_out; a.n_in = n_in; a.gated = 0;
-  a.tiles_m = (n_rows + 127) / 128;
-  a.tiles_n = (n_out + 127) / 128;
+  const PartialPlan plan = partial_plan(n_rows, n_out, n_in, packed && n_in % 64 == 0);
+  const int tile = plan.big ? 256 : 128;
+  a.tiles_m = (n_rows + tile - 1) / tile;
+  a.tiles_n = (n_out + tile - 1) / tile;
   const long long blocks = (long long)a.tiles_m * a.tiles_n;
   SB_SUPPORT(blocks <= 0x7fffffffLL, "sb_gemm_mfma_partial_bf16: too many tiles");
   const unsigned long long w_rows = (unsigned long long)((n_out + 15) / 16 * 16);
@@ -877,12 +924,13 @@ extern "C" int sb_gemm_mfma_partial_bf16(float *partial, const void *x, const vo
              "sb_gemm_mfma_partial_bf16: an operand of 4 GiB or more");
   a.w_tiles = (n_out + 15) / 16;
   a.w_steps = (n_in + 31) / 32;
-  const int slices = partial_slices(n_rows, n_out, n_in);
+  const int slices = plan.slices;
   const int n_k = (n_in + 63) / 64;
   a.partial = partial;
   a.vec4 = n_out % 4 == 0 && reinterpret_cast<uintptr_t>(partial) % 16 == 0;
   a.stages_per_slice = (n_k + slices - 1) / slices;
-  const int rc = launch<2, 2, 64, 2, true>(a, blocks, packed, (hipStream_t)stream);
+  const int rc = plan.big ? launch_direct_one<8, 4, 64, 2, 0, false>(a, blocks, 0, (hipStream_t)stream)
+                          : launch<2, 2, 64, 2, true>(a, blocks, packed, (hipStream_t)stream);
   if (rc != SB_OK) return rc;
   return sb::check_launch("sb_gemm_mfma_partial_bf16");
 }

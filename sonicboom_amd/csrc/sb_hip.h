@@ -239,7 +239,7 @@ int sb_gemm_stream_partial_bf16(float *partial, const void *x, const void *w, in
 int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void *w, const void *bias,   /* tiled */
                       int bias_dtype, const float *resid, int n_rows, int n_out, int n_in, int gated,
                       int packed, int tile_shape, void *stream);
-int sb_gemm_mfma_slices(int n_rows, int n_out, int n_in);
+int sb_gemm_mfma_slices(int n_rows, int n_out, int n_in, int packed);
 int sb_gemm_mfma_partial_bf16(float *partial, const void *x, const void *w, int n_rows, int n_out,
                               int n_in, int packed, void *stream);
 

@@ -381,8 +381,9 @@ def gemm_bf16_partial(x: torch.Tensor, w: torch.Tensor, packed_shape=None) -> Op
     Packed weights, up to 64 rows: the kernel whose waves split the output features and share
     the rows through LDS, with K cut over the grid so that the blocks fill the GPU.
     Packed weights, more rows: the tiled kernel with K cut over the grid, as long as the cut gives
-    more than one slice (a narrow matrix and up to a few hundred rows; one slice would leave most
-    of the GPU without a tile).  Row-major weights, up to 64 rows: the kernel whose waves split K.  None when
+    more than one slice (a narrow matrix and up to a few hundred rows, where one slice would leave
+    most of the GPU without a tile; or a thousand or two, where tiles of 256 x 256 with K cut in
+    two to four beat the whole product in smaller tiles).  Row-major weights, up to 64 rows: the kernel whose waves split K.  None when
     none applies: the caller then takes the whole product."""
     _dev(x, w)
     if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or x.dim() != 2:
@@ -401,7 +402,7 @@ def gemm_bf16_partial(x: torch.Tensor, w: torch.Tensor, packed_shape=None) -> Op
         check(lib.sb_gemm_stream_partial_bf16(_p(partial), _p(x), _p(w), t, n, k, _hints.stream, _stream()))
         return partial
     if packed_shape is not None and (t > SKINNY_MAX_ROWS or which == "tiled"):
-        slices = lib.sb_gemm_mfma_slices(t, n, k)
+        slices = lib.sb_gemm_mfma_slices(t, n, k, 1)
         if slices > 1 or t <= SKINNY_MAX_ROWS:
             partial = torch.empty((slices, t, n), dtype=torch.float32, device=x.device)
             check(lib.sb_gemm_mfma_partial_bf16(_p(partial), _p(x), _p(w), t, n, k, 1, _stream()))

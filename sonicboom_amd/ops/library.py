@@ -47,7 +47,7 @@ _OPTIONAL_SIGNATURES = {
     "sb_gemm_stream_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _P],
     "sb_gemm_stream_slices": [_I, _I, _I, _I],
     "sb_gemm_stream_partial_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
-    "sb_gemm_mfma_slices": [_I, _I, _I],
+    "sb_gemm_mfma_slices": [_I, _I, _I, _I],
     "sb_gemm_mfma_partial_bf16": [_P, _P, _P, _I, _I, _I, _I, _P],
 }
 _ATTN_SIGNATURES = {

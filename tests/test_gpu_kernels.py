@@ -348,6 +348,34 @@ def test_gemm_bf16_partial_slices_add_up(t, n, k, packed):
         close(rd, ref_gemm(x, w, bias, resid), atol=3e-5 * math.sqrt(k), rtol=1e-5, what="slices + bias + residual")
 
 
+def test_gemm_bf16_partial_in_big_tiles():
+    """Two thousand rows against a narrow matrix with a long inner size: 56 tiles of 256 x 256 with
+    K cut in four fill the GPU where 224 tiles of 128 x 128 would multiply whole.  The slices add
+    up to the product (sampled rows against float64, all of it against the whole product), and
+    the pass that adds them gives product + bias + residual and the norm of that."""
+    from sonicboom_amd import ops
+    t, n, k = 2048, 1792, 18944
+    x, w = randn(t, k, dtype=BF16), randn(n, k, dtype=BF16, scale=0.02)
+    xd, wp = x.to(DEV), ops.pack_weight(w.to(DEV))
+    partial = ops.gemm_bf16_partial(xd, wp, packed_shape=(n, k))
+    assert partial is not None and tuple(partial.shape) == (4, t, n)
+    total = partial.double().sum(0)
+    rows = [0, 1, 255, 256, 1000, 2047]
+    close(total[rows], ref_gemm(x[rows], w), atol=3e-5 * math.sqrt(k), rtol=1e-5, what="sampled rows")
+    whole = ops.gemm_bf16(xd, wp, None, None, F32, packed_shape=(n, k))
+    close(total, whole.double().cpu(), atol=3e-5 * math.sqrt(k), rtol=1e-5, what="against the whole product")
+    resid, bias, nw = randn(t, n), randn(n, scale=0.1), 1.0 + randn(n, scale=0.1)
+    rd = resid.to(DEV)
+    normed = ops.reduce_resid_norm(partial, bias.to(DEV), rd, nw.to(DEV), 1e-5, F32)
+    want = whole.double().cpu() + bias.double() + resid.double()
+    close(rd, want, atol=3e-5 * math.sqrt(k), rtol=1e-5, what="slices + bias + residual")
+    want_n = want / torch.sqrt((want * want).mean(-1, keepdim=True) + 1e-5) * nw.double()
+    close(normed, want_n, atol=1e-4, rtol=1e-4, what="and the norm")
+    # a short inner size: the pass over four slices would cost more than the cut saves
+    assert ops.gemm_bf16_partial(xd[:, :1024].contiguous(), ops.pack_weight(w[:, :1024].contiguous().to(DEV)),
+                                 packed_shape=(n, 1024)) is None
+
+
 @pytest.mark.parametrize("which, waves, slices", [("stream", 4, 1), ("stream", 5, 3), ("stream", 7, 8), ("stream", 8, 5),
                                                   ("tiled", 0, 0), ("skinny", 0, 0)])
 @pytest.mark.parametrize("t", [3, 16, 33, 64])
