@@ -562,8 +562,9 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
   // waves (measured against the path through registers below, 8,192 tokens, groups of 4: head
   // size 64 5 % faster, 96 22 %, 128 10 %, 144 12 %, 192 2.4 times, 256 7 times, whose two sets of
   // staging registers no longer fit; two and more heads per wave at head sizes up to 128, and eight
-  // waves, are 5 to 11 % slower with them and keep the registers).
-  constexpr bool kAllBring = WAVES == 4 && (NC == 1 || HD > 128);
+  // waves at those head sizes, are 5 to 11 % slower with them and keep the registers; eight waves
+  // with bigger heads have no registers to keep pages in).
+  constexpr bool kAllBring = (WAVES == 4 && (NC == 1 || HD > 128)) || (WAVES == 8 && HD > 128);
   const int n_busy = min(head_tiles - yb * WAVES, WAVES), n_stagers = WAVES - n_busy;
   if (n_stagers > 0 || kAllBring) {
     typedef __attribute__((address_space(3))) uint4 *lds_ptr_t;
@@ -1479,8 +1480,10 @@ extern "C" int sb_attn_prefill_bf16(void *out, const void *q, const void *k_cach
   const int group = heads_q / heads_kv;
   // Waves of a block and query heads of a kv head that one wave takes together: the block's
   // waves cover the group, eight of them (two per SIMD) when the group is big enough to use them,
-  // as far as the accumulators fit the registers.
-  int waves = (group >= 5 && group <= 8 && HD <= 128) ? 8 : 4;
+  // as far as the accumulators fit the registers.  Heads of more than 128 take eight waves with
+  // one head each for every group from 5 on (a page of theirs fills so much of LDS that a CU holds
+  // one block, and four waves would leave it half empty: measured 1.3 to 2.2 times slower).
+  int waves = (group >= 5 && (group <= 8 || HD > 128)) ? 8 : 4;
   int nc = (group + waves - 1) / waves;
   const int nc_max = waves == 8 ? 1 : (DT <= 4 ? 4 : (DT <= 12 ? 2 : 1));
   if (nc > nc_max) nc = nc_max;
@@ -1506,7 +1509,7 @@ extern "C" int sb_attn_prefill_bf16(void *out, const void *q, const void *k_cach
   } while (0)
   // (forms that nc_max rules out for this head size are not compiled)
   if (waves == 8) {
-    if constexpr (HD <= 128) SB_GO(1, 8);
+    SB_GO(1, 8);
   } else if (nc == 4) {
     if constexpr (DT <= 4) SB_GO(4, 4);
   } else if (nc == 3) {

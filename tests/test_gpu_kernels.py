@@ -624,10 +624,11 @@ def attention_case(hq, hkv, hd, lens, rows_per_seq, window, seed=0):
 
 # (groups of 7, 5 and 8 query heads per kv head run prefill with eight waves a block: one, three
 # and no wave without a head; the last shape makes a second block of one head and three such waves)
-# (the last three: every wave of a block of four has a head, with one head per wave and with
-# two heads of more than 128 per wave, where all waves share the loads that bring a page in)
+# (from (8, 2, 128) on: every wave of a block of four has a head and all waves share the loads that
+# bring a page in; heads of more than 128 in blocks of eight waves: sixteen heads in two blocks,
+# five heads and three waves without one, eight heads)
 MFMA_SHAPES = [(4, 2, 16), (3, 1, 32), (5, 5, 48), (6, 2, 80), (28, 4, 128), (2, 1, 256), (40, 2, 64), (10, 2, 128),
-               (16, 2, 64), (8, 2, 128), (4, 1, 256), (16, 1, 192)]
+               (16, 2, 64), (8, 2, 128), (4, 1, 256), (16, 1, 192), (10, 2, 160), (8, 1, 144)]
 
 
 @pytest.mark.parametrize("hq, hkv, hd", MFMA_SHAPES)
