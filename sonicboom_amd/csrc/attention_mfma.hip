@@ -446,7 +446,8 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
                     const bf16_t *__restrict__ k_cache, const bf16_t *__restrict__ v_cache,
                     const int32_t *__restrict__ page_table, int max_pages, int n_pages_total,
                     const int32_t *__restrict__ row_pos, const int32_t *__restrict__ tiles, int n_tiles,
-                    int heads_q, int heads_kv, int head_tiles, int y_per_kv, float scale_log2, int window) {
+                    int heads_q, int heads_kv, int head_tiles, int y_per_kv, float scale_log2, int window,
+                    int row_groups) {
   constexpr int kThreads = 64 * WAVES;
   constexpr int kStageLoads = (kPageChunks + kThreads - 1) / kThreads;
   extern __shared__ uint4 lds_pages[];               // [2 buffers][keys | values][kPageChunks]
@@ -456,9 +457,17 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
   const int tile = n_tiles - 1 - int(blockIdx.x) / n_y, by = int(blockIdx.x) % n_y;
   const int group = heads_q / heads_kv;
   const int kvh = by / y_per_kv, yb = by - kvh * y_per_kv;
-  const int ht = yb * WAVES + wave;                      // this wave's head tile
-  const bool active = ht < head_tiles;
-  const int row0 = tiles[tile * 4 + 0], n_rows = tiles[tile * 4 + 1], seq = tiles[tile * 4 + 2];
+  // A block's waves cover the head tiles of its kv head; where those are fewer than half the
+  // waves (groups of one or two heads), a tile is row_groups x 16 rows high and wave w takes
+  // rows 16 * (w / heads_here) .. of head tile w % heads_here, so that the waves that would have
+  // no head share the pages with rows of their own.
+  const int heads_here = WAVES / row_groups;             // head tiles a block covers
+  const int rw = wave / heads_here, hw = wave - rw * heads_here;
+  const int ht = yb * heads_here + hw;                   // this wave's head tile
+  const int tile_row0 = tiles[tile * 4 + 0], tile_rows = tiles[tile * 4 + 1], seq = tiles[tile * 4 + 2];
+  const int n_rows = max(0, min(tile_rows - 16 * rw, 16));
+  const int row0 = tile_row0 + (n_rows > 0 ? 16 * rw : 0);
+  const bool active = ht < head_tiles && n_rows > 0;
   const int r = lane & 15, g = lane >> 4;
   const bool col_ok = r < n_rows;
   const int row = row0 + (col_ok ? r : 0);
@@ -466,11 +475,14 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
   const int col_pos = col_ok ? pos : -1;
   const int col_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
   // rows of a tile are consecutive positions: the first row has the lowest window start,
-  // the last valid row the highest position
-  const int pos_first = row_pos[row0], pos_last = row_pos[row0 + n_rows - 1];
+  // the last valid row the highest position.  tile_*: of the whole tile, which decide the pages
+  // the block brings in; the others of this wave's rows, which decide what it multiplies.
+  const int tile_first = row_pos[tile_row0], tile_last = row_pos[tile_row0 + tile_rows - 1];
+  const int tile_lo = (window > 0 && tile_first >= window) ? tile_first - window + 1 : 0;
+  const int pos_first = row_pos[row0], pos_last = row_pos[row0 + max(n_rows, 1) - 1];
   const int key_lo = (window > 0 && pos_first >= window) ? pos_first - window + 1 : 0;
   const int key_hi = pos_last;
-  // first key that every row of the tile sees (the last row's window start)
+  // first key that every row of the wave sees (the last row's window start)
   const int lo_last = (window > 0 && pos_last >= window) ? pos_last - window + 1 : 0;
 
   bf16x8_t qf[NC][KS];
@@ -487,7 +499,7 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
   init_state<NC>(st);
 
   const int32_t *pt = page_table + size_t(seq) * max_pages;
-  const int pg_hi = min(key_hi / SB_PAGE, max_pages - 1);
+  const int pg_hi = min(tile_last / SB_PAGE, max_pages - 1);
   // the next page from pg on that the table holds (uniform over the block)
   auto next_valid = [&](int pg) {
     while (pg <= pg_hi) {
@@ -532,6 +544,7 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
   auto attend = [&](int pg, int buf) __attribute__((always_inline)) {
     const uint4 *kl = lds_pages + buf * 2 * kPageChunks, *vl = kl + kPageChunks;
     const int page_pos = pg * SB_PAGE;
+    if (page_pos > key_hi || page_pos + SB_PAGE - 1 < key_lo) return;      // a page of other waves' rows only
     if (HD > 128) {
       // too many fragments for the registers at once: half a page at a time
       HalfPage h;
@@ -552,7 +565,7 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
     }
   };
 
-  int pg = next_valid(key_lo / SB_PAGE);                      // the page being multiplied
+  int pg = next_valid(tile_lo / SB_PAGE);                     // the page being multiplied
   // Waves without a head (the block's last ones, when the kv head's group does not fill it) bring
   // the pages in alone, straight into LDS (a load of 64 lanes x 16 bytes lands in 1 KB of
   // consecutive LDS, and a page lies in the cache as LDS wants it): the waves that multiply then
@@ -565,7 +578,8 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
   // waves at those head sizes, are 5 to 11 % slower with them and keep the registers; eight waves
   // with bigger heads have no registers to keep pages in).
   constexpr bool kAllBring = (WAVES == 4 && (NC == 1 || HD > 128)) || (WAVES == 8 && HD > 128);
-  const int n_busy = min(head_tiles - yb * WAVES, WAVES), n_stagers = WAVES - n_busy;
+  // (tiles of several row groups: every wave has a head)
+  const int n_busy = row_groups > 1 ? WAVES : min(head_tiles - yb * WAVES, WAVES), n_stagers = WAVES - n_busy;
   if (n_stagers > 0 || kAllBring) {
     typedef __attribute__((address_space(3))) uint4 *lds_ptr_t;
     constexpr int kWaveLoads = kPageChunks / 64;       // per page of keys, and of values
@@ -1465,12 +1479,21 @@ extern "C" int sb_attn_decode_rope_bf16(void *out, const float *qkv, int row_str
                        pages_per_wave, stream);
 }
 
-// q, out: bf16 [n_rows, heads_q * HD]; tiles int32 [n_tiles][4] = (first row, rows <= 16, sequence, 0),
-// every tile inside one sequence and its rows at consecutive positions.
+// The tile height that suits these heads: 16 rows, or 64 and 32 for groups of one and two query
+// heads per kv head, whose blocks would otherwise have waves without a head.
+extern "C" int sb_attn_prefill_tile_rows(int heads_q, int heads_kv) {
+  if (heads_kv <= 0 || heads_q % heads_kv) return 16;
+  const int group = heads_q / heads_kv;
+  return group == 1 ? 64 : (group == 2 ? 32 : 16);
+}
+
+// q, out: bf16 [n_rows, heads_q * HD]; tiles int32 [n_tiles][4] = (first row, rows <= tile_rows,
+// sequence, 0), every tile inside one sequence and its rows at consecutive positions.  tile_rows:
+// 16, or what sb_attn_prefill_tile_rows gives for these heads.
 extern "C" int sb_attn_prefill_bf16(void *out, const void *q, const void *k_cache, const void *v_cache,
                                     const int32_t *page_table, int max_pages, int n_pages_total,
                                     const int32_t *row_pos, const int32_t *tiles, int n_tiles, int heads_q,
-                                    int heads_kv, float scale, int window, void *stream) {
+                                    int heads_kv, float scale, int window, int tile_rows, void *stream) {
   int rc = check_common(out, q, k_cache, v_cache, page_table, row_pos, max_pages, n_pages_total, heads_q,
                         heads_kv, window, "sb_attn_prefill_bf16");
   if (rc != SB_OK) return rc;
@@ -1489,6 +1512,9 @@ extern "C" int sb_attn_prefill_bf16(void *out, const void *q, const void *k_cach
   if (nc > nc_max) nc = nc_max;
   const int head_tiles = (group + nc - 1) / nc;
   const int y_per_kv = (head_tiles + waves - 1) / waves;
+  SB_REQUIRE(tile_rows == 16 || tile_rows == sb_attn_prefill_tile_rows(heads_q, heads_kv),
+             "sb_attn_prefill_bf16: tiles of %d rows do not suit %d heads on %d kv heads", tile_rows, heads_q, heads_kv);
+  const int row_groups = tile_rows / 16;       // more than one: waves == 4, nc == 1, head_tiles * row_groups == 4
   SB_SUPPORT((long long)n_tiles * heads_kv * y_per_kv <= 0x7fffffffLL, "sb_attn_prefill_bf16: too many blocks");
   dim3 grid(unsigned(n_tiles) * unsigned(heads_kv * y_per_kv));
   constexpr int lds_bytes = 2 * 2 * kPageChunks * 16;
@@ -1505,7 +1531,7 @@ extern "C" int sb_attn_prefill_bf16(void *out, const void *q, const void *k_cach
     attn_prefill_kernel<NC, WAVES><<<grid, 64 * WAVES, lds_bytes, s>>>(                                  \
         (bf16_t *)out, (const bf16_t *)q, (const bf16_t *)k_cache, (const bf16_t *)v_cache, page_table,  \
         max_pages, n_pages_total, row_pos, tiles, n_tiles, heads_q, heads_kv, head_tiles, y_per_kv,      \
-        scale * kLog2e, window);                                                                         \
+        scale * kLog2e, window, row_groups);                                                             \
   } while (0)
   // (forms that nc_max rules out for this head size are not compiled)
   if (waves == 8) {

@@ -676,9 +676,10 @@ def attention_decode_pages_per_wave(head_dim: int, pages: int):
 
 
 def attention_prefill_mfma(q, k_cache, v_cache, page_table, row_pos, tiles, heads_q, heads_kv, head_dim, scale,
-                           window):
-    """bf16 query rows over the cache; ``tiles`` int32 [n, 4] = (first row, rows <= 16, sequence, 0)
-    cuts the rows into runs of consecutive positions of one sequence."""
+                           window, tile_rows=16):
+    """bf16 query rows over the cache; ``tiles`` int32 [n, 4] = (first row, rows <= tile_rows, sequence, 0)
+    cuts the rows into runs of consecutive positions of one sequence.  ``tile_rows``: 16, or what
+    :func:`attention_row_tile` gives for these heads."""
     _dev(q, k_cache, v_cache, page_table, row_pos, tiles)
     n = q.shape[0]
     if q.dim() != 2 or q.shape[1] != heads_q * head_dim or q.dtype != torch.bfloat16:
@@ -693,7 +694,7 @@ def attention_prefill_mfma(q, k_cache, v_cache, page_table, row_pos, tiles, head
     out = torch.empty_like(q)
     check(lib.sb_attn_prefill_bf16(_p(out), _p(q), _p(k_cache), _p(v_cache), _p(page_table), page_table.shape[1],
                                    k_cache.shape[0], _p(row_pos), _p(tiles), tiles.shape[0], heads_q, heads_kv,
-                                   float(scale), int(window), _stream()), lib, "sb_attn_last_error")
+                                   float(scale), int(window), int(tile_rows), _stream()), lib, "sb_attn_last_error")
     return out
 
 
@@ -703,9 +704,18 @@ def attention_prefill_mfma(q, k_cache, v_cache, page_table, row_pos, tiles, head
 ATTENTION_ROW_TILE = 16
 
 
+def attention_row_tile(heads_q: int, heads_kv: int, head_dim: int, dtype=torch.bfloat16) -> int:
+    """The height of row tiles that suits attention with these heads: 16, or 64 and 32 where the
+    matrix-core kernel runs groups of one and two query heads per kv head (its blocks' waves
+    that would have no head take further rows of the tile)."""
+    if dtype != torch.bfloat16 or not attention_mfma_ok(dtype, dtype, head_dim) or not torch.cuda.is_available():
+        return ATTENTION_ROW_TILE
+    return int(library.attention_library(head_dim).sb_attn_prefill_tile_rows(int(heads_q), int(heads_kv)))
+
+
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor, ctx,
               heads_q: int, heads_kv: int, head_dim: int, scale: float, window: int,
-              fast: bool = True) -> torch.Tensor:
+              fast: bool = True, row_tile: int = ATTENTION_ROW_TILE) -> torch.Tensor:
     """Attention of a step's rows over the cache; ``ctx`` is the step's context.  bfloat16 with a
     head size in steps of 16 runs on the matrix cores (a decode kernel when every sequence brings
     one row, else the prefill kernel); everything else takes the plain kernel."""
@@ -713,8 +723,7 @@ def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, pag
         if ctx.is_decode:
             return attention_decode_mfma(q, k_cache, v_cache, page_table, ctx.row_pos, heads_q, heads_kv,
                                          head_dim, scale, window)
-        return attention_prefill_mfma(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_tiles(ATTENTION_ROW_TILE),
-                                      heads_q, heads_kv,
-                                      head_dim, scale, window)
+        return attention_prefill_mfma(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_tiles(row_tile),
+                                      heads_q, heads_kv, head_dim, scale, window, tile_rows=row_tile)
     return attention_plain(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_seq, heads_q, heads_kv,
                            head_dim, scale, window)

@@ -70,6 +70,9 @@ class Attention(Mixer):
         self.scale = float(np.float32(base_scale) * np.float32(self.position.score_scale))
         self.q_width = self.heads_q * self.head_dim
         self.kv_width = self.heads_kv * self.head_dim
+        if rt.fast_kernels:
+            # (groups of one and two heads per kv head take higher tiles on the matrix cores)
+            self.row_tile = ops.attention_row_tile(self.heads_q, self.heads_kv, self.head_dim, rt.act_dtype)
 
         ws = [tensors["q_weight"], tensors["k_weight"], tensors["v_weight"]]
         w_qkv = torch.cat(ws, dim=0) if all(w.dtype == ws[0].dtype for w in ws) \
@@ -137,5 +140,5 @@ class Attention(Mixer):
             page_table if writes else None, self.heads_q, self.heads_kv if writes else 0, self.head_dim,
             bias=bias)
         a = ops.attention(q, binding.k_cache, binding.v_cache, page_table, ctx, self.heads_q, self.heads_kv,
-                          self.head_dim, self.scale, self.window, fast=rt.fast_kernels)
+                          self.head_dim, self.scale, self.window, fast=rt.fast_kernels, row_tile=self.row_tile)
         return self.out.add_into(a, x, then_norm, rt.act_dtype)

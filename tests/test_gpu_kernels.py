@@ -626,9 +626,9 @@ def attention_case(hq, hkv, hd, lens, rows_per_seq, window, seed=0):
 # and no wave without a head; the last shape makes a second block of one head and three such waves)
 # (from (8, 2, 128) on: every wave of a block of four has a head and all waves share the loads that
 # bring a page in; heads of more than 128 in blocks of eight waves: sixteen heads in two blocks,
-# five heads and three waves without one, eight heads)
+# five heads and three waves without one, eight heads; groups of one and two heads at usual head sizes)
 MFMA_SHAPES = [(4, 2, 16), (3, 1, 32), (5, 5, 48), (6, 2, 80), (28, 4, 128), (2, 1, 256), (40, 2, 64), (10, 2, 128),
-               (16, 2, 64), (8, 2, 128), (4, 1, 256), (16, 1, 192), (10, 2, 160), (8, 1, 144)]
+               (16, 2, 64), (8, 2, 128), (4, 1, 256), (16, 1, 192), (10, 2, 160), (8, 1, 144), (3, 3, 128), (4, 2, 64)]
 
 
 @pytest.mark.parametrize("hq, hkv, hd", MFMA_SHAPES)
@@ -712,15 +712,22 @@ def test_attention_prefill_matrix_cores(hq, hkv, hd, window):
     rows_per_seq = [list(range(s0, n)) for s0, n in zip(starts, lens)]
     q, kc, vc, table, rows, scale, want = attention_case(hq, hkv, hd, lens, rows_per_seq, window, seed=3)
     pos = torch.tensor([p for _, p in rows], dtype=torch.int32)
-    tiles, row0 = [], 0
-    for s_, ps in enumerate(rows_per_seq):
-        for r0 in range(0, len(ps), 16):
-            tiles.append((row0 + r0, min(16, len(ps) - r0), s_, 0))
-        row0 += len(ps)
-    tiles = torch.tensor(tiles, dtype=torch.int32)
-    got = ops.attention_prefill_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), tiles.to(DEV), hq, hkv, hd,
-                                     scale, window)
-    close(got, want, atol=1.5e-2, rtol=1e-2, what="prefill")
+    # tiles of 16 rows, and of the height that suits the group (64 and 32 rows for groups of one and two heads)
+    for height in sorted({16, ops.attention_row_tile(hq, hkv, hd)}):
+        tiles, row0 = [], 0
+        for s_, ps in enumerate(rows_per_seq):
+            for r0 in range(0, len(ps), height):
+                tiles.append((row0 + r0, min(height, len(ps) - r0), s_, 0))
+            row0 += len(ps)
+        tiles = torch.tensor(tiles, dtype=torch.int32)
+        got = ops.attention_prefill_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), tiles.to(DEV), hq, hkv, hd,
+                                         scale, window, tile_rows=height)
+        close(got, want, atol=1.5e-2, rtol=1e-2, what=f"prefill, tiles of {height} rows")
+    assert ops.attention_row_tile(hq, hkv, hd) == (64 if hq == hkv else 32 if hq == 2 * hkv else 16)
+    if hq > 2 * hkv:
+        with pytest.raises(ops.KernelLibraryError, match="do not suit"):
+            ops.attention_prefill_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), tiles.to(DEV), hq, hkv, hd,
+                                       scale, window, tile_rows=64)
 
 
 def test_attention_reference_vectors():
