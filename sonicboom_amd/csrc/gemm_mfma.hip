@@ -842,10 +842,11 @@ namespace {
 // what was measured on MI355X with the 7B products at 768 to 2,304 rows: a shape's tile takes
 // 2 bm bn K flops at its kernel's rate on a full GPU (pick_shape's speeds, 1 standing for 0.93
 // PFLOP/s over 256 CUs); a round that leaves CUs idle runs faster (0.72 of the time with up to 170
-// blocks, rising to 1 at 256: the chip's clock follows its load); a whole product costs 14 us
-// beside its tiles and a cut one 6; the consumer's pass over the additional slices moves
-// (2 slices - 2) x the result's bytes at 4 TB/s.  The cut is taken when it comes out under 0.92 of
-// the best whole product.  Measured, whole + norm against cut + the pass that adds the slices, the
+// blocks, rising to 1 at 256: the chip's clock follows its load); either kernel costs 14 us
+// beside its tiles; the consumer's pass over the additional slices moves (2 slices - 2) x the
+// result's bytes at 4 TB/s.  The cut is taken when it comes out under 0.9 of the best whole
+// product (at the 3B and 1.5B products of 2,048 rows, whose 128 x 128 tiles fill the GPU in one
+// round as it is, a cut priced at 0.9 to 0.97 measured 0.99 to 1.04).  Measured, whole + norm against cut + the pass that adds the slices, the
 // residual and the norm: down (3,584 x 18,944) at 1,280 rows 237 against 152 us, at 2,048 rows 272
 // against 247; output (3,584 x 3,584) at 1,280 rows 69 against 52.
 struct PartialPlan { int slices; bool big; };
@@ -875,11 +876,11 @@ PartialPlan partial_plan(int n_rows, int n_out, int n_in, bool direct_ok) {
     long long s_best = 0;
     for (long long s2 = 2; s2 <= 8 && s2 * big_grid <= kCus && s2 <= n_k / 4; ++s2) {
       const int per = int((n_k + s2 - 1) / s2);
-      const double t = 2.0 * 256 * 256 * (64.0 * per) / (speed[2] * per_cu) * load_factor(s2 * big_grid) + 6.0 +
+      const double t = 2.0 * 256 * 256 * (64.0 * per) / (speed[2] * per_cu) * load_factor(s2 * big_grid) + 14.0 +
                        (2.0 * s2 - 2.0) * n_rows * double(n_out) * 4.0 / 4e6;
       if (s_best == 0 || t < t_best) t_best = t, s_best = s2;
     }
-    if (s_best && t_best < 0.92 * t_whole) {
+    if (s_best && t_best < 0.9 * t_whole) {
       const int per = int((n_k + s_best - 1) / s_best);
       return {(n_k + per - 1) / per, true};
     }
