@@ -506,10 +506,11 @@ def gemm_bf16(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], re
         wave_units = -(-n // 16) if gated else -(-n // 32)
         which = "stream" if packed and wave_units >= 4 * STREAM_MIN_BLOCKS else "skinny"
         if t > SKINNY_MAX_ROWS and which == "stream":
-            # 65 to 128 rows: the tiled kernel's 128 x 128 tiles do as well or better unless their
-            # count leaves the last round over the 256 CUs nearly empty
+            # 65 to 128 rows: the tiled kernel's 128 x 128 tiles do as well or better unless the
+            # matrix is wide and their count leaves the last round over the 256 CUs nearly empty
+            # (8,960 x 1,536 and 11,008 x 2,048 at 96 rows: 21 and 26 us tiled, 25 and 34 streamed)
             rounds = -(-n // (64 if gated else 128)) / 256.0
-            if math.ceil(rounds) / rounds < 1.4:
+            if wave_units < 4 * STREAM_MIN_BLOCKS_MORE_ROWS or math.ceil(rounds) / rounds < 1.4:
                 which = "tiled"
     if t <= STREAM_MAX_ROWS and which == "stream" and packed:
         check(lib.sb_gemm_stream_bf16(_p(out), _dt(out), _p(x), _p(w), _p(bias), bdt, _p(resid), t, n, k,
@@ -563,7 +564,14 @@ def gemm_few_rows_kernel(which: Optional[str], waves: int = 0, slices: int = 0):
 
 
 MFMA_MAX_HEAD_DIM = 256
-STREAM_MIN_BLOCKS = 192
+# Blocks of four waves that a matrix must give the stream kernel.  A block streams its share of W at
+# what one CU pulls, whatever the count of blocks, so fewer blocks than CUs only pay while the
+# other kernel, which spreads K over the whole GPU, has more bytes to move than a block's share
+# takes: gate/up pairs of 8,960 x 1,536 (140 blocks) 13 to 18 us against 18 to 29 at up to 64 rows,
+# 11,008 x 2,048 (172 blocks) 19 to 25 against 25 to 34; 8,192 x 2,048 (128 blocks) 18 against 16,
+# and 4,864 x 896 (76 blocks) 4 % slower in a whole decode step.
+STREAM_MIN_BLOCKS = 136
+STREAM_MIN_BLOCKS_MORE_ROWS = 192        # for 65 to 128 rows
 STREAM_MAX_ROWS = 128
 
 
