@@ -664,11 +664,12 @@ def test_attention_decode_matrix_cores_many_sequences(window, longest):
 
 
 @pytest.mark.parametrize("window", [0, 300])
-@pytest.mark.parametrize("n_seqs, longest", [(30, 2000), (12, 5000), (3, 9000)])
+@pytest.mark.parametrize("n_seqs, longest", [(30, 2000), (12, 5000), (3, 9000), (70, 1500)])
 def test_attention_decode_matrix_cores_long_rows_of_unequal_length(window, n_seqs, longest):
     """Rows long enough for the launcher to deal several pages to a wave and cut the rows into
     chunks of its own choosing; lengths from one key to thousands in one batch, so that chunks
-    are full, partly filled and empty side by side."""
+    are full, partly filled and empty side by side.  (70 sequences on 4 kv heads: a few blocks
+    more than the GPU has CUs, for which the launcher takes smaller chunks.)"""
     from sonicboom_amd import ops
     hq, hkv, hd = 8, 4, 64
     rng = np.random.default_rng(n_seqs)
