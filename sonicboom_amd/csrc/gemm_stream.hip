@@ -240,7 +240,9 @@ Cut cut_for(int tiles, int n_steps, int tt, int hint) {
     for (int w = 4; w <= 8; ++w) {
       if (force_waves >= 4 && force_waves <= 8 && w != force_waves) continue;
       const long long blocks = (long long)((tiles + w - 1) / w) * slices;
-      const long long cost = (blocks + n_cu - 1) / n_cu * (sps + 24) * (2 * w + tt) + 12LL * slices;
+      // (+ 4 per wave: between choices that this prices alike, the one with fewer waves and slices
+      // measured 1 to 2 % faster in whole decode steps of the 14B and 32B sizes at up to 16 rows)
+      const long long cost = (blocks + n_cu - 1) / n_cu * (sps + 24) * (2 * w + tt) + 12LL * slices + 4LL * w;
       if (best_cost < 0 || cost < best_cost) best = Cut{w, slices, sps}, best_cost = cost;
     }
   }
