@@ -266,7 +266,10 @@ extern "C" int sb_rmsnorm(void *y, int out_dtype, const float *x, const void *w,
   if (out_dtype == SB_F32) {
     rmsnorm_kernel<float, 1024, 2><<<n_rows, 1024, 0, s>>>((float *)y, x, w, w_dtype, rows, width, eps);
   } else {
-    if (many) rmsnorm_kernel<bf16_t, 256, 4><<<n_rows, 256, 0, s>>>((bf16_t *)y, x, w, w_dtype, rows, width, eps);
+    // (rows of 4,097 to 8,192: eight groups a thread, so that none goes through the scalar loops:
+    // 2,048 rows of 8,192 27.7 us before)
+    if (many && width > 4096) rmsnorm_kernel<bf16_t, 256, 8><<<n_rows, 256, 0, s>>>((bf16_t *)y, x, w, w_dtype, rows, width, eps);
+    else if (many) rmsnorm_kernel<bf16_t, 256, 4><<<n_rows, 256, 0, s>>>((bf16_t *)y, x, w, w_dtype, rows, width, eps);
     else rmsnorm_kernel<bf16_t, 1024, 2><<<n_rows, 1024, 0, s>>>((bf16_t *)y, x, w, w_dtype, rows, width, eps);
   }
   return sb::check_launch("sb_rmsnorm");

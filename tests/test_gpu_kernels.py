@@ -45,7 +45,7 @@ def test_embed(dtype):
 
 
 @pytest.mark.parametrize("n_rows", [7, 300])       # few rows and many rows take different block shapes
-@pytest.mark.parametrize("width", [64, 201, 338, 3584, 5000])
+@pytest.mark.parametrize("width", [64, 201, 338, 3584, 5000, 8192, 9004])     # up to 4,096, up to 8,192, beyond
 @pytest.mark.parametrize("out_dtype, w_dtype", [(F32, F32), (BF16, BF16), (BF16, F32)])
 def test_rmsnorm(width, out_dtype, w_dtype, n_rows):
     from sonicboom_amd import ops
