@@ -14,6 +14,15 @@ ids.  One JSON line is printed: decoded tokens a second (from the median step), 
 2,048-token prompt, the decode step against the HBM roofline with the rates of its kernels, and
 decode at batch 1 and 64.
 
+The same line carries the context-length curve as further ``points`` (and with bytes, flops and
+fractions under ``curve``): for cached depths of 512, 4,096, 8,192, 16,384 and 32,768 tokens the
+decode rate at batch 1 and batch 8 (``decode_b1_d8192`` ...) and the prefill rate of one prompt of
+that length (``prefill_8192`` ...); ``--no-curve`` leaves it out, ``--curve 512,4096`` picks depths.
+``--runs R`` (R > 1) starts R fresh processes of the same command one after the other, before
+anything touches the GPU here, and prints the run whose ``value`` is the median, with all values.
+Beside the JSON line on standard output, every metric goes to standard error as a
+``RESULT key=value ...`` line; the engine clock sampled during the timed decode steps is in both.
+
 ``--workload mixed`` runs what the baseline names for the larger sizes through the generation
 loop itself: ``--sizes 14b``: 16 prompts of seeded lengths uniform in [256, 4096] in a cache of
 8192 tokens a sequence, prompts in one step, then 256 greedy steps; ``--sizes 72b``: 8 prompts of
@@ -32,7 +41,7 @@ CONFIG_7B = {
     "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
     "num_hidden_layers": 28, "hidden_size": 3584, "num_attention_heads": 28, "num_key_value_heads": 4,
     "intermediate_size": 18944, "vocab_size": 152064, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
-    "max_position_embeddings": 32768, "tie_word_embeddings": False, "use_sliding_window": False,
+    "max_position_embeddings": 131072, "tie_word_embeddings": False, "use_sliding_window": False,
     "hidden_act": "silu",
 }
 # the other sizes the baseline names, for runs beyond the default one (--sizes)
@@ -54,6 +63,8 @@ MIXED = {"72b": (8, 512, 2048, 128, 4096), "32b": (8, 512, 2048, 128, 4096)}
 MIXED_DEFAULT = (16, 256, 4096, 256, 8192)
 CONTEXT = 4096
 PROMPT = 2048
+CURVE_DEPTHS = (512, 4096, 8192, 16384, 32768)
+CURVE_BATCHES = (1, 8)
 
 
 def model_numbers(cfg, n_layers):
@@ -83,8 +94,9 @@ def decode_bytes(m, batch, lengths):
 
 
 class ClockSampler:
-    """Samples the GPU's engine clock with ``rocm-smi --showclocks`` in a thread while work runs
-    (``--clocks``): what the matrix pipes' peak has to be scaled by under load."""
+    """Samples the GPU's engine clock in a thread while work runs (the driver's ``pp_dpm_sclk``
+    file, else ``rocm-smi --showclocks``): what the matrix pipes' peak has to be scaled by under
+    load, and what a run's figures have to be read against."""
 
     def __init__(self, period=0.4):
         import threading
@@ -93,8 +105,18 @@ class ClockSampler:
 
     @staticmethod
     def read():
+        import glob
         import re
         import subprocess
+        # the driver's own file first (microseconds to read): the level marked with a star
+        for path in sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk")):
+            try:
+                with open(path) as f:
+                    m = re.search(r"(\d+)\s*Mhz\s*\*", f.read(), re.IGNORECASE)
+            except OSError:
+                continue
+            if m:
+                return int(m.group(1))
         try:
             out = subprocess.run(["rocm-smi", "--showclocks"], capture_output=True, text=True, timeout=20).stdout
         except (OSError, subprocess.SubprocessError):
@@ -229,10 +251,25 @@ def main() -> int:
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel rates")
     ap.add_argument("--clocks", action="store_true",
                     help="also run prompt steps back to back for a few seconds and sample the engine clock meanwhile")
+    ap.add_argument("--curve", default=",".join(str(d) for d in CURVE_DEPTHS),
+                    help="cached depths of the context-length curve (decode at batch 1 and 8, prefill of one prompt)")
+    ap.add_argument("--no-curve", action="store_true", help="skip the context-length curve")
+    ap.add_argument("--runs", type=int, default=1,
+                    help="fresh processes to run one after the other; the median run is printed")
     a = ap.parse_args()
     if a.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {a.gpus} is not supported")
         return 2
+    if a.runs > 1:
+        argv, skip = [], False
+        for arg in sys.argv[1:]:
+            if skip:
+                skip = False
+            elif arg == "--runs":
+                skip = True
+            elif not arg.startswith("--runs="):
+                argv.append(arg)
+        return median_of_runs(argv, a.runs)
 
     import numpy as np
     import torch
@@ -243,11 +280,14 @@ def main() -> int:
     from sonicboom_amd.sampling import SamplingParams
 
     PROMPT, CONTEXT = a.prompt, max(a.context, a.prompt + a.steps + a.warmup + 64)
+    if a.prompt != 2048 and "--curve" not in " ".join(sys.argv[1:]):
+        a.no_curve = True           # a run at a depth of its own is one point, not the curve
     model_name, base_cfg = SIZES[a.sizes]
     cfg = dict(base_cfg)
     full_layers = cfg["num_hidden_layers"]
     if a.layers:
         cfg["num_hidden_layers"] = a.layers
+    cfg["max_position_embeddings"] = max(cfg["max_position_embeddings"], CONTEXT)
     m = model_numbers(cfg, cfg["num_hidden_layers"])
     t0 = time.time()
     model = DecoderModel.from_random(cfg, seed=0, dtype="bfloat16", device="cuda:0")
@@ -333,23 +373,29 @@ def main() -> int:
         return 0
 
     # ---- prefill of one prompt (2,048 tokens unless --prompt says otherwise) ----------------
+    def prefill_run(engine, n_tokens, timed, kernels):
+        """Median seconds of ``timed`` prompt steps of one prompt of ``n_tokens`` in an empty slot
+        (after one untimed step), as the bench line's ``prefill`` entry."""
+        times = []
+        for i in range(timed + 1):
+            p = random_prompts([n_tokens])[0]
+            slot = engine.alloc_slot()
+            times.append(sync_time(lambda: engine.step([StepEntry(slot, p, (n_tokens - 1,))])))
+            engine.free_slot(slot)
+        secs = statistics.median(times[1:])
+        pf = prefill_flops(m, [n_tokens])
+        out = {"value": round(n_tokens / secs, 1), "tokens": n_tokens, "ms": round(secs * 1e3, 3),
+               "frac": round(pf / secs / PEAK_FLOPS["bf16"], 4), "flops": int(pf)}
+        if kernels:
+            slot = engine.alloc_slot()
+            with OpTimer(m) as timer:
+                engine.step([StepEntry(slot, random_prompts([n_tokens])[0], (n_tokens - 1,))])
+            engine.free_slot(slot)
+            out["kernels"] = kernel_rates(m, timer.totals(), n_tokens, 0, prefill_lengths=[n_tokens])
+        return out, pf
+
     engine = Engine(model, max_tokens=CONTEXT)
-    times = []
-    for i in range(5):
-        p = random_prompts([PROMPT])[0]
-        slot = engine.alloc_slot()
-        times.append(sync_time(lambda: engine.step([StepEntry(slot, p, (PROMPT - 1,))])))
-        engine.free_slot(slot)
-    prefill_s = statistics.median(times[1:])
-    pf = prefill_flops(m, [PROMPT])
-    prefill = {"value": round(PROMPT / prefill_s, 1), "tokens": PROMPT, "ms": round(prefill_s * 1e3, 3),
-               "frac": round(pf / prefill_s / PEAK_FLOPS["bf16"], 4)}
-    if not a.no_kernels:
-        slot = engine.alloc_slot()
-        with OpTimer(m) as timer:
-            engine.step([StepEntry(slot, random_prompts([PROMPT])[0], (PROMPT - 1,))])
-        engine.free_slot(slot)
-        prefill["kernels"] = kernel_rates(m, timer.totals(), PROMPT, 0, prefill_lengths=[PROMPT])
+    prefill, pf = prefill_run(engine, PROMPT, 4, not a.no_kernels)
     if a.clocks:
         idle = ClockSampler.read()
         p = random_prompts([PROMPT])[0]
@@ -370,19 +416,19 @@ def main() -> int:
     del engine
 
     # ---- decode -----------------------------------------------------------------------------
-    def decode_run(batch, steps, warmup, kernels=False):
-        eng = Engine(model, max_tokens=CONTEXT * batch)
+    def decode_steps(eng, slots, first, steps, warmup, kernels=False, clock=None):
+        """Time ``steps`` decode steps of the sequences in ``slots`` (fed ``first``) after
+        ``warmup`` untimed ones: median and mean seconds a step, the lengths after the run, the
+        kernels' rates, and the tokens the next step would feed."""
         loop = DecodeLoop(eng, use_graph=not a.no_graph)
-        slots = [eng.alloc_slot() for _ in range(batch)]
-        ps = random_prompts([PROMPT] * batch)
-        # the prompts in one step; the engine runs it in portions of its row limit
-        logits = eng.step([StepEntry(s, p, (PROMPT - 1,)) for s, p in zip(slots, ps)])
-        first = torch.argmax(logits, dim=-1).tolist()
+        batch = len(slots)
         loop.start(slots, first)
         for _ in range(warmup):
             loop.step()
         torch.cuda.synchronize()
         per_step = []
+        if clock is not None:
+            clock.__enter__()
         t_all = time.perf_counter()
         for _ in range(steps):
             t = time.perf_counter()
@@ -390,6 +436,8 @@ def main() -> int:
             per_step.append(time.perf_counter() - t)
         torch.cuda.synchronize()
         mean = (time.perf_counter() - t_all) / steps
+        if clock is not None:
+            clock.__exit__()
         lengths = [eng.length(s) for s in slots]
         rates = None
         if kernels:
@@ -399,28 +447,89 @@ def main() -> int:
             with OpTimer(m) as timer:
                 plain.step()
             rates = kernel_rates(m, timer.totals(), batch, sum(lengths) + batch, None)
+            loop.pending = plain.pending
+        pending = list(loop.pending)
         loop.close()
+        return statistics.median(per_step), mean, lengths, rates, pending
+
+    def fill(eng, batch, prompt):
+        """``batch`` slots, each with a cached prompt of ``prompt`` random tokens, and the first
+        token of each; the prompts run in one step (in portions of the engine's row limit)."""
+        slots = [eng.alloc_slot() for _ in range(batch)]
+        ps = random_prompts([prompt] * batch)
+        logits = eng.step([StepEntry(s, p, (prompt - 1,)) for s, p in zip(slots, ps)])
+        return slots, torch.argmax(logits, dim=-1).tolist()
+
+    def per_sequence(prompt, steps, warmup):
+        """Cache tokens a sequence needs for these runs (whole pages, with room to spare)."""
+        return ((prompt + 2 * (steps + warmup) + 8 + 127) // 64) * 64
+
+    def decode_run(batch, steps, warmup, kernels=False, clock=None):
+        eng = Engine(model, max_tokens=max(CONTEXT, per_sequence(PROMPT, steps, warmup)) * batch)
+        slots, first = fill(eng, batch, PROMPT)
+        out = decode_steps(eng, slots, first, steps, warmup, kernels, clock)
         for s in slots:
             eng.free_slot(s)
         del eng
-        return statistics.median(per_step), mean, lengths, rates
+        return out[:4]
 
-    step_s, mean_s, lengths, rates = decode_run(a.batch, a.steps, a.warmup, kernels=not a.no_kernels)
-    value = a.batch / step_s
-    nbytes = decode_bytes(m, a.batch, lengths)
-    roofline = {"bound": "hbm", "achieved": round(nbytes / step_s / 1e9, 1), "peak": PEAK_HBM_GBS,
-                "unit": "GB/s", "frac": round(nbytes / step_s / 1e9 / PEAK_HBM_GBS, 4),
+    def hbm(nbytes, secs):
+        return {"bound": "hbm", "achieved": round(nbytes / secs / 1e9, 1), "peak": PEAK_HBM_GBS,
+                "unit": "GB/s", "frac": round(nbytes / secs / 1e9 / PEAK_HBM_GBS, 4),
                 "peak_measured": peak_measured, "bytes_per_step": int(nbytes)}
+
+    sampler = ClockSampler(period=0.2)
+    idle_mhz = ClockSampler.read()
+    step_s, mean_s, lengths, rates = decode_run(a.batch, a.steps, a.warmup, kernels=not a.no_kernels, clock=sampler)
+    clock = sampler.summary()
+    if clock is not None:
+        clock["idle_mhz"] = idle_mhz
+    value = a.batch / step_s
+    roofline = hbm(decode_bytes(m, a.batch, lengths), step_s)
     if rates is not None:
         roofline["kernels"] = rates
     print(f"[bench] decode b{a.batch}: {value:.1f} tok/s, median {step_s * 1e3:.3f} ms/step "
-          f"(mean {mean_s * 1e3:.3f}), {roofline}", file=sys.stderr, flush=True)
+          f"(mean {mean_s * 1e3:.3f}), {roofline}, engine clock {clock}", file=sys.stderr, flush=True)
     points = {}
     if not a.no_points:
         for b in (1, 64):
             dt, _, _, _ = decode_run(b, max(8, a.steps // 2), max(2, a.warmup // 2))
             points[f"decode_b{b}"] = round(b / dt, 1)
             print(f"[bench] decode b{b}: {points[f'decode_b{b}']} tok/s", file=sys.stderr, flush=True)
+
+    # ---- the context-length curve --------------------------------------------------------------
+    curve = {}
+    depths = [] if (a.no_curve or a.no_points) else [int(d) for d in a.curve.split(",") if d.strip()]
+    steps_c, warm_c = max(8, min(a.steps, 32)), max(3, min(a.warmup, 8))
+    for depth in depths:
+        per_seq = per_sequence(depth, steps_c, warm_c)
+        eng = Engine(model, max_tokens=per_seq * max(CURVE_BATCHES))
+        item, _ = prefill_run(eng, depth, 2, not a.no_kernels)
+        if "kernels" in item:          # the curve keeps the rate of the kernel that grows with the depth
+            item["attention_TFLOPs"] = item["kernels"].get("attention", {}).get("TFLOP/s")
+            item["attention_frac"] = item["kernels"].get("attention", {}).get("frac")
+            del item["kernels"]
+        entry = {"prefill": item}
+        points[f"prefill_{depth}"] = item["value"]
+        slots, first = fill(eng, max(CURVE_BATCHES), depth)
+        for b in sorted(CURVE_BATCHES, reverse=True):        # the larger batch first, then its first sequences
+            for s in slots[b:]:
+                eng.free_slot(s)
+            slots, first = slots[:b], first[:b]
+            dt, _, lens, rates_c, first = decode_steps(eng, slots, first, steps_c, warm_c, kernels=not a.no_kernels)
+            d_item = {"value": round(b / dt, 1), "ms": round(dt * 1e3, 4)}
+            d_item.update({k: v for k, v in hbm(decode_bytes(m, b, lens), dt).items()
+                           if k in ("achieved", "frac", "bytes_per_step")})
+            if rates_c is not None and "attention" in rates_c:
+                d_item["attention_us"] = rates_c["attention"]["us"]
+                d_item["attention_GBs"] = rates_c["attention"].get("GB/s")
+            entry[f"decode_b{b}"] = d_item
+            points[f"decode_b{b}_d{depth}"] = d_item["value"]
+        for s in slots:
+            eng.free_slot(s)
+        del eng
+        curve[f"d{depth}"] = entry
+        print(f"[bench] depth {depth}: {entry}", file=sys.stderr, flush=True)
 
     line = {
         "metric": f"decode tokens/s, {model_name} sizes, batch {a.batch}, {PROMPT}-token cached prompts",
@@ -429,8 +538,55 @@ def main() -> int:
         "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": config(global_batch=a.batch, seq_len=CONTEXT, cached_prompt_tokens=PROMPT),
-        "prefill": prefill, "roofline": roofline, "points": points,
+        "prefill": prefill, "roofline": roofline, "points": points, "clock": clock,
     }
+    if curve:
+        line["curve"] = curve
+    result_lines(line)
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+def result_lines(line, out=sys.stderr):
+    """The run's metrics as ``RESULT key=value ...`` lines, one a metric, for tools that parse
+    such lines rather than JSON; the engine clock the timed steps ran at is on every line."""
+    clock = line.get("clock") or {}
+    mhz = clock.get("median_mhz")
+    tail = f" sclk_mhz={mhz if mhz is not None else 'unknown'}"
+    print(f"RESULT metric=decode_tok_s batch={line['config']['global_batch']} value={line['value']} "
+          f"ms_per_step={line['ms_per_step']} hbm_frac={line['roofline']['frac']}{tail}", file=out)
+    pre = line.get("prefill")
+    if pre:
+        print(f"RESULT metric=prefill_tok_s tokens={pre['tokens']} value={pre['value']} ms={pre['ms']} "
+              f"flops_frac={pre['frac']}{tail}", file=out)
+    for name, v in (line.get("points") or {}).items():
+        print(f"RESULT metric={name} value={v}{tail}", file=out)
+    out.flush()
+
+
+def median_of_runs(argv, runs):
+    """``runs`` fresh processes of this program, one after the other (nothing here has touched
+    the GPU); the line of the run whose value is the median, with every run's value."""
+    import os
+    import subprocess
+    lines = []
+    for i in range(runs):
+        cmd = [sys.executable, os.path.abspath(__file__)] + argv + ["--runs", "1"]
+        p = subprocess.run(cmd, stdout=subprocess.PIPE, text=True)
+        if p.returncode != 0:
+            print(f"bench.py: run {i + 1} of {runs} ended with {p.returncode}", file=sys.stderr)
+            return p.returncode or 1
+        found = [ln for ln in p.stdout.splitlines() if ln.startswith("{")]
+        lines.append(json.loads(found[-1]))
+        print(f"[bench] run {i + 1} of {runs}: {lines[-1]['value']} {lines[-1]['unit']}", file=sys.stderr, flush=True)
+    order = sorted(range(runs), key=lambda i: lines[i]["value"])
+    line = lines[order[(runs - 1) // 2]]
+    line["process_runs"] = runs
+    line["values_of_runs"] = [ln["value"] for ln in lines]
+    if all("points" in ln for ln in lines):
+        line["points"] = {k: statistics.median(ln["points"][k] for ln in lines) for k in line["points"]
+                          if all(k in ln["points"] for ln in lines)}
+    result_lines(line)
     print(json.dumps(line), flush=True)
     return 0
 
