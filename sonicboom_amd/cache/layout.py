@@ -14,7 +14,7 @@ import functools
 import numpy as np
 import torch
 
-PAGE = 64
+from ..csrc.header import PAGE
 
 
 def key_swizzle(slot: int, head_dim: int) -> int:

@@ -11,8 +11,13 @@ per-sequence state of fixed size.
   rows of a shape of its own, ``[entries, pages, PAGE, *shape]``, in groups by
   (shape, window).  A group
   that only reads a window of keys gives pages back as the window leaves them.
-* ``max_tokens`` sizes every pool: the most tokens live sequences hold at any
+* ``max_tokens`` sizes the pools: the most tokens live sequences hold at any
   time, each sequence's count rounded up to a whole page (PAGE = 64 tokens).
+  A group that keeps every key gets that many pages.  A group with a window
+  never holds more of a sequence than its window and the rows of the step
+  that is running, so with ``max_slots`` sequences and steps of at most
+  ``step_rows`` rows its pool is ``max_slots * (pages(window) + 2) +
+  pages(step_rows)`` pages when that is less (:func:`pool_pages`).
 * **State**: an entry whose mixer asks for fixed-size state gets a tensor
   ``[max_slots, *shape]``; a slot's row is zeroed when the slot is handed out,
   because a recurrence reads its state before it writes it.  Keys and values
@@ -30,7 +35,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 
-PAGE = 64
+from ..csrc.header import PAGE          # tokens per page: SB_PAGE of csrc/sb_hip.h
 
 
 class CacheError(RuntimeError):
@@ -82,16 +87,31 @@ class _Slot:
     pages: List[List[int]] = field(default_factory=list)   # per group: logical page -> physical or -1
 
 
+def pool_pages(n_pages: int, window: int, max_slots: int, step_rows: int) -> int:
+    """Pages of a group's pool in a cache of ``n_pages``: all of them for a group that keeps
+    every key (``window`` 0); for a windowed group what ``max_slots`` sequences can hold at
+    once, if that is less: after a step a sequence keeps the pages its window touches
+    (pages(window) + 1 at most), and a step of up to ``step_rows`` rows adds pages(rows) + 1 pages
+    a sequence before the old ones are given back."""
+    if window <= 0 or step_rows <= 0:
+        return n_pages
+    return min(n_pages, max_slots * (pages_for(window) + 2) + pages_for(step_rows))
+
+
 class PagedCache:
     def __init__(self, groups: Sequence[GroupSpec], max_tokens: int, dtype=None, device=None,
                  state_shapes: Optional[Dict[int, tuple]] = None, max_slots: Optional[int] = None,
-                 allocate: bool = True):
+                 allocate: bool = True, step_rows: int = 0):
+        """``step_rows``: the most rows the caller feeds between two calls of :meth:`advance`
+        (0: no bound is promised, and every group gets pages for ``max_tokens``)."""
         if max_tokens <= 0:
             raise CacheError("max_tokens must be positive")
         self.groups = list(groups)
         self.n_pages = pages_for(max_tokens)
         self.max_slots = max_slots if max_slots is not None else self.n_pages
-        self.pools = [PagePool(self.n_pages) for _ in self.groups]
+        self.step_rows = int(step_rows)
+        self.pools = [PagePool(pool_pages(self.n_pages, g.window, self.max_slots, self.step_rows))
+                      for g in self.groups]
         self._slots: Dict[int, _Slot] = {}
         self._free_slots = list(range(self.max_slots - 1, -1, -1))
         self.entry_place: Dict[int, Tuple[int, int]] = {}      # entry -> (group, index within group)
@@ -106,16 +126,16 @@ class PagedCache:
         self.dtype, self.device = dtype, device
         if allocate:
             import torch
-            for spec in self.groups:
-                n = len(spec.entries)
+            for spec, pool in zip(self.groups, self.pools):
+                n, pages = len(spec.entries), pool.n_pages
                 if spec.row_shape:
-                    self.k.append(torch.zeros((n, self.n_pages, PAGE, *spec.row_shape), dtype=dtype, device=device))
+                    self.k.append(torch.zeros((n, pages, PAGE, *spec.row_shape), dtype=dtype, device=device))
                     self.v.append(None)
                     continue
                 # keys [.., position, d]; values transposed [.., d, position] (see csrc/sb_hip.h)
-                self.k.append(torch.zeros((n, self.n_pages, spec.kv_heads, PAGE, spec.head_dim),
+                self.k.append(torch.zeros((n, pages, spec.kv_heads, PAGE, spec.head_dim),
                                           dtype=dtype, device=device))
-                self.v.append(torch.zeros((n, self.n_pages, spec.kv_heads, spec.head_dim, PAGE),
+                self.v.append(torch.zeros((n, pages, spec.kv_heads, spec.head_dim, PAGE),
                                           dtype=dtype, device=device))
             for key, (shape, sdtype) in (state_shapes or {}).items():
                 self.state[key] = torch.zeros((self.max_slots, *shape), dtype=sdtype, device=device)
@@ -154,7 +174,7 @@ class PagedCache:
         return sorted(self._slots)
 
     def held_pages(self, group: int = 0) -> int:
-        return self.n_pages - self.pools[group].free_count
+        return self.pools[group].n_pages - self.pools[group].free_count
 
     # ---- a step ------------------------------------------------------------
     def _first_needed_page(self, g: int, length: int) -> int:
@@ -164,27 +184,45 @@ class PagedCache:
             return 0
         return max(0, length - w + 1) // PAGE
 
-    def reserve(self, slots: Sequence[int], n_new: Sequence[int]) -> None:
-        """Pages for ``n_new[i]`` more tokens of ``slots[i]``, all or nothing."""
+    def windowed(self, flag: bool) -> List[int]:
+        """The groups that read a window of keys (``flag`` true) or every key (false)."""
+        return [g for g, spec in enumerate(self.groups) if (spec.window > 0) == flag]
+
+    def reserve(self, slots: Sequence[int], n_new: Sequence[int], groups: Optional[Sequence[int]] = None) -> None:
+        """Pages for ``n_new[i]`` more tokens of ``slots[i]``, all or nothing; ``groups``: in
+        these groups only (a long step reserves the groups that keep every key for all its rows
+        at once, and the windowed ones portion by portion, as their pools are sized)."""
         if len(set(slots)) != len(slots):
             raise CacheError("a slot appears twice in one step")
-        need = [0] * len(self.groups)
+        groups = range(len(self.groups)) if groups is None else list(groups)
+        need = {g: 0 for g in groups}
         for s, n in zip(slots, n_new):
             if n <= 0:
                 raise CacheError("a step must bring at least one token for every sequence")
             sl = self._slot(s)
-            for g in range(len(self.groups)):
-                need[g] += pages_for(sl.length + n) - len(sl.pages[g])
-        for g, n in enumerate(need):
+            for g in groups:
+                need[g] += max(0, pages_for(sl.length + n) - len(sl.pages[g]))
+        for g, n in need.items():
             if n > self.pools[g].free_count:
                 raise CacheError(
                     f"out of cache pages: the step needs {n} more pages of {PAGE} tokens, "
-                    f"{self.pools[g].free_count} of {self.n_pages} are free")
+                    f"{self.pools[g].free_count} of {self.pools[g].n_pages} are free")
         for s, n in zip(slots, n_new):
             sl = self._slots[s]
-            for g in range(len(self.groups)):
+            for g in groups:
                 while len(sl.pages[g]) < pages_for(sl.length + n):
                     sl.pages[g].append(self.pools[g].alloc())
+
+    def trim(self, slots: Sequence[int]) -> None:
+        """Give back the pages that ``slots`` hold beyond their lengths: what a step reserved
+        for rows that did not run."""
+        for s in slots:
+            sl = self._slot(s)
+            for g, pages in enumerate(sl.pages):
+                while len(pages) > pages_for(sl.length):
+                    p = pages.pop()
+                    if p >= 0:
+                        self.pools[g].free(p)
 
     def page_table(self, group: int, slots: Sequence[int], min_width: int = 1) -> np.ndarray:
         """int32 [len(slots), width]: logical page -> physical page, -1 for none."""

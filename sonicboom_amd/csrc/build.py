@@ -39,6 +39,7 @@ FLAGS = [
 CORE_SOURCES = [
     "status.hip", "embed_norm.hip", "elementwise.hip", "gemm_plain.hip", "rope_kv.hip",
     "attention_plain.hip", "sampling.hip", "gemm_skinny.hip", "gemm_stream.hip", "gemm_mfma.hip",
+    "random_fill.hip",
 ]
 HEADERS = ["common.h", "sb_hip.h", "mfma.h"]
 ATTN_SOURCES = ["attention_mfma.hip"]

@@ -243,6 +243,15 @@ int sb_gemm_mfma_slices(int n_rows, int n_out, int n_in, int packed);
 int sb_gemm_mfma_partial_bf16(float *partial, const void *x, const void *w, int n_rows, int n_out,
                               int n_in, int packed, void *stream);
 
+/* Seeded normal weights: elements first .. first + n - 1 (first a multiple of 4) of tensor number
+ * `tensor_index` under `seed`, as float32(mean + std z) (out_kind 0), the same rounded to bfloat16
+ * (1), or the float64 standard normals z themselves (2).  Element e comes from Philox4x32-10 with
+ * the seed as key and the counter (e / 4 low, e / 4 high, tensor_index, 0), words 0 and 1 making the
+ * normals of elements 4c and 4c + 1, words 2 and 3 those of 4c + 2 and 4c + 3 (Box and Muller).  The
+ * host computes the same bits (sonicboom_amd/weights/random_stream.py). */
+int sb_random_normal(void *out, int out_kind, uint64_t n, uint64_t first, uint64_t seed, int tensor_index,
+                     double mean, double std, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -12,9 +12,12 @@ char *error_slot() {
 #define SB_BUILD_FLAGS ""
 #endif
 
+#define SB_STR_(x) #x
+#define SB_STR(x) SB_STR_(x)
+
 extern "C" const char *sb_last_error(void) { return sb::error_slot(); }
 
 extern "C" const char *sb_build_info(void) {
   return "{\"library\": \"sonicboom_amd\", \"target\": \"gfx950\", \"wave\": 64, "
-         "\"page\": 64, \"flags\": \"" SB_BUILD_FLAGS "\"}";
+         "\"page\": " SB_STR(SB_PAGE) ", \"flags\": \"" SB_BUILD_FLAGS "\"}";
 }

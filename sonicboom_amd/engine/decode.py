@@ -24,7 +24,7 @@ import torch
 
 from .. import ops
 from ..cache.paged import CacheError, pages_for
-from .step import StepError
+from .step import ContextLayout, StepError, _Context, row_runs
 
 WIDTH_STEP = 16      # page-table widths are rounded up to this many pages (1024 tokens)
 CAPTURE_AFTER = 2    # kernel-by-kernel steps of a shape before its graph is captured
@@ -47,47 +47,38 @@ def batch_bucket(n: int) -> int:
         p *= 2
 
 
-class _StaticContext:
-    """A decode step's bookkeeping in device buffers whose addresses never change."""
+class _StaticContext(_Context):
+    """A decode step's bookkeeping in device buffers whose addresses never change: the tables of
+    :class:`~sonicboom_amd.engine.step.ContextLayout` for ``batch`` sequences of one row each and
+    page tables ``width`` wide, refilled every step."""
 
     def __init__(self, engine, batch: int, width: int):
         cache = engine.cache
         self.batch, self.width = batch, width
-        self.n_groups = len(cache.groups)
         self.n_rows = self.n_seqs = self.n_wanted = batch
-        self.trace = None
         self.is_decode = True
         self.max_new = 1
-        sizes = [batch, batch, batch, batch + 1, batch, batch, batch, 4 * batch] + [batch * width] * self.n_groups
-        total = sum(sizes)
+        heights = engine.model.row_tiles
+        self.layout = layout = ContextLayout(batch, batch, batch, {h: batch for h in heights},
+                                             [(batch, width)] * len(cache.groups))
         dev = engine.device
         # two pinned staging buffers used in turn: a step never overwrites the one whose copy
         # may still be in flight
-        self._hosts = [torch.zeros(total, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self._hosts = [torch.zeros(layout.total, dtype=torch.int32, pin_memory=True) for _ in range(2)]
         self._turn = 0
-        self.dev = torch.zeros(total, dtype=torch.int32, device=dev)
+        self.dev = torch.zeros(layout.total, dtype=torch.int32, device=dev)
         self.next_ids = torch.zeros(batch, dtype=torch.int32, device=dev)
-        offs = np.concatenate([[0], np.cumsum(sizes)])
-        self._off = offs
-        v = [self.dev[offs[i]:offs[i + 1]] for i in range(len(sizes))]
-        (self.ids, self.row_pos, self.row_seq, self.cu_rows, self.len_before, self.slots, self.want_rows,
-         flat_tiles) = v[:8]
-        self._tiles = flat_tiles.view(-1, 4)       # one row a sequence: the same for every height
-        self._tables = [t.view(batch, width) for t in v[8:]]
-        # the parts that never change for a decode step of this batch size
+        layout.bind(self, self.dev)
+        # the parts that never change for a decode step of this batch size: a row a sequence,
+        # every row wanted, and whatever the height a run is that one row
         ar = np.arange(batch, dtype=np.int32)
         for h in self._hosts:
             n = h.numpy()
-            n[offs[2]:offs[3]] = ar
-            n[offs[3]:offs[4]] = np.arange(batch + 1, dtype=np.int32)
-            n[offs[6]:offs[7]] = ar
-            n[offs[7]:offs[8]] = np.stack([ar, np.ones_like(ar), ar, np.zeros_like(ar)], axis=1).reshape(-1)
-
-    def page_table(self, group: int) -> torch.Tensor:
-        return self._tables[group]
-
-    def row_tiles(self, height: int) -> torch.Tensor:
-        return self._tiles
+            layout.view(n, "row_seq")[:] = ar
+            layout.view(n, "cu_rows")[:] = np.arange(batch + 1, dtype=np.int32)
+            layout.view(n, "want_rows")[:] = ar
+            for height in layout.heights:
+                layout.view(n, ("tiles", height))[:] = row_runs([1] * batch, np.arange(batch + 1), height)
 
     def refresh(self, cache, slots: Sequence[int], tokens: Sequence[int]) -> None:
         """This step's ids, positions and page tables, in one copy to the device.  Fewer
@@ -95,18 +86,20 @@ class _StaticContext:
         page at all (they store nothing and attend to nothing; their logits are not read)."""
         host = self._hosts[self._turn]
         self._turn ^= 1
-        n, o = host.numpy(), self._off
+        n, layout = host.numpy(), self.layout
         live = len(slots)
         lengths = np.zeros(self.batch, dtype=np.int32)
         lengths[:live] = [cache.length(s) for s in slots]
-        n[o[0]:o[0] + live] = np.asarray(tokens, dtype=np.int32)
-        n[o[0] + live:o[1]] = 0
-        n[o[1]:o[2]] = lengths
-        n[o[4]:o[5]] = lengths
-        n[o[5]:o[5] + live] = np.asarray(slots, dtype=np.int32)
-        n[o[5] + live:o[6]] = slots[0]
-        for g in range(self.n_groups):
-            table = n[o[8 + g]:o[9 + g]].reshape(self.batch, self.width)
+        ids = layout.view(n, "ids")
+        ids[:live] = np.asarray(tokens, dtype=np.int32)
+        ids[live:] = 0
+        layout.view(n, "row_pos")[:] = lengths
+        layout.view(n, "len_before")[:] = lengths
+        slot_row = layout.view(n, "slots")
+        slot_row[:live] = np.asarray(slots, dtype=np.int32)
+        slot_row[live:] = slots[0]
+        for g in range(layout.n_groups):
+            table = layout.view(n, ("table", g))
             table[:live] = cache.page_table(g, slots, min_width=self.width)
             table[live:] = -1
         self.max_len_after = int(lengths.max()) + 1

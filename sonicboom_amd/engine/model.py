@@ -92,20 +92,23 @@ class DecoderModel:
             tensors.close()
 
     @classmethod
-    def from_random(cls, config, seed: int, dtype: str = "bfloat16", device=None, fast_kernels: bool = True):
-        """Random weights drawn on the device, for a typed configuration or a config.json dict."""
+    def from_random(cls, config, seed: int, dtype: str = "bfloat16", device=None, fast_kernels: bool = True,
+                    stored: Optional[str] = None):
+        """Random weights drawn on the device, for a typed configuration or a config.json dict: the
+        model that a folder written by ``write_random_model(folder, config, seed, stored or dtype)``
+        gives when it is loaded as ``dtype``, to the bit."""
         d = config if isinstance(config, dict) else config.to_dict()
         arch = architecture_of(d)
         cfg = arch.config_class.from_dict(d)
         spec = arch.build_spec(cfg)
         dev = require_gpu(device)
-        tensors = random_source(spec, seed, dtype, dev)       # drawn as the parts ask for them
+        tensors = random_source(spec, seed, dtype, dev, stored)       # drawn as the parts ask for them
         return cls(spec, tensors, Runtime(dev, DTYPES[dtype], fast_kernels), cfg)
 
     # ---- cache -----------------------------------------------------------------
-    def new_cache(self, max_tokens: int, max_slots: Optional[int] = None) -> PagedCache:
+    def new_cache(self, max_tokens: int, max_slots: Optional[int] = None, step_rows: int = 0) -> PagedCache:
         return PagedCache(self.groups, max_tokens, self.rt.cache_dtype, self.rt.device,
-                          self.state_specs, max_slots)
+                          self.state_specs, max_slots, step_rows=step_rows)
 
     def bindings(self, cache: PagedCache) -> List[LayerBinding]:
         out = []

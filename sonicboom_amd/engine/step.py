@@ -60,7 +60,72 @@ class StepEntry:
     want: Sequence[int] = ()        # indices into ``tokens`` whose logits are wanted
 
 
-class StepContext:
+class ContextLayout:
+    """The int32 tables of a step and where each lies in the one buffer that carries them to the
+    device: the single description of that buffer, for a step whose tables are computed on the
+    spot (:class:`StepContext`) and for the decode loop's fixed buffers that are refilled every
+    step (``engine/decode.py``).
+
+    Fields, in order: ``ids``, ``row_pos``, ``row_seq`` [rows]; ``cu_rows`` [seqs + 1];
+    ``len_before``, ``slots`` [seqs]; ``want_rows`` [wanted]; for every row-tile height ``h``
+    that a mixer of the model has asked for, ``("tiles", h)`` [n, 4] = (first row, rows <= h,
+    sequence, 0); for every cache group ``g``, ``("table", g)`` [seqs, width]."""
+
+    def __init__(self, n_rows: int, n_seqs: int, n_wanted: int, tiles, tables):
+        """``tiles``: {height: number of runs}; ``tables``: per cache group (rows, width)."""
+        self.heights = sorted(int(h) for h in tiles)
+        self.shapes = {"ids": (n_rows,), "row_pos": (n_rows,), "row_seq": (n_rows,), "cu_rows": (n_seqs + 1,),
+                       "len_before": (n_seqs,), "slots": (n_seqs,), "want_rows": (n_wanted,)}
+        for h in self.heights:
+            self.shapes[("tiles", h)] = (int(tiles[h]), 4)
+        for g, shape in enumerate(tables):
+            self.shapes[("table", g)] = tuple(int(n) for n in shape)
+        self.n_groups = len(tables)
+        self.offsets, off = {}, 0
+        for key, shape in self.shapes.items():
+            self.offsets[key] = off
+            off += int(np.prod(shape, dtype=np.int64))
+        self.total = off
+
+    def view(self, buffer, key):
+        """The part of ``buffer`` (a torch tensor or NumPy array of ``total`` int32) that holds ``key``."""
+        shape = self.shapes[key]
+        off = self.offsets[key]
+        return buffer[off:off + int(np.prod(shape, dtype=np.int64))].reshape(shape)
+
+    def bind(self, ctx, device_buffer) -> None:
+        """Give ``ctx`` its device tensors as views of ``device_buffer``."""
+        for name in ("ids", "row_pos", "row_seq", "cu_rows", "len_before", "slots", "want_rows"):
+            setattr(ctx, name, self.view(device_buffer, name))
+        ctx._tiles = {h: self.view(device_buffer, ("tiles", h)) for h in self.heights}
+        ctx._tables = [self.view(device_buffer, ("table", g)) for g in range(self.n_groups)]
+
+
+def row_runs(n_new: Sequence[int], cu, height: int) -> np.ndarray:
+    """int32 [n, 4]: the rows of a step in runs of up to ``height`` consecutive rows of one
+    sequence, as (first row, rows, sequence, 0)."""
+    runs = [(int(cu[i]) + r0, min(height, n - r0), i, 0) for i, n in enumerate(n_new) for r0 in range(0, n, height)]
+    return np.asarray(runs, dtype=np.int32).reshape(-1, 4)
+
+
+class _Context:
+    """What the parts read of a step's bookkeeping (see :class:`StepContext`)."""
+
+    trace = None            # set by the engine while a tracer listens
+
+    def page_table(self, group: int) -> torch.Tensor:
+        return self._tables[group]
+
+    def row_tiles(self, height: int) -> torch.Tensor:
+        """The step's rows in runs of up to ``height`` consecutive rows of one sequence."""
+        try:
+            return self._tiles[int(height)]
+        except KeyError:
+            raise StepError(f"no mixer of the model has asked for row tiles of {height} rows "
+                            f"(a mixer asks with its row_tile attribute; asked for: {sorted(self._tiles)})") from None
+
+
+class StepContext(_Context):
     """Row and sequence bookkeeping of one step, on the host and on the device.
 
     Device tensors (int32): ``ids`` [rows], ``row_pos`` [rows] absolute
@@ -73,7 +138,7 @@ class StepContext:
     ``page_table(group)`` [seqs, pages].
     Host: ``n_rows``, ``n_seqs``, ``n_new`` list, ``lengths_before`` list,
     ``is_decode`` (every sequence brings one token), ``max_new``,
-    ``max_len_after``.
+    ``max_len_after``, ``host_row_pos``.
     """
 
     def __init__(self, cache: PagedCache, entries: Sequence[StepEntry], device, row_tiles: Sequence[int] = ()):
@@ -87,49 +152,32 @@ class StepContext:
         self.max_len_after = max(l + n for l, n in zip(self.lengths_before, self.n_new))
         cu = np.zeros(self.n_seqs + 1, dtype=np.int32)
         cu[1:] = np.cumsum(self.n_new)
-        ids = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries]).astype(np.int32)
         row_seq = np.repeat(np.arange(self.n_seqs, dtype=np.int32), self.n_new)
         row_pos = (np.arange(self.n_rows, dtype=np.int32) - cu[row_seq]
                    + np.asarray(self.lengths_before, dtype=np.int32)[row_seq]).astype(np.int32)
         want = [int(cu[i]) + int(w) for i, e in enumerate(entries) for w in e.want]
         self.n_wanted = len(want)
-        tables = [cache.page_table(g, self.slot_list) for g in range(len(cache.groups))]
-        # runs of up to h consecutive rows of one sequence: (first row, rows, sequence, 0)
-        heights = sorted({int(h) for h in row_tiles})
-        tiles = [np.asarray([(int(cu[i]) + r0, min(h, n - r0), i, 0)
-                             for i, n in enumerate(self.n_new) for r0 in range(0, n, h)], dtype=np.int32)
-                 for h in heights]
-        parts = [ids, row_pos, row_seq, cu, np.asarray(self.lengths_before, dtype=np.int32),
-                 np.asarray(self.slot_list, dtype=np.int32), np.asarray(want, dtype=np.int32)]
-        parts += [t.reshape(-1) for t in tiles]
-        parts += [t.reshape(-1) for t in tables]
-        sizes = [p.size for p in parts]
+        values = {
+            "ids": np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries]).astype(np.int32),
+            "row_pos": row_pos, "row_seq": row_seq, "cu_rows": cu,
+            "len_before": np.asarray(self.lengths_before, dtype=np.int32),
+            "slots": np.asarray(self.slot_list, dtype=np.int32), "want_rows": np.asarray(want, dtype=np.int32),
+        }
+        for h in sorted({int(h) for h in row_tiles}):
+            values[("tiles", h)] = row_runs(self.n_new, cu, h)
+        for g in range(len(cache.groups)):
+            values[("table", g)] = cache.page_table(g, self.slot_list)
+        layout = ContextLayout(self.n_rows, self.n_seqs, self.n_wanted,
+                               {k[1]: len(v) for k, v in values.items() if isinstance(k, tuple) and k[0] == "tiles"},
+                               [values[("table", g)].shape for g in range(len(cache.groups))])
         # One pinned staging buffer, one copy to the device, views into it.
-        host = torch.empty(sum(sizes), dtype=torch.int32, pin_memory=(torch.device(device).type == "cuda"))
-        host.numpy()[:] = np.concatenate(parts) if parts else np.zeros(0, np.int32)
-        dev = host.to(device, non_blocking=True)
+        host = torch.empty(layout.total, dtype=torch.int32, pin_memory=(torch.device(device).type == "cuda"))
+        flat = host.numpy()
+        for key, v in values.items():
+            layout.view(flat, key)[...] = v
         self._host = host
-        views, off = [], 0
-        for n in sizes:
-            views.append(dev[off:off + n])
-            off += n
-        (self.ids, self.row_pos, self.row_seq, self.cu_rows, self.len_before, self.slots,
-         self.want_rows) = views[:7]
-        self._tiles = {h: v.view(-1, 4) for h, v in zip(heights, views[7:7 + len(heights)])}
-        self._tables = [v.view(t.shape) for v, t in zip(views[7 + len(heights):], tables)]
+        layout.bind(self, host.to(device, non_blocking=True))
         self.host_row_pos = row_pos
-        self.trace = None            # set by the engine while a tracer listens
-
-    def page_table(self, group: int) -> torch.Tensor:
-        return self._tables[group]
-
-    def row_tiles(self, height: int) -> torch.Tensor:
-        """The step's rows in runs of up to ``height`` consecutive rows of one sequence."""
-        try:
-            return self._tiles[int(height)]
-        except KeyError:
-            raise StepError(f"no mixer of the model has asked for row tiles of {height} rows "
-                            f"(a mixer asks with its row_tile attribute; asked for: {sorted(self._tiles)})") from None
 
 
 class Engine:
@@ -144,7 +192,7 @@ class Engine:
         own = int(getattr(model.spec, "max_positions", 0) or 0)
         self.max_positions = own if max_positions is None else int(max_positions)
         self.device = model.rt.device
-        self.cache = model.new_cache(max_tokens, max_slots)
+        self.cache = model.new_cache(max_tokens, max_slots, step_rows=self.max_step_rows)
         self.bindings = model.bindings(self.cache)
         self.use_graphs = True
         self._loop = None
@@ -202,32 +250,54 @@ class Engine:
         A step of more than ``max_step_rows`` rows runs in portions, one after the other from
         the cache the earlier ones left: whole sequences while they fit, a sequence cut where
         the portion is full.  The logits come back in the order of the entries and of their
-        ``want`` all the same."""
+        ``want`` all the same.  When a portion fails (a kernel refuses a size, memory runs out),
+        the portions before it stay in the cache, the sequences' lengths count them, the pages
+        reserved for the rest are given back and the logits of the step are lost: free the slots,
+        or look at ``length(slot)`` and feed the remaining tokens again."""
         entries = [e if isinstance(e, StepEntry) else StepEntry(*e) for e in entries]
+        cache = self.cache
+        slots = [e.slot for e in entries]
+        n_new = [len(e.tokens) for e in entries]
+        portions = portion_rows(n_new, self.max_step_rows)
         try:
             self._check(entries)
-            slots = [e.slot for e in entries]
-            n_new = [len(e.tokens) for e in entries]
-            self.cache.reserve(slots, n_new)
+            # all or nothing: the groups that keep every key take the pages of all rows now;
+            # windowed groups, whose pools hold a window and one portion a sequence, take theirs
+            # portion by portion (a single portion: everything at once)
+            cache.reserve(slots, n_new, None if len(portions) == 1 else cache.windowed(False))
         except CacheError as e:
             raise StepError(str(e)) from None
-        portions = portion_rows(n_new, self.max_step_rows)
         if len(portions) == 1:
-            ctx = StepContext(self.cache, entries, self.device, self.model.row_tiles)
-            logits = self.forward(ctx)
-            self.cache.advance(slots, n_new)
+            ctx = StepContext(cache, entries, self.device, self.model.row_tiles)
+            try:
+                logits = self.forward(ctx)
+            except BaseException:
+                cache.trim(slots)               # the rows did not run: their pages go back
+                raise
+            cache.advance(slots, n_new)
             return logits
         pieces, place = [], []          # place[i] = (entry, index in its want) of output row i
-        for portion in portions:
-            sub = []
-            for i, a, b in portion:
-                e = entries[i]
-                picked = [(k, w - a) for k, w in enumerate(e.want) if a <= w < b]
-                sub.append(StepEntry(e.slot, e.tokens[a:b], [w for _, w in picked]))
-                place += [(i, k) for k, _ in picked]
-            ctx = StepContext(self.cache, sub, self.device, self.model.row_tiles)
-            pieces.append(self.forward(ctx))
-            self.cache.advance([e.slot for e in sub], [len(e.tokens) for e in sub])
+        try:
+            for portion in portions:
+                sub = []
+                for i, a, b in portion:
+                    e = entries[i]
+                    picked = [(k, w - a) for k, w in enumerate(e.want) if a <= w < b]
+                    sub.append(StepEntry(e.slot, e.tokens[a:b], [w for _, w in picked]))
+                    place += [(i, k) for k, _ in picked]
+                sub_slots, sub_new = [e.slot for e in sub], [len(e.tokens) for e in sub]
+                cache.reserve(sub_slots, sub_new, cache.windowed(True))
+                ctx = StepContext(cache, sub, self.device, self.model.row_tiles)
+                pieces.append(self.forward(ctx))
+                cache.advance(sub_slots, sub_new)
+        except BaseException as e:
+            # A portion failed.  The portions before it have run: their rows are in the cache and
+            # the sequences' lengths say so; what was reserved for the rows that did not run goes
+            # back.  The caller frees the slots or feeds the remaining tokens again.
+            cache.trim(slots)
+            if isinstance(e, CacheError):
+                raise StepError(str(e)) from None
+            raise
         logits = torch.cat(pieces, dim=0)
         order = sorted(range(len(place)), key=place.__getitem__)
         if order != list(range(len(place))):
@@ -239,7 +309,7 @@ class Engine:
         their run order, and for the wanted rows the final norm and the head."""
         model = self.model
         tracer = self.tracer
-        x = model.embedding.forward(ctx.ids)
+        x = model.embedding.forward(ctx.ids, ctx)
         if tracer is not None:
             tracer("embedding", x)
         h = None

@@ -32,7 +32,7 @@ class _Hints(threading.local):
 
 _hints = _Hints()
 
-PAGE = 64          # tokens per cache page; SB_PAGE of csrc/sb_hip.h
+from ..csrc.header import PAGE          # tokens per cache page: SB_PAGE of csrc/sb_hip.h
 MAX_CANDIDATES = 256
 
 _DT = {torch.float32: 0, torch.bfloat16: 1}
@@ -367,6 +367,29 @@ def read_bandwidth(n_bytes: int = 1 << 30, blocks: int = 512, repeats: int = 5, 
         e1.synchronize()
         best = max(best, n_bytes / (e0.elapsed_time(e1) * 1e-3))
     return best
+
+
+_RANDOM_KINDS = {torch.float32: 0, torch.bfloat16: 1, torch.float64: 2}
+
+
+def random_normal(shape, seed: int, tensor_index: int, mean: float = 0.0, std: float = 1.0,
+                  dtype: torch.dtype = torch.float32, device="cuda:0", first: int = 0) -> torch.Tensor:
+    """Seeded normal values of ``shape`` drawn on the device: float32(mean + std z) as float32 or
+    rounded to bfloat16, or (``dtype`` float64) the standard normals z themselves.  Element e of
+    the tensor (counted from ``first``, a multiple of four) is a function of (seed, tensor_index,
+    e) alone, the one the host computes in :mod:`sonicboom_amd.weights.random_stream`."""
+    try:
+        kind = _RANDOM_KINDS[dtype]
+    except KeyError:
+        raise KernelLibraryError(f"random values come as float32, bfloat16 or float64, not {dtype}") from None
+    out = torch.empty(tuple(shape), dtype=dtype, device=device)
+    if not out.is_cuda:
+        raise KernelLibraryError("random values are drawn on the GPU (the host has its own function for them)")
+    lib = library.core()
+    with torch.cuda.device(out.device):
+        check(lib.sb_random_normal(_p(out), kind, out.numel(), int(first), int(seed) & (2 ** 64 - 1),
+                                   int(tensor_index), float(mean), float(std), _stream()))
+    return out
 
 
 # --------------------------------------------------------------------------

@@ -37,6 +37,7 @@ _CORE_SIGNATURES = {
     "sb_mask_logits": [_P, _I, _I, _P, _I, _P],
     "sb_draw": [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I, c_double, c_uint64, _P],
     "sb_draw_after": [_P, _P, _P, _P, _I, _I, _I, _I, _F, _I, c_double, c_uint64, _P],
+    "sb_random_normal": [_P, _I, c_uint64, c_uint64, c_uint64, _I, c_double, c_double, _P],
 }
 # Entry points of later kernels; declared when the library has them.
 _OPTIONAL_SIGNATURES = {

@@ -25,7 +25,7 @@ copy in the activation type, ``ctx`` the step's
                 optionally ``first_norm``, the norm the block starts with (the block before
                 may then hand over ``h`` = first_norm(x) from its last pass), and calls of
                 ``ctx.trace(name, x)`` after its mixer and feed-forward when that is set.
-* **embedding** ``forward(ids) -> x``
+* **embedding** ``forward(ids, ctx) -> x`` (``ctx.row_pos`` for embeddings that add a position's row)
 * **head**      ``forward(h) -> float32 logits [rows, vocab]``
 """
 from __future__ import annotations

@@ -35,7 +35,9 @@ class Embedding(Part):
         self.table = tensors["table"]
         self.vocab, self.width = self.table.shape
 
-    def forward(self, ids: torch.Tensor) -> torch.Tensor:
+    def forward(self, ids: torch.Tensor, ctx=None) -> torch.Tensor:
+        """``ctx``: the step's context, for embeddings that look at more than the ids (the
+        rows' positions, say); this one does not."""
         return ops.embed(self.table, ids)
 
 

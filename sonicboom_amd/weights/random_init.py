@@ -1,13 +1,16 @@
 """Seeded random weights.
 
 ``write_random_model`` makes a model folder (config.json, model.safetensors)
-from a configuration and a seed; ``random_tensors`` makes the same kind of
-weights straight on a device, for sizes too large to route through a file.
+from a configuration and a seed; ``random_source`` draws the same weights
+straight on a device, for sizes too large to route through a file.
 Each tensor is drawn as mean + std * N(0,1) with the (mean, std) of its
 :class:`~sonicboom_amd.parts.spec.TensorSpec`: projections and biases
-N(0, 0.02), norm weights 1 + N(0, 0.02).  In a folder, tensor number i of the
-spec comes from a Philox generator keyed by (seed, i), so the file does not
-depend on the order or the machine that wrote it.
+N(0, 0.02), norm weights 1 + N(0, 0.02).  Element e of tensor number i of the
+spec is a function of (seed, i, e) alone (:mod:`.random_stream`: Philox4x32-10
+keyed by the seed, Box and Muller), computed to the same bits by NumPy here and
+by the kernel ``sb_random_normal`` on the GPU: a folder written from (config,
+seed, dtype) and a model drawn on the device from the same three are the same
+model, whatever the order, the machine or the side that drew it.
 """
 from __future__ import annotations
 
@@ -20,31 +23,45 @@ import torch
 
 from ..config.registry import architecture_of
 from ..parts.spec import ModelSpec
+from . import random_stream
 from .safetensors_io import f32_to_bf16_bits, write_safetensors
 
 
-def _draw(seed: int, index: int, shape, mean: float, std: float) -> np.ndarray:
-    gen = np.random.Generator(np.random.Philox(key=[int(seed) & (2**64 - 1), index]))
-    a = gen.standard_normal(size=shape, dtype=np.float32)
-    return (a * np.float32(std) + np.float32(mean)).astype(np.float32)
+# tensors of at least this many elements are drawn by the GPU's kernel when a folder is written
+# on a machine that has one (same bits, a few hundred times faster than NumPy)
+DEVICE_DRAW_FROM = 1 << 22
 
 
-def random_arrays(spec: ModelSpec, seed: int) -> Dict[str, np.ndarray]:
+def _draw(seed: int, index: int, shape, mean: float, std: float, device=None) -> np.ndarray:
+    n = int(np.prod(shape, dtype=np.int64)) if len(shape) else 1
+    if device is not None and n >= DEVICE_DRAW_FROM:
+        from .. import ops
+        return ops.random_normal(shape, seed, index, mean, std, torch.float32, device).cpu().numpy()
+    return random_stream.draw(seed, index, shape, mean, std)
+
+
+def random_arrays(spec: ModelSpec, seed: int, device=None) -> Dict[str, np.ndarray]:
     """float32 arrays (int32 zeros for integer tables) for every tensor of the spec."""
-    out = {}
+    return dict(iter_random_arrays(spec, seed, device))
+
+
+def iter_random_arrays(spec: ModelSpec, seed: int, device=None):
+    """(name, array) for every tensor of the spec, one at a time: float32 arrays, int32 zeros for
+    integer tables.  ``device``: a GPU that draws the large tensors (same bits as the host)."""
     for i, t in enumerate(spec.all_tensors()):
         if t.kind == "int":
-            out[t.name] = np.zeros(t.shape, dtype=np.int32)
+            yield t.name, np.zeros(t.shape, dtype=np.int32)
         else:
-            out[t.name] = _draw(seed, i, t.shape, *t.init)
-    return out
+            yield t.name, _draw(seed, i, t.shape, *t.init, device=device)
 
 
 def write_random_model(folder: str, config, seed: int, dtype: str = "bfloat16",
-                       float32_tensors=()) -> ModelSpec:
+                       float32_tensors=(), device="auto") -> ModelSpec:
     """Write ``config.json`` and ``model.safetensors`` for a typed configuration
     (or a config.json dict).  ``dtype`` is the stored type of floating tensors;
-    names in ``float32_tensors`` are stored in float32 regardless."""
+    names in ``float32_tensors`` are stored in float32 regardless.  ``device``: the GPU that
+    draws the large tensors ("auto": the first one if there is one; None: the host draws all);
+    the file is the same either way."""
     if dtype not in ("bfloat16", "float32"):
         raise ValueError("stored dtype must be bfloat16 or float32")
     d = config if isinstance(config, dict) else config.to_dict()
@@ -57,8 +74,11 @@ def write_random_model(folder: str, config, seed: int, dtype: str = "bfloat16",
     with open(os.path.join(folder, "config.json"), "w") as f:
         json.dump(d, f, indent=2, sort_keys=True)
 
+    if device == "auto":
+        device = "cuda:0" if torch.cuda.is_available() else None
+
     def entries():
-        for name, a in random_arrays(spec, seed).items():
+        for name, a in iter_random_arrays(spec, seed, device):
             if a.dtype == np.int32:
                 yield name, "I32", a
             elif dtype == "float32" or name in float32_tensors:
@@ -70,29 +90,31 @@ def write_random_model(folder: str, config, seed: int, dtype: str = "bfloat16",
     return spec
 
 
-def random_source(spec: ModelSpec, seed: int, dtype: str, device):
+def random_source(spec: ModelSpec, seed: int, dtype: str, device, stored=None):
     """The spec's tensors drawn on ``device`` as they are asked for (a model of 145 GB is then
     built block by block without its row-major weights ever standing whole beside the packed
-    ones).  Tensor number i of the spec comes from torch's generator seeded by (seed, i): the
-    values do not depend on the order of asking.  Another stream of numbers than the folder
-    writer's, the same distributions."""
+    ones).  Tensor number i of the spec is drawn by ``sb_random_normal`` under (seed, i): the
+    values do not depend on the order of asking, and they are the bits that
+    :func:`write_random_model` stores for the same (configuration, seed, dtype).  ``stored``
+    (default: ``dtype``) is the type such a folder would be stored in: "bfloat16" with a ``dtype``
+    of "float32" gives the float32 model of a bfloat16 folder."""
+    from .. import ops
     from .loader import LazyTensors
-    tdt = torch.float32 if dtype == "float32" else torch.bfloat16
+    out_dt = torch.float32 if dtype == "float32" else torch.bfloat16
+    tdt = out_dt if stored is None else (torch.float32 if stored == "float32" else torch.bfloat16)
     specs = {t.name: (i, t) for i, t in enumerate(spec.all_tensors())}
 
     def make(name):
         i, t = specs[name]
         if t.kind == "int":
             return torch.zeros(t.shape, dtype=torch.int32, device=device)
-        gen = torch.Generator(device=device)
-        gen.manual_seed((int(seed) * 1000003 + i) & (2**63 - 1))
         mean, std = t.init
-        a = torch.empty(t.shape, dtype=torch.float32, device=device)
-        a.normal_(mean, std, generator=gen)
-        return a.to(tdt)
+        if torch.device(device).type == "cpu":          # the host's own function: the same bits
+            return torch.from_numpy(random_stream.draw(seed, i, t.shape, mean, std)).to(tdt).to(out_dt)
+        return ops.random_normal(t.shape, seed, i, mean, std, tdt, device).to(out_dt)
     return LazyTensors(specs, make)
 
 
-def random_tensors(spec: ModelSpec, seed: int, dtype: str, device) -> Dict[str, torch.Tensor]:
+def random_tensors(spec: ModelSpec, seed: int, dtype: str, device, stored=None) -> Dict[str, torch.Tensor]:
     """All of :func:`random_source` at once, as a dict."""
-    return random_source(spec, seed, dtype, device).materialize()
+    return random_source(spec, seed, dtype, device, stored).materialize()

@@ -62,5 +62,14 @@ def test_real_layer_sizes(folder, dtype):
         for i, (r, g) in enumerate(zip(reqs, got)):
             assert_logits_close(g, plain_logits(folder, r), dtype, f"batch of {n_req}, request {i}", sharp="wide")
         assert eng.cache.held_pages() == 0 and not eng.cache.live_slots
-    del eng, model
+    # the same model drawn on the device (the folder's seed and stored type): the same bits
+    from sonicboom_amd.engine import StepEntry
+    drawn = Engine(DecoderModel.from_random(dict(CONFIG), 4242, dtype, stored="bfloat16"), 128)
+    logits = []
+    for e in (eng, drawn):
+        s = e.alloc_slot()
+        logits.append(e.step([StepEntry(s, one, range(len(one)))]).cpu())
+        e.free_slot(s)
+    assert torch.equal(logits[0], logits[1]), "the model drawn on the device is not the folder's"
+    del eng, model, drawn
     torch.cuda.empty_cache()
