@@ -531,6 +531,27 @@ def main() -> int:
         curve[f"d{depth}"] = entry
         print(f"[bench] depth {depth}: {entry}", file=sys.stderr, flush=True)
 
+    # ---- prefix reuse: a 512-token prefix is in the cache, 64 new tokens come, time to the first token ----
+    prefix_reuse = None
+    if depths:
+        from sonicboom_amd.api import Model
+        session = Model(model).session(max_tokens=64 * 32)
+        base = random_prompts([512])[0]
+        session.generate([base], max_tokens=1, stop_tokens=[], keep=True)
+        with_reuse, whole = [], []
+        for i in range(6):
+            new = base + random_prompts([64])[0]
+            with_reuse.append(sync_time(lambda: session.generate([new], max_tokens=1, stop_tokens=[], keep=True)))
+            assert session.reused == [512]
+        session.forget()
+        for i in range(4):
+            new = base + random_prompts([64])[0]
+            whole.append(sync_time(lambda: session.generate([new], max_tokens=1, stop_tokens=[])))
+        prefix_reuse = {"prefix": 512, "new": 64, "ttft_ms": round(statistics.median(with_reuse[1:]) * 1e3, 3),
+                        "ttft_ms_without_reuse": round(statistics.median(whole[1:]) * 1e3, 3)}
+        print(f"[bench] prefix reuse {prefix_reuse}", file=sys.stderr, flush=True)
+        del session
+
     line = {
         "metric": f"decode tokens/s, {model_name} sizes, batch {a.batch}, {PROMPT}-token cached prompts",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
@@ -542,6 +563,8 @@ def main() -> int:
     }
     if curve:
         line["curve"] = curve
+    if prefix_reuse:
+        line["prefix_reuse"] = prefix_reuse
     result_lines(line)
     print(json.dumps(line), flush=True)
     return 0
@@ -561,6 +584,10 @@ def result_lines(line, out=sys.stderr):
               f"flops_frac={pre['frac']}{tail}", file=out)
     for name, v in (line.get("points") or {}).items():
         print(f"RESULT metric={name} value={v}{tail}", file=out)
+    reuse = line.get("prefix_reuse")
+    if reuse:
+        print(f"RESULT metric=prefix_reuse_ttft_ms prefix={reuse['prefix']} new={reuse['new']} value={reuse['ttft_ms']} "
+              f"without_reuse={reuse['ttft_ms_without_reuse']}{tail}", file=out)
     out.flush()
 
 

@@ -17,6 +17,7 @@ from __future__ import annotations
 from typing import Callable, Iterable, List, Optional, Sequence
 
 from .engine import DecoderModel, Engine, StepEntry, generate
+from .engine.prefix import KeptSequences
 from .sampling import SamplingParams
 
 
@@ -60,6 +61,8 @@ class Session:
                  max_positions: Optional[int] = None):
         self.model = model
         self.engine = Engine(model.decoder, max_tokens, max_slots, max_positions=max_positions)
+        self.kept = KeptSequences(self.engine)      # sequences the last generate(keep=True) left
+        self.keep = False                           # what generate does when it is not told
 
     def alloc_slot(self) -> int:
         return self.engine.alloc_slot()
@@ -76,11 +79,32 @@ class Session:
                  repeat_penalty: float = 1.0, repeat_last_n: int = 64, presence_penalty: float = 0.0,
                  frequency_penalty: float = 0.0, stop_tokens: Optional[Iterable[int]] = None,
                  max_batch: int = 64, callback: Optional[Callable] = None,
-                 allowed: Optional[Callable] = None) -> List[List[int]]:
+                 allowed: Optional[Callable] = None, keep: Optional[bool] = None) -> List[List[int]]:
         """``allowed(i, history)`` returns the bitmap of the ids request i may choose next (bit
-        i & 7 of byte i >> 3 for id i; None: any): the mask of constrained decoding."""
+        i & 7 of byte i >> 3 for id i; None: any): the mask of constrained decoding.
+
+        ``keep`` (default: the session's ``keep`` attribute): the requests' sequences stay in
+        the cache when they end, and a prompt of the next call that starts with the tokens of
+        one of them feeds only the rest (prefix reuse: a conversation that goes on; at most all
+        but the prompt's last token are reused).  ``reused`` then tells how many tokens of each
+        prompt were not fed again.  The produced tokens do not depend on it.  A call without
+        ``keep`` frees what an earlier one kept."""
+        keep = self.keep if keep is None else bool(keep)
         params = SamplingParams(temperature=temperature, top_p=top_p, top_k=top_k, seed=seed,
                                 max_tokens=max_tokens, min_p=min_p, repeat_penalty=repeat_penalty,
                                 repeat_last_n=repeat_last_n, presence_penalty=presence_penalty,
                                 frequency_penalty=frequency_penalty)
-        return generate(self.engine, prompts, params, stop_tokens, max_batch, callback, allowed=allowed)
+        if not keep:
+            self.forget()
+        return generate(self.engine, prompts, params, stop_tokens, max_batch, callback, allowed=allowed,
+                        kept=self.kept if keep else None)
+
+    @property
+    def reused(self) -> List[int]:
+        """Per prompt of the last ``generate(keep=True)``: the tokens taken from a kept sequence."""
+        return list(self.kept.reused)
+
+    def forget(self) -> None:
+        """Free the sequences that ``generate(keep=True)`` has left in the cache."""
+        self.kept.drop_all()
+        self.kept.reused = []

@@ -173,6 +173,13 @@ class PagedCache:
     def live_slots(self) -> List[int]:
         return sorted(self._slots)
 
+    def free_pages(self) -> int:
+        """Pages that every group can still hand out (the least over the groups' pools)."""
+        return min((p.free_count for p in self.pools), default=self.n_pages)
+
+    def free_slots(self) -> int:
+        return len(self._free_slots)
+
     def held_pages(self, group: int = 0) -> int:
         return self.pools[group].n_pages - self.pools[group].free_count
 
@@ -245,6 +252,35 @@ class PagedCache:
                     if pages[i] >= 0:
                         self.pools[g].free(pages[i])
                         pages[i] = -1
+
+    # ---- taking a sequence back ----------------------------------------------
+    def can_truncate(self, slot: int, length: int) -> bool:
+        """Whether ``slot`` can go back to its first ``length`` tokens: not when a mixer keeps
+        per-sequence state (a recurrence cannot be run backwards), and not below what a windowed
+        group still holds (the pages its window has left are gone)."""
+        sl = self._slot(slot)
+        if not 0 <= length <= sl.length:
+            return False
+        if length == sl.length:
+            return True
+        if self.state:
+            return False
+        return all(self._first_needed_page(g, sl.length) == self._first_needed_page(g, length)
+                   for g in range(len(self.groups)))
+
+    def truncate(self, slot: int, length: int) -> None:
+        """Forget all but the first ``length`` tokens of ``slot``: the next step's rows start at
+        position ``length`` and see the keys before it, as if the later tokens had never been
+        fed.  Pages past the new end go back to their pools (what a kept page holds past the new
+        end is never read: a row sees keys up to its own position only)."""
+        if not self.can_truncate(slot, length):
+            sl = self._slot(slot)
+            raise CacheError(f"slot {slot} holds {sl.length} tokens and cannot go back to {length}"
+                             + (": its per-sequence state cannot be taken back" if self.state and 0 <= length < sl.length
+                                else ": a windowed group has given up the keys before it" if 0 <= length < sl.length else ""))
+        sl = self._slots[slot]
+        sl.length = length
+        self.trim([slot])
 
     # ---- storage -------------------------------------------------------------
     def entry_views(self, entry: int):

@@ -86,6 +86,22 @@ def _generate(session, prompts, sampling, stop, cb_addr, user_addr, out_addr, n_
     return len(outs)
 
 
+def _session_keep(session, on):
+    session.keep = bool(on)
+    if not session.keep:
+        session.forget()
+
+
+def _session_reused(session, out_addr, cap):
+    """Counts of the last generate's reused tokens, copied to out_addr when cap holds them."""
+    counts = session.reused
+    if counts and cap >= len(counts):
+        buf = (ctypes.c_uint64 * len(counts)).from_address(out_addr)
+        for i, n in enumerate(counts):
+            buf[i] = n
+    return len(counts)
+
+
 def _build_info():
     from .. import __version__
     from ..ops import library
@@ -110,5 +126,7 @@ _ENTRIES = {
     "slot_free": lambda s, slot: s.free_slot(int(slot)),
     "step": _step,
     "generate": _generate,
+    "session_keep": _session_keep,
+    "session_reused": _session_reused,
     "build_info": _build_info,
 }

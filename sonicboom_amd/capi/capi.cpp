@@ -392,6 +392,29 @@ boom_status boom_llm_generate(boom_llm_session *session, const boom_token *const
   return st;
 }
 
+boom_status boom_llm_session_keep(boom_llm_session *session, int keep, boom_error **err_out) {
+  if (!live(session)) return fail(err_out, BOOM_ERR_INTERNAL, "boom_llm_session_keep: bad argument");
+  Gil gil;
+  return bridge("session_keep", Py_BuildValue("(Oi)", session->obj, keep ? 1 : 0), nullptr, err_out);
+}
+
+boom_status boom_llm_session_reused(boom_llm_session *session, uint64_t *out, size_t cap, size_t *n_out,
+                                    boom_error **err_out) {
+  if (!live(session) || !n_out || (!out && cap))
+    return fail(err_out, BOOM_ERR_INTERNAL, "boom_llm_session_reused: bad argument");
+  Gil gil;
+  PyObject *res = nullptr;
+  const boom_status st =
+      bridge("session_reused",
+             Py_BuildValue("(OKK)", session->obj, (unsigned long long)(uintptr_t)out, (unsigned long long)cap), &res,
+             err_out);
+  if (st != BOOM_OK) return st;
+  *n_out = (size_t)PyLong_AsUnsignedLongLong(res);
+  Py_DECREF(res);
+  if (*n_out > cap) return fail(err_out, BOOM_ERR_BINDING, "boom_llm_session_reused: the buffer is too small");
+  return BOOM_OK;
+}
+
 const char *boom_error_message(const boom_error *err) { return err ? err->message.c_str() : ""; }
 void boom_error_free(boom_error *err) { delete err; }
 

@@ -122,6 +122,17 @@ boom_status boom_llm_generate(boom_llm_session *session, const boom_token *const
                               boom_llm_batch_token_cb cb, void *user, boom_token *out, uint32_t *n_out,
                               boom_error **err_out);
 
+/* Prefix reuse.  With keep != 0, the sequences of a boom_llm_generate call stay in the cache when
+ * they end, and a prompt of the next call that starts with the tokens of one of them feeds only
+ * the rest (at most all but its last token are reused); sequences that no prompt of the next call
+ * continues are freed when it starts.  keep == 0 (the default) frees what is kept.  The produced
+ * tokens do not depend on it. */
+boom_status boom_llm_session_keep(boom_llm_session *session, int keep, boom_error **err_out);
+/* Per prompt of the last boom_llm_generate call: the tokens that were taken from a kept sequence
+ * instead of being fed again.  Two-call sizing as above. */
+boom_status boom_llm_session_reused(boom_llm_session *session, uint64_t *out, size_t cap, size_t *n_out,
+                                    boom_error **err_out);
+
 /* --- errors, build ----------------------------------------------------------------------- */
 const char *boom_error_message(const boom_error *err);  /* never NULL */
 void boom_error_free(boom_error *err);

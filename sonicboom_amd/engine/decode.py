@@ -139,6 +139,7 @@ class DecodeLoop:
     def close(self) -> None:
         self._graphs.clear()
         self._ctx.clear()
+        self._uses.clear()
 
     def _key(self) -> Tuple[int, int]:
         cache = self.engine.cache
@@ -175,9 +176,12 @@ class DecodeLoop:
         except CacheError as e:
             raise StepError(str(e)) from None
         key = self._key()
-        ctx = self._ctx.get(key)
+        ctx = self._ctx.pop(key, None)
         if ctx is None:
-            ctx = self._ctx[key] = _StaticContext(eng, *key)
+            ctx = _StaticContext(eng, *key)
+            while len(self._ctx) >= MAX_GRAPHS:          # the shape unused for longest goes, with
+                self._forget(next(iter(self._ctx)))      # its pinned buffers and its recordings
+        self._ctx[key] = ctx                             # most recently used last
         ctx.refresh(cache, self.slots, tokens)
         gkey = (*key, choose)
         entry = self._graphs.pop(gkey, None)
@@ -188,9 +192,12 @@ class DecodeLoop:
         else:
             logits = eng.forward(ctx)
             self._choose(logits, ctx, choose)
-            n = self._uses[gkey] = self._uses.get(gkey, 0) + 1
+            n = self._uses[gkey] = self._uses.pop(gkey, 0) + 1
             if self.use_graph and n >= CAPTURE_AFTER:
                 self._capture(gkey, ctx, choose)
+                del self._uses[gkey]                     # counted only until it is recorded
+            while len(self._uses) > 4 * MAX_GRAPHS:      # choices seen once or twice and not again
+                del self._uses[next(iter(self._uses))]
         cache.advance(self.slots, ones)
         live = len(self.slots)
         return logits[:live], ctx.next_ids[:live]
@@ -217,8 +224,16 @@ class DecodeLoop:
         while len(self._graphs) >= MAX_GRAPHS:
             oldest = next(iter(self._graphs))
             del self._graphs[oldest]            # its memory pool goes with it
-            self._uses.pop(oldest, None)
+            if not any(k[:2] == oldest[:2] for k in self._graphs) and oldest[:2] != gkey[:2]:
+                self._ctx.pop(oldest[:2], None)         # no recording reads these buffers any more
         self._graphs[gkey] = (graph, logits)
+
+    def _forget(self, key: Tuple[int, int]) -> None:
+        """Drop a step shape: its fixed buffers, and the recordings and counts that belong to it."""
+        self._ctx.pop(key, None)
+        for table in (self._graphs, self._uses):
+            for k in [k for k in table if k[:2] == key]:
+                del table[k]
 
     def step(self, draw=None) -> List[int]:
         """Feed the pending tokens and choose on the device, greedily or with ``draw`` (what

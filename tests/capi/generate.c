@@ -124,6 +124,31 @@ int main(int argc, char **argv) {
     for (uint32_t j = 0; j < counts[i]; ++j) printf(" %d", out[i * 6 + j]);
     printf("\n");
   }
+  /* prefix reuse: a conversation that goes on feeds only what is new, and says the same */
+  sp.temperature = 0.0f;
+  sp.top_k = 0;
+  sp.max_tokens = 4;
+  MUST(boom_llm_session_keep(session, 1, &err));
+  boom_token first[4];
+  uint32_t n_first = 0;
+  const boom_token *one[1] = {p1};
+  const size_t one_len[1] = {7};
+  MUST(boom_llm_generate(session, one, one_len, 1, &sp, no_stop, 0, NULL, NULL, first, &n_first, &err));
+  boom_token longer[7 + 3 + 2] = {4, 5, 6, 7, 8, 9, 10, 0, 0, 0, 33, 34};
+  for (int j = 0; j < 3; ++j) longer[7 + j] = first[j];
+  const boom_token *two[1] = {longer};
+  const size_t two_len[1] = {12};
+  boom_token second[4];
+  uint32_t n_second = 0;
+  MUST(boom_llm_generate(session, two, two_len, 1, &sp, no_stop, 0, NULL, NULL, second, &n_second, &err));
+  uint64_t reused[1] = {0};
+  size_t n_reused = 0;
+  if (boom_llm_session_reused(session, NULL, 0, &n_reused, &err) != BOOM_ERR_BINDING || n_reused != 1) return 9;
+  MUST(boom_llm_session_reused(session, reused, 1, &n_reused, &err));
+  printf("reused %llu:", (unsigned long long)reused[0]);
+  for (uint32_t j = 0; j < n_second; ++j) printf(" %d", second[j]);
+  printf("\n");
+  MUST(boom_llm_session_keep(session, 0, &err));
   free(logits);
   free(arch);
   boom_llm_session_free(session);

@@ -19,7 +19,7 @@ def check_invariants(c: PagedCache):
     for g, pool in enumerate(c.pools):
         held = [p for s in c.live_slots for p in c._slots[s].pages[g] if p >= 0]
         assert len(held) == len(set(held)), "a page is held twice"
-        assert len(held) + pool.free_count == c.n_pages, "a page is lost"
+        assert len(held) + pool.free_count == pool.n_pages, "a page is lost"
         assert set(held).isdisjoint(pool._free)
     assert len(c.live_slots) + len(c._free_slots) == c.max_slots
     assert set(c.live_slots).isdisjoint(c._free_slots)
@@ -184,3 +184,52 @@ def test_the_caches_order_of_elements_is_a_permutation_of_every_row():
     assert len({int(kp[j, 0]) // 8 for j in keys}) == 16
     vp = layout.value_positions(128)
     assert len({(int(vp[d, 0]) // 8, d % 2) for d in range(16)}) == 16           # sixteen rows: 8 offsets x 2 rows of 128 bytes
+
+
+def test_a_windowed_group_gets_a_pool_of_its_own_size():
+    """With bounds on the sequences and on the rows between two advances, a windowed group holds
+    at most a window and a step's rows a sequence: its pool is that big and never runs out,
+    whatever the lengths; the group that keeps every key is what refuses."""
+    from sonicboom_amd.cache.paged import pool_pages
+    assert pool_pages(100, 0, 4, 64) == 100 and pool_pages(100, 50, 4, 0) == 100
+    assert pool_pages(100, 50, 4, 64) == 4 * 3 + 1 and pool_pages(10, 50, 4, 64) == 10
+    groups = [GroupSpec(2, 16, 0, (0,)), GroupSpec(1, 32, 100, (1,))]
+    c = PagedCache(groups, 64 * 40, allocate=False, max_slots=3, step_rows=128)
+    assert [p.n_pages for p in c.pools] == [40, 3 * 4 + 2]
+    rng = random.Random(3)
+    slots = [c.alloc_slot() for _ in range(3)]
+    for _ in range(60):
+        # a step of at most 128 rows over the three sequences, in any split
+        total = rng.randint(3, 128)
+        first = rng.randint(1, total - 2)
+        second = rng.randint(1, total - first - 1)
+        n_new = [first, second, total - first - second]
+        try:
+            c.reserve(slots, n_new, c.windowed(False))
+        except CacheError:
+            break                                   # the full group is out of pages: 40 pages are held
+        c.reserve(slots, n_new, c.windowed(True))   # never refuses
+        c.advance(slots, n_new)
+        check_invariants(c)
+        assert c.held_pages(1) <= 3 * 3
+    else:
+        raise AssertionError("the cache never filled up")
+    assert c.windowed(True) == [1] and c.windowed(False) == [0]
+
+
+def test_trim_gives_back_what_was_reserved_for_rows_that_did_not_run():
+    c = make(window=70)
+    a, b = c.alloc_slot(), c.alloc_slot()
+    c.reserve([a, b], [100, 10])
+    c.advance([a, b], [100, 10])
+    before = [c.held_pages(g) for g in range(2)]
+    c.reserve([a, b], [200, 60])                    # a step that then fails: nothing advances
+    assert c.held_pages(0) == before[0] + 3 + 1
+    c.trim([a, b])
+    assert [c.held_pages(g) for g in range(2)] == before
+    assert (c.length(a), c.length(b)) == (100, 10)
+    check_invariants(c)
+    c.trim([a])                                     # nothing to give back: no harm
+    c.reserve([a], [1])
+    c.advance([a], [1])
+    check_invariants(c)

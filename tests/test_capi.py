@@ -118,7 +118,16 @@ def test_a_c_program_gets_what_the_package_gives(tmp_path, model_folders, dtype)
     want.append("short struct:" + "".join(f" {t}" for t in pen[0]))
     outs = session.generate(prompts, max_tokens=6, stop_tokens=[], temperature=0.8, seed=7, top_k=40)
     want += [f"sampled {i}:" + "".join(f" {t}" for t in o) for i, o in enumerate(outs)]
+    # the conversation that the C program continues on a kept sequence, here fed whole
+    first = session.generate([prompts[1]], max_tokens=4, stop_tokens=[])[0]
+    longer = prompts[1] + first[:3] + [33, 34]
+    whole = session.generate([longer], max_tokens=4, stop_tokens=[])[0]
+    want.append("reused 10:" + "".join(f" {t}" for t in whole))
     want.append("ok")
+    if dtype == "bfloat16":
+        # a sequence fed in other cuts rounds differently in bfloat16: the count is held, the tokens in 32-bit
+        got = [g.split(":")[0] if g.startswith("reused") else g for g in got]
+        want = [w.split(":")[0] if w.startswith("reused") else w for w in want]
     assert got == want
 
 

@@ -30,6 +30,9 @@ class TableEngine:
     def free_slot(self, s):
         self.cache.free_slot(s)
 
+    def length(self, s):
+        return self.cache.length(s)
+
     def step(self, entries):
         slots = [e.slot for e in entries]
         n_new = [len(e.tokens) for e in entries]
@@ -189,3 +192,91 @@ def test_masks_reach_the_sampler_and_a_request_that_may_choose_nothing_ends():
     # without ``allowed`` a sampler of the three-argument form is called as before
     assert generate(TableEngine(64 * 8), prompts, SamplingParams(max_tokens=2), stop_tokens=(), sampler=HostSampler()) \
         == [expected(p, 2) for p in prompts]
+
+
+# ---- sequences kept for the next call ------------------------------------------------------------
+def test_a_kept_sequence_feeds_only_what_is_new():
+    from sonicboom_amd.engine.prefix import KeptSequences, common_prefix_len
+    assert common_prefix_len([1, 2, 3], [1, 2, 4, 5]) == 2 and common_prefix_len([], [1]) == 0
+    eng = TableEngine(64 * 8)
+    kept = KeptSequences(eng)
+    first = [[3] * 24, [5, 6, 7]]
+    outs = generate(eng, first, SamplingParams(max_tokens=4), stop_tokens=(), sampler=HostSampler(), kept=kept)
+    assert outs == [expected(p, 4) for p in first] and kept.reused == [0, 0]
+    # both sequences stay, with every token that was fed (the last produced one was not)
+    assert sorted(len(t) for _, t in kept.items) == [3 + 3, 24 + 3] and len(eng.cache.live_slots) == 2
+    eng.steps.clear()
+    # the same conversation goes on: 24 tokens + 3 of the 4 produced + 13 new ones
+    longer = first[0] + outs[0][:3] + [9] * 13
+    other = [8] * 10                                          # starts like nothing that was kept
+    outs2 = generate(eng, [other, longer], SamplingParams(max_tokens=5), stop_tokens=(), sampler=HostSampler(), kept=kept)
+    assert outs2 == [expected(other, 5), expected(longer, 5)] and kept.reused == [0, 27]
+    assert sorted(n for _, n in eng.steps[0]) == [10, 13]     # only the 13 new tokens were fed
+    # the sequence no prompt continued was freed at the start; the two new ones are kept now
+    assert len(kept) == 2 and len(eng.cache.live_slots) == 2
+    # a prompt the session holds in full still feeds its last token; a shorter one cuts the sequence back
+    eng.steps.clear()
+    again = longer[:20]
+    outs3 = generate(eng, [again], SamplingParams(max_tokens=2), stop_tokens=(), sampler=HostSampler(), kept=kept)
+    assert outs3 == [expected(again, 2)] and kept.reused == [19] and eng.steps[0] == [(eng.steps[0][0][0], 1)]
+    assert len(kept) == 1 and eng.cache.held_pages() == 1
+    kept.drop_all()
+    assert not eng.cache.live_slots and eng.cache.held_pages() == 0
+
+
+def test_kept_sequences_never_cost_a_request_its_room():
+    """Pages and slots of kept sequences count while earlier batches run; when they leave an
+    earlier request no room, the call goes without them."""
+    from sonicboom_amd.engine.prefix import KeptSequences
+    assert plan_batches([128, 64, 64], 0, 3, 8) == [[0, 1], [2]]
+    assert plan_batches([128, 64, 64], 0, 3, 8, held=[0, 0, 1]) == [[0], [1, 2]]     # request 2's page is taken meanwhile
+    assert plan_batches([64, 64, 64], 0, 8, 8, max_slots=2, held=[0, 0, 1]) == [[0], [1, 2]]     # and so is its slot
+    eng = TableEngine(64 * 4, max_slots=2)
+    kept = KeptSequences(eng)
+    a, b = [1] * 100, [2] * 100
+    generate(eng, [a, b], SamplingParams(max_tokens=2), stop_tokens=(), sampler=HostSampler(), kept=kept)
+    assert len(kept) == 2 and eng.cache.held_pages() == 4
+    # a request that needs three pages of the four comes first; b's kept sequence would leave it two
+    big = [3] * 150
+    outs = generate(eng, [big, b + [7]], SamplingParams(max_tokens=2), stop_tokens=(), sampler=HostSampler(), kept=kept)
+    assert outs == [expected(big, 2), expected(b + [7], 2)] and kept.reused == [0, 0]
+    kept.drop_all()
+    assert not eng.cache.live_slots and eng.cache.held_pages() == 0
+    # an exception on the way frees what the call held
+    generate(eng, [a], SamplingParams(max_tokens=2), stop_tokens=(), sampler=HostSampler(), kept=kept)
+
+    def refuse(i, t):
+        raise RuntimeError("stop")
+    with pytest.raises(RuntimeError):
+        generate(eng, [a + [4]], SamplingParams(max_tokens=2), stop_tokens=(), sampler=HostSampler(), kept=kept,
+                 callback=refuse)
+    assert not eng.cache.live_slots and eng.cache.held_pages() == 0 and len(kept) == 0
+
+
+def test_truncate_refuses_what_cannot_be_taken_back():
+    from sonicboom_amd.cache import CacheError
+    c = PagedCache([GroupSpec(1, 16, 0, (0,)), GroupSpec(1, 16, 100, (1,))], 64 * 16, allocate=False)
+    s = c.alloc_slot()
+    c.reserve([s], [300])
+    c.advance([s], [300])
+    assert c.can_truncate(s, 300) and c.can_truncate(s, 292) and not c.can_truncate(s, 290) and not c.can_truncate(s, 301)
+    with pytest.raises(CacheError, match="windowed group"):
+        c.truncate(s, 100)
+    c.reserve([s], [30])
+    c.advance([s], [30])
+    assert c.held_pages(0) == 6
+    c.truncate(s, 292)                         # back over a page's edge: the sixth page goes
+    assert c.length(s) == 292 and c.held_pages(0) == 5 and c.held_pages(1) == 2
+    c.reserve([s], [60])
+    c.advance([s], [60])
+    assert c.length(s) == 352
+    # a cache whose mixers keep per-sequence state only goes back to where it is
+    state = PagedCache([GroupSpec(1, 16, 0, (0,))], 64 * 4, allocate=False)
+    import torch
+    state.state[0] = torch.zeros((state.max_slots, 3))
+    t = state.alloc_slot()
+    state.reserve([t], [10])
+    state.advance([t], [10])
+    assert state.can_truncate(t, 10) and not state.can_truncate(t, 9)
+    with pytest.raises(CacheError, match="state"):
+        state.truncate(t, 5)

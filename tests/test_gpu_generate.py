@@ -363,3 +363,56 @@ def test_command_line(model_folders, tmp_path):
     bad = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "sb-gen"), "--tokens", str(tokens)],
                          capture_output=True, text=True, timeout=60)
     assert bad.returncode == 2 and "usage" in bad.stderr
+
+
+def test_prefix_reuse_gives_the_bits_of_the_whole_prompt(model_folders):
+    """A conversation that goes on: 24 tokens, 16 more on the kept sequence, against the 40 fed
+    whole (/root/reference/tests/core/test_guarantees.cpp:300-326): in 32-bit the same logits to
+    the bit and the same tokens, greedy and drawn; only the new tokens are fed."""
+    import torch
+    from sonicboom_amd.api import Model
+    from sonicboom_amd.engine import StepEntry
+    model = Model.load(model_folders["B"], dtype="float32")
+    rng = np.random.default_rng(21)
+    head, more = random_prompt(rng, 384, 24), random_prompt(rng, 384, 16)
+    other = random_prompt(rng, 384, 30)
+    for sampling in (dict(), dict(temperature=0.9, seed=5, top_p=0.95)):
+        whole = model.session(64 * 8)
+        want = whole.generate([head + more, other], max_tokens=12, stop_tokens=[], **sampling)
+        ses = model.session(64 * 8)
+        fed = []
+        step = ses.engine.step
+        ses.engine.step = lambda entries: (fed.append([len(e.tokens) for e in entries]), step(entries))[1]
+        first = ses.generate([head], max_tokens=3, stop_tokens=[], keep=True, **sampling)[0]
+        assert ses.reused == [0] and len(ses.kept) == 1
+        fed.clear()
+        got = ses.generate([other, head + more], max_tokens=12, stop_tokens=[], keep=True, **sampling)
+        # the kept sequence holds the 24 tokens and two of the three produced; the new prompt shares the 24
+        assert ses.reused == [0, 24] and fed[0] == [30, 16]
+        assert got == [want[1], want[0]]
+        assert len(ses.kept) == 2
+        ses.forget()
+        assert not ses.engine.cache.live_slots and ses.engine.cache.held_pages() == 0
+    # the logits themselves: 24 + 16 on the same slot against 40 at once
+    eng = model.session(64 * 4).engine
+    a, b = eng.alloc_slot(), eng.alloc_slot()
+    eng.step([StepEntry(a, head + random_prompt(rng, 384, 9), ())])        # a sequence that went elsewhere
+    eng.cache.truncate(a, 24)                                              # back to the shared prefix
+    cut = eng.step([StepEntry(a, more, range(16))])
+    full = eng.step([StepEntry(b, head + more, range(24, 40))])
+    assert torch.equal(cut, full)
+
+
+def test_prefix_reuse_in_bfloat16_stays_within_the_bounds(model_folders):
+    from helpers import assert_logits_close, plain_logits
+    from sonicboom_amd.api import Model
+    from sonicboom_amd.engine import StepEntry
+    folder = model_folders["A"]
+    eng = Model.load(folder, dtype="bfloat16").session(64 * 8).engine
+    rng = np.random.default_rng(3)
+    head, more = random_prompt(rng, 256, 70), random_prompt(rng, 256, 30)
+    s = eng.alloc_slot()
+    eng.step([StepEntry(s, head + random_prompt(rng, 256, 20), ())])
+    eng.cache.truncate(s, 70)
+    got = eng.step([StepEntry(s, more, range(30))]).cpu().numpy()
+    assert_logits_close(got, plain_logits(folder, head + more)[70:], "bfloat16", "on a sequence taken back")

@@ -266,6 +266,18 @@ def register_toys():
                 expert.forward(h[rows].contiguous(), out, ctx)
                 x[rows] += out * share[rows, slot][:, None]
 
+    @register_part("embedding", "toy_learned_positions")
+    class PositionedEmbedding(Part):
+        """x_t = E[token_t] + P[position_t]: an embedding that reads the step's context."""
+        category = "embedding"
+
+        def __init__(self, spec, tensors, parts, rt):
+            super().__init__(spec, tensors, parts, rt)
+            self.table, self.places = tensors["table"], tensors["places"].float()
+
+        def forward(self, ids, ctx):
+            return ops.embed(self.table, ids) + self.places[ctx.row_pos.long()]
+
     return ops, register_architecture
 
 
@@ -320,7 +332,11 @@ def toy_spec(cfg):
                                          rmsnorm_spec(p + "n2", w, d["eps"]), ffn))
     for e in d["order"]:
         order.append(OrderEntry(e["block"], e.get("cache"), e.get("writes", True)))
-    return ModelSpec("ToyForCausalLM", w, v, embedding_spec("emb", v, w), blocks, order,
+    embedding = embedding_spec("emb", v, w)
+    if d.get("learned_positions"):
+        embedding = PartSpec("embedding", "toy_learned_positions", {"vocab": v, "width": w}, {
+            "table": TensorSpec("emb", (v, w)), "places": TensorSpec("places", (d["learned_positions"], w))})
+    return ModelSpec("ToyForCausalLM", w, v, embedding, blocks, order,
                      rmsnorm_spec("norm", w, d["eps"]), head_spec("head", v, w))
 
 
@@ -332,6 +348,8 @@ def plain_toy(cfg, w, tokens, margins=None):
     n = len(tokens)
     pos = np.arange(n)
     x = P.embedding(w["emb"], tokens)
+    if d.get("learned_positions"):
+        x = (x + w["places"][pos]).astype(np.float32)
     kv = {}
     for e in d["order"]:
         i = e["block"]
@@ -434,7 +452,17 @@ TOY_ROUTED = {
 }
 
 
-def build_toy(cfg_dict, dtype):
+TOY_PLACES = {
+    "architectures": ["ToyForCausalLM"], "vocab_size": 140, "width": 48, "eps": 1e-5, "learned_positions": 200,
+    # no rotation anywhere: the shift "encoding" with slope 0 leaves queries and keys as they are,
+    # so the order of the tokens reaches the model through the embedding alone
+    "layers": [{"mixer": "attention", "heads": 3, "kv_heads": 3, "head_dim": 16, "ff": 64, "position": "shift",
+                "slope": 0.0}],
+    "order": [{"block": 0, "cache": 0}],
+}
+
+
+def build_toy(cfg_dict, dtype, **engine_options):
     from sonicboom_amd.config import architecture_of
     from sonicboom_amd.engine import DecoderModel, Engine
     _, register_architecture = register_toys()
@@ -444,7 +472,7 @@ def build_toy(cfg_dict, dtype):
     spec = arch.build_spec(cfg)
     dev, ref = tensors_for(spec, dtype, seed=3, scale=0.1)
     model = DecoderModel(spec, dev, runtime(dtype), cfg)
-    return cfg, ref, model, Engine(model, max_tokens=64 * 12)
+    return cfg, ref, model, Engine(model, max_tokens=64 * 12, **engine_options)
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
@@ -570,3 +598,56 @@ def test_toy_feed_forward_with_routing(dtype):
     eng.free_slot(sa)
     eng.free_slot(sb)
     assert eng.cache.held_pages() == 0
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_toy_embedding_that_adds_a_row_per_position(dtype):
+    """Learned absolute positions: an embedding part defined above in this file that adds a row
+    of a table by each row's position, which it reads from the step's context.  Whole, cut, two
+    sequences at once, and through the generation loop (where the step's context is the decode
+    loop's fixed buffers)."""
+    from sonicboom_amd.engine import StepEntry, generate
+    from sonicboom_amd.sampling import SamplingParams
+    cfg, ref, model, eng = build_toy(TOY_PLACES, dtype)
+    rng = np.random.default_rng(8)
+    a, b = ([int(t) for t in rng.integers(0, 140, size=n)] for n in (90, 33))
+    want_a, want_b = plain_toy(cfg, ref, a), plain_toy(cfg, ref, b)
+    moved = plain_toy(cfg, dict(ref, places=np.roll(ref["places"], 1, axis=0)), a)
+    assert np.abs(moved - want_a).max() > 0.05            # the positions' rows do matter
+    sa, sb = eng.alloc_slot(), eng.alloc_slot()
+    out = eng.step([StepEntry(sa, a[:60], range(60)), StepEntry(sb, b[:10], range(10))])
+    close(out[:60], want_a[:60], dtype, "places, a's prompt")
+    close(out[60:], want_b[:10], dtype, "places, b's prompt")
+    for i in range(23):
+        out = eng.step([StepEntry(sa, [a[60 + i]], [0]), StepEntry(sb, [b[10 + i]], [0])])
+        close(out[:1], want_a[60 + i:61 + i], dtype, f"places, a token {i}")
+        close(out[1:], want_b[10 + i:11 + i], dtype, f"places, b token {i}")
+    eng.free_slot(sa)
+    eng.free_slot(sb)
+    toks = generate(eng, [a[:7], b[:12]], SamplingParams(max_tokens=8), stop_tokens=())
+    if dtype == F32:
+        for prompt, out_t in zip((a[:7], b[:12]), toks):
+            logits = plain_toy(cfg, ref, prompt + out_t)
+            assert out_t == [int(np.argmax(logits[len(prompt) - 1 + i])) for i in range(8)]
+
+
+def test_windowed_groups_get_pools_of_their_own_size():
+    """With a bound on the sequences and on a step's rows, a windowed group's pool holds a window
+    and a step's rows a sequence instead of the whole cache, and a prompt longer than that pool
+    runs through it portion by portion."""
+    from sonicboom_amd.engine import StepEntry
+    cfg, ref, model, eng = build_toy(TOY_WINDOWS, F32, max_slots=2, max_step_rows=64)
+    pools = {g.window: eng.cache.pools[i].n_pages for i, g in enumerate(eng.cache.groups)}
+    assert pools == {0: 12, 50: 2 * 3 + 1, 70: 2 * 4 + 1}
+    assert eng.cache.k[[g.window for g in eng.cache.groups].index(50)].shape[1] == 7
+    rng = np.random.default_rng(2)
+    a, b = ([int(t) for t in rng.integers(0, 150, size=n)] for n in (400, 300))      # 7 + 5 pages of all keys
+    sa, sb = eng.alloc_slot(), eng.alloc_slot()
+    out = eng.step([StepEntry(sa, a, range(len(a))), StepEntry(sb, b, range(len(b)))])      # eleven portions
+    close(out[:400], plain_toy(cfg, ref, a), F32, "a through small pools")
+    close(out[400:], plain_toy(cfg, ref, b), F32, "b through small pools")
+    held = {g.window: eng.cache.held_pages(i) for i, g in enumerate(eng.cache.groups)}
+    assert held[0] == 12 and held[50] <= 4 and held[70] <= 6
+    eng.free_slot(sa)
+    eng.free_slot(sb)
+    assert all(eng.cache.held_pages(i) == 0 for i in range(3))
