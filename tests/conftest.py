@@ -20,6 +20,15 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a HIP GPU (MI355X)")
 
 
+def pytest_terminal_summary(terminalreporter):
+    """What the bfloat16 comparisons measured, beside their bounds."""
+    import helpers
+    for kind, (worst, rms) in sorted(helpers.BF16_SEEN.items()):
+        terminalreporter.write_line(
+            f"[bfloat16 against the plain implementation, {kind}] largest difference {worst:.4f} of the logits' spread "
+            f"(bound {helpers.BF16_MAX[kind]}), root mean square {rms:.4f} (bound {helpers.BF16_RMS[kind]})")
+
+
 # Tiny A and B differ in every size and option: layers, width, heads and groups
 # (GQA 2:1 / MQA 3:1), head size, inner width, vocabulary (no powers of two in
 # B), rope base, eps, maximum positions, tied or separate head.  C adds what

@@ -50,13 +50,18 @@ def forget_plain(folder):
 # rounding of queries and keys: measured on the GPU the largest difference was 0.23 spreads and
 # the root mean square 0.022, against 0.018 and 0.004 on the tiny models of plain random weights.
 # "wide" is for models of real layer sizes, where a row of 3,584 and a sum over 18,944 products
-# round more often: measured 0.058 and 0.0095 there, where the smallest of the mistakes that
+# round more often: measured 0.066 and 0.013 there (the largest over two layers of the 7B, 14B and
+# 72B sizes; the 7B sizes alone 0.058 and 0.0095), where the smallest of the mistakes that
 # tests/test_plain.py::test_sharp_models_show_attention_mistakes plants, a dropped query bias,
-# moves the plain logits by 0.20 and 0.031 (a wrong scale by 4.6 and 0.88).
+# moves the plain logits by 0.20 and 0.031 (a wrong scale by 4.6 and 0.88): the bounds are what
+# was measured times 1.4, and that mistake is 2.2 and 1.7 times beyond them.
 F32_TOL = dict(atol=5e-5, rtol=5e-5)
-BF16_MAX = {"tiny": 0.04, "wide": 0.16, "sharp": 0.5}     # largest difference, in spreads (plus BF16_REL * |logit|)
-BF16_RMS = {"tiny": 0.01, "wide": 0.02, "sharp": 0.05}    # root mean square of the differences, in spreads
+BF16_MAX = {"tiny": 0.04, "wide": 0.09, "sharp": 0.5}     # largest difference, in spreads (plus BF16_REL * |logit|)
+BF16_RMS = {"tiny": 0.01, "wide": 0.018, "sharp": 0.05}   # root mean square of the differences, in spreads
 BF16_REL = 0.02
+# the largest of both that the bfloat16 comparisons of this run have seen, by kind (the summary
+# at the end of a test run prints them: what the bounds above are set from)
+BF16_SEEN = {}
 
 
 def bf16_limits(want, sharp=False):
@@ -78,6 +83,12 @@ def assert_logits_close(got, want, dtype, what="", sharp=False):
     else:
         bound, rms_bound = bf16_limits(want, sharp)
         rms = float(np.sqrt((err ** 2).mean())) if err.size else 0.0
+        spread = float(want.std())
+        if err.size and spread > 0:
+            kind = {False: "tiny", True: "sharp"}.get(sharp, sharp)
+            seen = BF16_SEEN.setdefault(kind, [0.0, 0.0])
+            seen[0] = max(seen[0], float((err - BF16_REL * np.abs(want)).max()) / spread)
+            seen[1] = max(seen[1], rms / spread)
         assert rms <= rms_bound, f"{what}: root mean square difference {rms:.3g} > {rms_bound:.3g}"
     if not (err <= bound).all():
         i = np.unravel_index(np.argmax(err - bound), err.shape)

@@ -156,6 +156,34 @@ def attention(q: np.ndarray, k: np.ndarray, v: np.ndarray, q_positions,
     return out.reshape(nq, n_heads_q * head_dim)
 
 
+def attention_causal_blocked(q: np.ndarray, k: np.ndarray, v: np.ndarray, n_heads_q: int, n_heads_kv: int,
+                             head_dim: int, scale: float, rows_at_once: int = 256) -> np.ndarray:
+    """:func:`attention` for the one case that long sequences need (row i at position i over keys
+    0..i, no window), a block of rows at a time with matrix products instead of a loop over rows:
+    the same formula and the same precisions (float64 sums rounded once, float32 scores, maximum,
+    exponentials and weights), thousands of times faster.  tests/test_plain.py holds it to
+    :func:`attention`."""
+    group = n_heads_q // n_heads_kv
+    n = q.shape[0]
+    qv = np.asarray(q, dtype=F32).reshape(n, n_heads_q, head_dim)
+    kv = np.asarray(k, dtype=F32).reshape(n, n_heads_kv, head_dim).astype(F64)
+    vv = np.asarray(v, dtype=F32).reshape(n, n_heads_kv, head_dim).astype(F64)
+    out = np.zeros((n, n_heads_q, head_dim), dtype=F32)
+    for r0 in range(0, n, rows_at_once):
+        r1 = min(n, r0 + rows_at_once)
+        hidden = np.arange(r1)[None, :] > np.arange(r0, r1)[:, None]
+        for h in range(n_heads_q):
+            kh = h // group
+            s = (qv[r0:r1, h, :].astype(F64) @ kv[:r1, kh, :].T).astype(F32)
+            s = (s * F32(scale)).astype(F32)
+            s[hidden] = -np.inf
+            e = np.exp((s - s.max(axis=1, keepdims=True)).astype(F32)).astype(F32)
+            inv = F32(1.0) / e.sum(axis=1, keepdims=True, dtype=F32)
+            p = (e * inv).astype(F32)
+            out[r0:r1, h, :] = (p.astype(F64) @ vv[:r1, kh, :]).astype(F32)
+    return out.reshape(n, n_heads_q * head_dim)
+
+
 def silu(x: np.ndarray) -> np.ndarray:
     """core/src/nn/activation.cpp:41-50: x / (1 + exp(-x)) in float32."""
     x = np.asarray(x, dtype=F32)
@@ -231,8 +259,12 @@ def self_attention(h: np.ndarray, positions, w: dict, prefix: str, cfg: dict) ->
     k = rope_neox(k, positions, hd, cfg["rope_theta"], freq_factors=ff)
     # core/src/model/recipe.cpp:165-167: the architecture's 1/sqrt(head_dim) times YaRN's magnitude term
     scale = F32(F32(1.0) / np.sqrt(F32(hd))) * F32(score_mult)
-    a = attention(q, k, v, positions, positions, hq, hkv, hd, float(scale),
-                  causal=True, window=0)
+    pos = np.asarray(positions)
+    if len(pos) > 4096 and np.array_equal(pos, np.arange(len(pos))):
+        a = attention_causal_blocked(q, k, v, hq, hkv, hd, float(scale))     # the same, in blocks of rows
+    else:
+        a = attention(q, k, v, positions, positions, hq, hkv, hd, float(scale),
+                      causal=True, window=0)
     return linear(a, w[prefix + "o_proj.weight"])
 
 

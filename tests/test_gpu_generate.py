@@ -10,7 +10,7 @@ import numpy as np
 import pytest
 
 from conftest import ROOT, TINY, random_prompt
-from helpers import assert_logits_close, plain_logits, plain_model
+from helpers import BF16_MAX, BF16_REL, assert_logits_close, plain_logits, plain_model
 from plain import qwen2_plain, sampling_plain
 
 pytestmark = pytest.mark.gpu
@@ -55,7 +55,9 @@ def test_greedy_bfloat16_follows_the_plain_logits(model_folders):
             logits = plain_logits(folder, p + out)
             for i, t in enumerate(out):
                 row = logits[len(p) - 1 + i]
-                assert row[t] >= row.max() - 0.05 * max(1.0, np.abs(row).max()), (name, i)
+                # the chosen token's plain logit trails the best by no more than bfloat16 moves two logits
+                slack = 2 * (BF16_MAX["tiny"] * float(row.std()) + BF16_REL * float(np.abs(row).max()))
+                assert row[t] >= row.max() - slack, (name, i, float(row.max() - row[t]), slack)
 
 
 def test_temperature_sampling_tiny_b(model_folders):

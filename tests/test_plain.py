@@ -389,3 +389,17 @@ def test_greedy_stops_after_the_stop_token(models):
     stopped = P.greedy(cfg, w, [5, 6, 7], 6, stop=(free[2],))
     assert stopped == free[:free.index(free[2]) + 1]
     assert P.argmax(np.array([0.5, 0.5, 0.1])) == 0             # ties to the lowest id
+
+
+def test_attention_in_blocks_of_rows_is_the_plain_attention():
+    """The form that long sequences use: the same numbers as the loop over rows (the row sums of
+    the exponentials may round differently by an ulp: numpy sums a row of a matrix pairwise as it
+    sums a vector, so they do not)."""
+    rng = np.random.default_rng(12)
+    for n, hq, hkv, hd in ((70, 4, 2, 16), (300, 3, 1, 32), (129, 2, 2, 8)):
+        q, k, v = (rng.standard_normal((n, h * hd)).astype(np.float32) * 1.5 for h in (hq, hkv, hkv))
+        pos = np.arange(n)
+        want = P.attention(q, k, v, pos, pos, hq, hkv, hd, 0.3)
+        for rows in (1, 64, 1000):
+            got = P.attention_causal_blocked(q, k, v, hq, hkv, hd, 0.3, rows_at_once=rows)
+            assert np.allclose(got, want, rtol=0, atol=2e-6), np.abs(got - want).max()
