@@ -662,6 +662,281 @@ attn_prefill_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
 }
 
 // ---------------------------------------------------------------------------------------------
+// Prefill in tiles of 32 rows, for long prompts: a block takes up to 32 consecutive rows of one
+// sequence and one kv head, wave w of its eight the query head w of that kv head's group (waves
+// past the group bring the pages in), and the products are v_mfma_f32_32x32x16_bf16:
+//   S^T[32 keys][32 rows] = K[32 keys][16 d] . Q^T[16 d][32 rows]      A = K rows out of LDS, B = Q rows in registers
+//   O^T[32 d][32 rows]   += V^T[32 d][16 keys] . P[16 keys][32 rows]   A = V^T rows out of LDS, B = P in registers
+// A page that lies in LDS serves twice the rows it serves in the 16-row kernel above, and every
+// fragment read from LDS feeds twice the products: per product half the LDS traffic, half the
+// copies into LDS and half the barriers.
+//
+// Lane l of such a product holds for A row l % 32, k = 8 (l / 32) .. + 7, for B column l % 32 and
+// the same k, and of the result column l % 32, rows 8 q + 4 (l / 32) + e for q, e = 0 .. 3
+// (register 4 q + e).  Which key a row of the score product stands for is this kernel's choice.
+// Row 8 q + 4 c + e of the tile of keys 32 t .. 32 t + 31 is key
+//   32 t + 16 c + 8 (q & 1) + 4 (q >> 1) + e:
+// the half of the wave c = l / 32 then holds, in registers 4 q .. 4 q + 3, the keys of the chunks
+// of eight 4 t + 2 c and 4 t + 2 c + 1 (lower halves in q = 0 and 1, upper halves in q = 2 and 3),
+// and a step of sixteen keys of the second product takes chunk 4 t + j from half 0 and 4 t + 2 + j
+// from half 1 (j = 0, 1): the eight k of a lane are one chunk of the value row, as the cache keeps
+// it, and P never leaves the registers.  The sixteen lanes that LDS serves together read key rows
+// that differ in bits 0, 1, 3 and 4, which the cache's order of a row's chunks (sb_key_swizzle)
+// spreads over all banks.
+constexpr int DS32 = HD / 16;        // k-steps (16 d) of the score product
+constexpr int DT32 = HD >= 32 ? HD / 32 : 1;        // 32-row tiles of O^T
+constexpr bool kTallOk = HD % 32 == 0 && HD <= 128;
+
+struct TallState {
+  floatx16_t o[DT32];
+  float m, l;               // running maximum of the lane's column (log2 domain), the lane's share of the sum
+};
+
+// The maximum of a value over the two halves of the wave (lanes l and l ^ 32), in both.
+__device__ __forceinline__ float max_over_halves(float v) {
+  const uint32_t u = __builtin_bit_cast(uint32_t, v);
+  const auto p = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const uint32_t p0 = p[0], p1 = p[1];
+  return fmaxf(__builtin_bit_cast(float, p0), __builtin_bit_cast(float, p1));
+}
+
+// Key (within its page) of register i = 4 q + e of score tile t in half c of the wave.
+__device__ __forceinline__ constexpr int tall_key(int t, int i, int c) {
+  return 32 * t + 16 * c + 8 * ((i >> 2) & 1) + 4 * (i >> 3) + (i & 3);
+}
+
+// One page out of LDS.  masked (uniform over the block): some key of the page is hidden from some
+// row, so every score is tested; the values of keys that no row of the tile may see have been
+// zeroed in LDS by then (they may be stale or never written, and 0 * garbage must not reach the sums).
+__device__ __forceinline__ void attend_page_tall(TallState &st, const bf16x8_t (&qf)[DS32], const uint4 *kl,
+                                                 const uint4 *vl, int page_pos, bool masked, int col_pos, int col_lo,
+                                                 float scale_log2, int lane) {
+  const int m = lane & 31, c = lane >> 5;
+  // this lane's key row of a tile: row m = 8 q + 4 cc + e of the product
+  const int q_ = m >> 3, cc = (m >> 2) & 1;
+  const int krow = 16 * cc + 8 * (q_ & 1) + 4 * (q_ >> 1) + (m & 3);
+  const int kswz = sb_key_swizzle(krow, HD);             // bits 0, 1, 3, 4 of the key: the same for krow + 32
+  floatx16_t s[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    floatx16_t acc;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+#pragma unroll
+    for (int ds = 0; ds < DS32; ++ds)
+      acc = mfma32(as_bf16x8(kl[(32 * t + krow) * CPRK + ((2 * ds + c) ^ kswz)]), qf[ds], acc);
+    s[t] = acc;
+  }
+  // the first tile's fragments are asked for at once, the second tile's while the first is multiplied
+  __builtin_amdgcn_sched_group_barrier(0x100, DS32, 0);
+#pragma unroll
+  for (int ds = 0; ds < DS32; ++ds) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+  }
+  __builtin_amdgcn_sched_group_barrier(0x008, DS32, 0);
+  __builtin_amdgcn_sched_barrier(0);          // (the value fragments are not asked for before the scores are done)
+  if (masked) {
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int j = page_pos + tall_key(t, i, c);
+        s[t][i] = (j <= col_pos && j >= col_lo) ? s[t][i] : -__builtin_inff();
+      }
+  }
+  float mx = -__builtin_inff();
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[t][i]);
+  mx = max_over_halves(mx) * scale_log2;                 // the scale is positive
+  // The running maximum only moves when a score exceeds it by more than kMaxSlack (see attend_page64).
+  const float m_old = st.m;
+  const bool move = mx > m_old + kMaxSlack;              // also the first key of a column
+  const float m_new = move ? mx : m_old;
+  const float m_use = m_new == -__builtin_inff() ? 0.f : m_new;
+  const float alpha = move ? __builtin_amdgcn_exp2f(m_old - m_use) : 1.f;      // m_old = -inf gives 0
+  float psum = 0.f;
+  uint4 pb[2][2];                                        // [tile][j]: the chunk 4 t + 2 c + j of the page
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    float p[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      p[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][i], scale_log2, -m_use));    // -inf gives 0
+      psum += p[i];
+    }
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+      pb[t][j] = make_uint4(pack_bf16(p[4 * j + 0], p[4 * j + 1]), pack_bf16(p[4 * j + 2], p[4 * j + 3]),
+                            pack_bf16(p[8 + 4 * j + 0], p[8 + 4 * j + 1]), pack_bf16(p[8 + 4 * j + 2], p[8 + 4 * j + 3]));
+  }
+  st.l = st.l * alpha + psum;
+  st.m = m_new;
+  if (__any(move)) {
+#pragma unroll
+    for (int dt = 0; dt < DT32; ++dt)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) st.o[dt][i] *= alpha;
+  }
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int dt = 0; dt < DT32; ++dt) {
+    const int d = 32 * dt + m;
+    floatx16_t acc = st.o[dt];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        acc = mfma32(as_bf16x8(vl[v_slot(d, 4 * t + 2 * c + j)]), as_bf16x8(pb[t][j]), acc);
+    st.o[dt] = acc;
+  }
+  // four fragments ahead of the products
+  __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+  for (int i = 0; i < 4 * DT32 - 4; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+  }
+  __builtin_amdgcn_sched_group_barrier(0x008, 4, 0);
+  __builtin_amdgcn_sched_barrier(0);
+}
+
+// tiles: int32 [n_tiles][4] = (first row, rows <= 32, sequence, unused).  Grid as above: the block
+// number counts (kv head, group of eight heads) fastest and row tiles from the last one down.
+template <bool OK>      // kTallOk: head sizes that this form does not take compile to nothing
+__global__ void __launch_bounds__(512, 2)
+attn_prefill_tall_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q, const bf16_t *__restrict__ k_cache,
+                         const bf16_t *__restrict__ v_cache, const int32_t *__restrict__ page_table, int max_pages,
+                         int n_pages_total, const int32_t *__restrict__ row_pos, const int32_t *__restrict__ tiles,
+                         int n_tiles, int heads_q, int heads_kv, int y_per_kv, float scale_log2, int window) {
+  if constexpr (OK) {
+  constexpr int WAVES = 8;
+  extern __shared__ uint4 lds_pages[];               // [2 buffers][keys | values][kPageChunks]
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n_y = heads_kv * y_per_kv;
+  const int tile = n_tiles - 1 - int(blockIdx.x) / n_y, by = int(blockIdx.x) % n_y;
+  const int group = heads_q / heads_kv;
+  const int kvh = by / y_per_kv, yb = by - kvh * y_per_kv;
+  const int hg = yb * WAVES + wave;                  // this wave's query head within the group
+  const int n_busy = min(group - yb * WAVES, WAVES), n_stagers = WAVES - n_busy;
+  const bool active = wave < n_busy;
+  const int head = kvh * group + (active ? hg : 0);
+  const int tile_row0 = tiles[tile * 4 + 0], n_rows = tiles[tile * 4 + 1], seq = tiles[tile * 4 + 2];
+  const int n = lane & 31, c = lane >> 5;
+  const bool col_ok = n < n_rows;
+  const int row = tile_row0 + (col_ok ? n : 0);
+  const int pos = row_pos[row];
+  const int col_pos = col_ok ? pos : -1;
+  const int col_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
+  // rows of a tile are consecutive positions: the first row has the lowest window start, the
+  // last one the highest position
+  const int pos_first = row_pos[tile_row0], pos_last = row_pos[tile_row0 + n_rows - 1];
+  const int key_lo = (window > 0 && pos_first >= window) ? pos_first - window + 1 : 0;
+  const int key_hi = pos_last;
+  const int lo_last = (window > 0 && pos_last >= window) ? pos_last - window + 1 : 0;
+
+  bf16x8_t qf[DS32];
+  {
+    const bf16_t *qrow = q + (size_t(row) * heads_q + head) * HD;
+#pragma unroll
+    for (int ds = 0; ds < DS32; ++ds) qf[ds] = as_bf16x8(ld16(qrow + 16 * ds + 8 * c, col_ok && active));
+  }
+  TallState st;
+#pragma unroll
+  for (int dt = 0; dt < DT32; ++dt)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) st.o[dt][i] = 0.f;
+  st.m = -__builtin_inff();
+  st.l = 0.f;
+
+  const int32_t *pt = page_table + size_t(seq) * max_pages;
+  const int pg_hi = min(pos_last / SB_PAGE, max_pages - 1);
+  auto next_valid = [&](int pg) {
+    while (pg <= pg_hi) {
+      const int page = pt[pg];
+      if (page >= 0 && page < n_pages_total) break;
+      ++pg;
+    }
+    return pg;
+  };
+  // Pages come straight into LDS (a load of 64 lanes x 16 bytes lands in 1 KB of consecutive LDS,
+  // and a page lies in the cache as LDS wants it): by the waves without a head when the group
+  // leaves some, else by all waves in turns.  While page p is multiplied out of one buffer, page
+  // p + 1 arrives in the other.
+  typedef __attribute__((address_space(3))) uint4 *lds_ptr_t;
+  constexpr int kWaveLoads = kPageChunks / 64;       // per page of keys, and of values
+  auto bring = [&](int pg_in, int buf_in) __attribute__((always_inline)) {
+    if (n_stagers > 0 && wave < n_busy) return;
+    const int first_load = n_stagers > 0 ? wave - n_busy : wave, step_load = n_stagers > 0 ? n_stagers : WAVES;
+    const size_t off = (size_t(pt[pg_in]) * heads_kv + kvh) * SB_PAGE * HD;
+    const __amdgpu_buffer_rsrc_t rsrc_k = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t *>(k_cache + off), 0, uint32_t(kPageChunks * 16), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rsrc_v = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t *>(v_cache + off), 0, uint32_t(kPageChunks * 16), 0x00020000);
+    for (int i = first_load; i < kWaveLoads; i += step_load) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_k, (lds_ptr_t)(lds_pages) + buf_in * 2 * kPageChunks + i * 64, 16,
+                                               lane * 16, i * 1024, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(
+          rsrc_v, (lds_ptr_t)(lds_pages) + buf_in * 2 * kPageChunks + kPageChunks + i * 64, 16, lane * 16, i * 1024, 0, 0);
+    }
+  };
+  auto landed = [&]() __attribute__((always_inline)) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+  };
+  int pg = next_valid(key_lo / SB_PAGE);
+  if (pg <= pg_hi) bring(pg, 0);
+  landed();
+  int buf = 0;
+  while (pg <= pg_hi) {
+    const int pg_next = next_valid(pg + 1);
+    if (pg_next <= pg_hi) bring(pg_next, buf ^ 1);
+    {
+      uint4 *kl = lds_pages + buf * 2 * kPageChunks, *vl = kl + kPageChunks;
+      const int page_pos = pg * SB_PAGE;
+      const bool masked = !(page_pos + SB_PAGE - 1 <= pos_first && page_pos >= lo_last);
+      if (masked) {
+        // (rare: the pages on the diagonal and at a window's edge)  The values of keys outside
+        // [key_lo, key_hi] go to zero in LDS, all threads of the block taking a share.
+        for (int idx = tid; idx < kPageChunks; idx += 64 * WAVES) {
+          const int d = idx >> 3, chunk = (idx & 7) ^ ((d >> 1) & 7);
+          const int k0 = page_pos + 8 * chunk;
+          vl[idx] = drop_first(keep_first(vl[idx], key_hi - k0 + 1), key_lo - k0);
+        }
+        __syncthreads();
+      }
+      if (active) attend_page_tall(st, qf, kl, vl, page_pos, masked, col_pos, col_lo, scale_log2, lane);
+    }
+    landed();
+    pg = pg_next;
+    buf ^= 1;
+  }
+  float l = st.l;
+  {
+    const uint32_t u = __builtin_bit_cast(uint32_t, l);
+    const auto p = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const uint32_t p0 = p[0], p1 = p[1];
+    l = __builtin_bit_cast(float, p0) + __builtin_bit_cast(float, p1);
+  }
+  if (!col_ok || !active) return;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  bf16_t *orow = out + (size_t(row) * heads_q + head) * HD;
+#pragma unroll
+  for (int dt = 0; dt < DT32; ++dt)
+#pragma unroll
+    for (int qq = 0; qq < 4; ++qq) {
+      const uint2 v = make_uint2(pack_bf16(st.o[dt][4 * qq + 0] * inv, st.o[dt][4 * qq + 1] * inv),
+                                 pack_bf16(st.o[dt][4 * qq + 2] * inv, st.o[dt][4 * qq + 3] * inv));
+      *reinterpret_cast<uint2 *>(orow + 32 * dt + 8 * qq + 4 * c) = v;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 // Decode: one row per sequence.  Block (chunk, kv head x head tile, sequence); wave w of the
 // block takes page 4 * chunk + w; columns are the query heads of the kv head.
 //
@@ -1485,6 +1760,12 @@ extern "C" int sb_attn_decode_rope_bf16(void *out, const float *qkv, int row_str
                        pages_per_wave, stream);
 }
 
+// 1 when the prefill kernel also takes tiles of 32 rows for these heads (head sizes that 32 divides,
+// up to 128; groups of three and more query heads per kv head): the form for long prompts.
+extern "C" int sb_attn_prefill_tall_ok(int heads_q, int heads_kv) {
+  return kTallOk && heads_kv > 0 && heads_q % heads_kv == 0 && heads_q / heads_kv >= 3;
+}
+
 // The tile height that suits these heads: 16 rows, or 64 and 32 for groups of one and two query
 // heads per kv head, whose blocks would otherwise have waves without a head.
 extern "C" int sb_attn_prefill_tile_rows(int heads_q, int heads_kv) {
@@ -1518,6 +1799,23 @@ extern "C" int sb_attn_prefill_bf16(void *out, const void *q, const void *k_cach
   if (nc > nc_max) nc = nc_max;
   const int head_tiles = (group + nc - 1) / nc;
   const int y_per_kv = (head_tiles + waves - 1) / waves;
+  if (tile_rows == 32 && sb_attn_prefill_tall_ok(heads_q, heads_kv)) {
+    const int y_tall = (group + 7) / 8;
+    SB_SUPPORT((long long)n_tiles * heads_kv * y_tall <= 0x7fffffffLL, "sb_attn_prefill_bf16: too many blocks");
+    constexpr int lds_tall = 2 * 2 * kPageChunks * 16;
+    static bool raised_tall = false;
+    if (lds_tall > 48 * 1024 && !raised_tall) {
+      const hipError_t e = hipFuncSetAttribute((const void *)attn_prefill_tall_kernel<kTallOk>,
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, lds_tall);
+      SB_REQUIRE(e == hipSuccess, "sb_attn_prefill_bf16: cannot reserve %d bytes of LDS: %s", lds_tall,
+                 hipGetErrorString(e));
+      raised_tall = true;
+    }
+    attn_prefill_tall_kernel<kTallOk><<<dim3(unsigned(n_tiles) * unsigned(heads_kv * y_tall)), 512, lds_tall, s>>>(
+        (bf16_t *)out, (const bf16_t *)q, (const bf16_t *)k_cache, (const bf16_t *)v_cache, page_table, max_pages,
+        n_pages_total, row_pos, tiles, n_tiles, heads_q, heads_kv, y_tall, scale * kLog2e, window);
+    return sb::check_launch("sb_attn_prefill_bf16");
+  }
   SB_REQUIRE(tile_rows == 16 || tile_rows == sb_attn_prefill_tile_rows(heads_q, heads_kv),
              "sb_attn_prefill_bf16: tiles of %d rows do not suit %d heads on %d kv heads", tile_rows, heads_q, heads_kv);
   const int row_groups = tile_rows / 16;       // more than one: waves == 4, nc == 1, head_tiles * row_groups == 4

@@ -57,8 +57,13 @@ class DecoderModel:
             if hasattr(b.mixer, "finish_build"):
                 b.mixer.finish_build()
         # heights of the runs of rows that the mixers' kernels take together (a mixer says so with
-        # a row_tile attribute); a step's context describes its rows in runs of each of them
-        self.row_tiles = sorted({int(b.mixer.row_tile) for b in self.blocks if getattr(b.mixer, "row_tile", 0)})
+        # a row_tile attribute: a height, or several); a step's context describes its rows in runs
+        # of each of them
+        heights = set()
+        for b in self.blocks:
+            asked = getattr(b.mixer, "row_tile", 0) or ()
+            heights.update((int(asked),) if isinstance(asked, int) else (int(h) for h in asked))
+        self.row_tiles = sorted(heights)
         # What every cache entry stores, and which order entries want per-sequence state.
         self.cache_specs: Dict[int, tuple] = {}
         self.state_specs: Dict[int, tuple] = {}

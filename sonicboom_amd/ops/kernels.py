@@ -744,17 +744,48 @@ def attention_row_tile(heads_q: int, heads_kv: int, head_dim: int, dtype=torch.b
     return int(library.attention_library(head_dim).sb_attn_prefill_tile_rows(int(heads_q), int(heads_kv)))
 
 
+# the prefill kernel's second form, for long prompts: tiles of 32 rows (head sizes that 32 divides,
+# up to 128, groups of three and more heads); taken when its blocks fill the GPU
+TALL_ROW_TILE = 32
+TALL_MIN_BLOCKS = 320
+
+
+def attention_tall_ok(heads_q: int, heads_kv: int, head_dim: int, dtype=torch.bfloat16) -> bool:
+    """Whether prefill attention with these heads also runs in tiles of 32 rows."""
+    if dtype != torch.bfloat16 or not attention_mfma_ok(dtype, dtype, head_dim) or not torch.cuda.is_available():
+        return False
+    fn = getattr(library.attention_library(head_dim), "sb_attn_prefill_tall_ok", None)
+    return bool(fn is not None and fn(int(heads_q), int(heads_kv)))
+
+
+def attention_row_tiles(heads_q: int, heads_kv: int, head_dim: int, dtype=torch.bfloat16):
+    """The heights of row tiles that a mixer calling :func:`attention` with these heads asks a
+    step's context for (its ``row_tile`` attribute): the usual one first."""
+    base = attention_row_tile(heads_q, heads_kv, head_dim, dtype)
+    if base != TALL_ROW_TILE and attention_tall_ok(heads_q, heads_kv, head_dim, dtype):
+        return (base, TALL_ROW_TILE)
+    return (base,)
+
+
 def attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, page_table: torch.Tensor, ctx,
               heads_q: int, heads_kv: int, head_dim: int, scale: float, window: int,
-              fast: bool = True, row_tile: int = ATTENTION_ROW_TILE) -> torch.Tensor:
+              fast: bool = True, row_tile=ATTENTION_ROW_TILE) -> torch.Tensor:
     """Attention of a step's rows over the cache; ``ctx`` is the step's context.  bfloat16 with a
     head size in steps of 16 runs on the matrix cores (a decode kernel when every sequence brings
-    one row, else the prefill kernel); everything else takes the plain kernel."""
+    one row, else the prefill kernel); everything else takes the plain kernel.  ``row_tile``: the
+    height of the context's row tiles to use, or several (what :func:`attention_row_tiles` gives):
+    tiles of 32 rows are then taken when their blocks fill the GPU."""
     if fast and attention_mfma_ok(q.dtype, k_cache.dtype, head_dim):
         if ctx.is_decode:
             return attention_decode_mfma(q, k_cache, v_cache, page_table, ctx.row_pos, heads_q, heads_kv,
                                          head_dim, scale, window)
-        return attention_prefill_mfma(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_tiles(row_tile),
-                                      heads_q, heads_kv, head_dim, scale, window, tile_rows=row_tile)
+        heights = (row_tile,) if isinstance(row_tile, int) else tuple(row_tile)
+        height = heights[0]
+        if TALL_ROW_TILE in heights[1:]:
+            blocks = ctx.row_tiles(TALL_ROW_TILE).shape[0] * heads_kv * ((heads_q // heads_kv + 7) // 8)
+            if blocks >= TALL_MIN_BLOCKS:
+                height = TALL_ROW_TILE
+        return attention_prefill_mfma(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_tiles(height),
+                                      heads_q, heads_kv, head_dim, scale, window, tile_rows=height)
     return attention_plain(q, k_cache, v_cache, page_table, ctx.row_pos, ctx.row_seq, heads_q, heads_kv,
                            head_dim, scale, window)

@@ -59,6 +59,7 @@ _ATTN_SIGNATURES = {
     # heads_kv, scale, window, stream
     "sb_attn_prefill_bf16": [_P, _P, _P, _P, _P, _I, _I, _P, _P, _I, _I, _I, _F, _I, _I, _P],
     "sb_attn_prefill_tile_rows": [_I, _I],
+    "sb_attn_prefill_tall_ok": [_I, _I],
     # out, qkv, row_stride, n_slices, bias, inv_freq, freq_factors, rot_dims, store_kv, k_cache, v_cache,
     # page_table, max_pages, n_pages, row_pos, part_o, part_ml, n_seqs, heads_q, heads_kv, scale, window,
     # pages per wave, stream

@@ -72,7 +72,7 @@ class Attention(Mixer):
         self.kv_width = self.heads_kv * self.head_dim
         if rt.fast_kernels:
             # (groups of one and two heads per kv head take higher tiles on the matrix cores)
-            self.row_tile = ops.attention_row_tile(self.heads_q, self.heads_kv, self.head_dim, rt.act_dtype)
+            self.row_tile = ops.attention_row_tiles(self.heads_q, self.heads_kv, self.head_dim, rt.act_dtype)
 
         ws = [tensors["q_weight"], tensors["k_weight"], tensors["v_weight"]]
         w_qkv = torch.cat(ws, dim=0) if all(w.dtype == ws[0].dtype for w in ws) \

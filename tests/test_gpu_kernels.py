@@ -628,7 +628,8 @@ def attention_case(hq, hkv, hd, lens, rows_per_seq, window, seed=0):
 # bring a page in; heads of more than 128 in blocks of eight waves: sixteen heads in two blocks,
 # five heads and three waves without one, eight heads; groups of one and two heads at usual head sizes)
 MFMA_SHAPES = [(4, 2, 16), (3, 1, 32), (5, 5, 48), (6, 2, 80), (28, 4, 128), (2, 1, 256), (40, 2, 64), (10, 2, 128),
-               (16, 2, 64), (8, 2, 128), (4, 1, 256), (16, 1, 192), (10, 2, 160), (8, 1, 144), (3, 3, 128), (4, 2, 64)]
+               (16, 2, 64), (8, 2, 128), (4, 1, 256), (16, 1, 192), (10, 2, 160), (8, 1, 144), (3, 3, 128), (4, 2, 64),
+               (12, 1, 96)]
 
 
 @pytest.mark.parametrize("hq, hkv, hd", MFMA_SHAPES)
@@ -713,8 +714,9 @@ def test_attention_prefill_matrix_cores(hq, hkv, hd, window):
     rows_per_seq = [list(range(s0, n)) for s0, n in zip(starts, lens)]
     q, kc, vc, table, rows, scale, want = attention_case(hq, hkv, hd, lens, rows_per_seq, window, seed=3)
     pos = torch.tensor([p for _, p in rows], dtype=torch.int32)
-    # tiles of 16 rows, and of the height that suits the group (64 and 32 rows for groups of one and two heads)
-    for height in sorted({16, ops.attention_row_tile(hq, hkv, hd)}):
+    # tiles of 16 rows, of the height that suits the group (64 and 32 rows for groups of one and two
+    # heads), and of 32 rows where the kernel has its form for long prompts
+    for height in sorted({16, ops.attention_row_tile(hq, hkv, hd)} | ({32} if ops.attention_tall_ok(hq, hkv, hd) else set())):
         tiles, row0 = [], 0
         for s_, ps in enumerate(rows_per_seq):
             for r0 in range(0, len(ps), height):
@@ -725,6 +727,9 @@ def test_attention_prefill_matrix_cores(hq, hkv, hd, window):
                                          scale, window, tile_rows=height)
         close(got, want, atol=1.5e-2, rtol=1e-2, what=f"prefill, tiles of {height} rows")
     assert ops.attention_row_tile(hq, hkv, hd) == (64 if hq == hkv else 32 if hq == 2 * hkv else 16)
+    assert ops.attention_tall_ok(hq, hkv, hd) == (hq >= 3 * hkv and hd % 32 == 0 and hd <= 128)
+    assert ops.attention_row_tiles(hq, hkv, hd) == ((16, 32) if ops.attention_tall_ok(hq, hkv, hd)
+                                                    else (ops.attention_row_tile(hq, hkv, hd),))
     if hq > 2 * hkv:
         with pytest.raises(ops.KernelLibraryError, match="do not suit"):
             ops.attention_prefill_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), tiles.to(DEV), hq, hkv, hd,
@@ -811,11 +816,12 @@ def test_attention_matrix_cores_when_the_maximum_moves(hq, hkv, hd, shape):
     want = plain.attention(q.float().numpy(), keys.reshape(n, -1).numpy(), vals.reshape(n, -1).numpy(), rows_pos,
                            np.arange(n), hq, hkv, hd, scale, causal=True, window=0)
     pos = torch.tensor(rows_pos, dtype=torch.int32)
-    tiles = torch.tensor([(r0, min(16, len(rows_pos) - r0), 0, 0) for r0 in range(0, len(rows_pos), 16)],
-                         dtype=torch.int32)
-    got = ops.attention_prefill_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), tiles.to(DEV), hq, hkv, hd,
-                                     scale, 0)
-    close(got, want, atol=1.5e-2, rtol=1e-2, what=f"prefill, {shape}")
+    for height in (16, 32) if ops.attention_tall_ok(hq, hkv, hd) else (16,):
+        tiles = torch.tensor([(r0, min(height, len(rows_pos) - r0), 0, 0) for r0 in range(0, len(rows_pos), height)],
+                             dtype=torch.int32)
+        got = ops.attention_prefill_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), tiles.to(DEV), hq, hkv, hd,
+                                         scale, 0, tile_rows=height)
+        close(got, want, atol=1.5e-2, rtol=1e-2, what=f"prefill, {shape}, tiles of {height}")
     # the same rows as single decode rows of sequences that share the pages
     for r in (0, 17, 47):
         got1 = ops.attention_decode_mfma(q[r:r + 1].to(DEV), kc, vc, table.to(DEV), pos[r:r + 1].to(DEV), hq, hkv,
@@ -915,21 +921,24 @@ def test_attention_prefill_window_edge(hq, hkv, hd, window):
     group = hq // hkv
     table = torch.tensor([[7, 2, 9, 4, 0, 5, 1, 8, 3, 6, 10]], dtype=torch.int32)
     pos = torch.tensor(rows_pos, dtype=torch.int32)
-    tiles = torch.tensor([(r0, min(16, len(rows_pos) - r0), 0, 0) for r0 in range(0, len(rows_pos), 16)],
-                         dtype=torch.int32)
-    for last_seeing in (rows_pos[0] + 20, rows_pos[0] + 47, rows_pos[0] + 48):     # inside a tile of 16, at its end, at its start
+    heights = (16, 32) if ops.attention_tall_ok(hq, hkv, hd) else (16,)
+    # inside a tile of 16, at its end, at its start; at the end of a tile of 32, at its start
+    for last_seeing in (rows_pos[0] + 20, rows_pos[0] + 47, rows_pos[0] + 48, rows_pos[0] + 63, rows_pos[0] + 64):
         d = last_seeing - window + 1
         k = keys.clone()
         k[d, :, 0] = rise
         kc, vc = fill_cache_from([k], [vals], table, BF16)
-        got = ops.attention_prefill_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), tiles.to(DEV), hq, hkv, hd,
-                                         scale, window)
         want = plain.attention(q.float().numpy(), k.reshape(n, -1).numpy(), vals.reshape(n, -1).numpy(), rows_pos,
                                np.arange(n), hq, hkv, hd, scale, causal=True, window=window)
         v_d = vals[d].repeat_interleave(group, dim=0).reshape(1, -1).numpy()
         r = last_seeing - rows_pos[0]
         assert np.abs(want[r] - v_d).max() < 2e-2 and np.abs(want[r + 1] - v_d).max() > 0.5     # the case is sharp
-        close(got, want, atol=2e-2, rtol=1e-2, what=f"window {window}, dominant key {d}")
+        for height in heights:
+            tiles = torch.tensor([(r0, min(height, len(rows_pos) - r0), 0, 0) for r0 in range(0, len(rows_pos), height)],
+                                 dtype=torch.int32)
+            got = ops.attention_prefill_mfma(q.to(DEV), kc, vc, table.to(DEV), pos.to(DEV), tiles.to(DEV), hq, hkv, hd,
+                                             scale, window, tile_rows=height)
+            close(got, want, atol=2e-2, rtol=1e-2, what=f"window {window}, dominant key {d}, tiles of {height}")
 
 
 FOLDED_SHAPES = [(4, 2, 16, 16), (3, 1, 32, 32), (5, 5, 48, 16), (6, 2, 80, 64), (28, 4, 128, 128), (16, 1, 64, 0),

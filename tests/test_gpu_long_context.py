@@ -88,9 +88,10 @@ def test_attention_decode_over_tens_of_thousands_of_keys(hq, n):
               what=f"dominant key at {far} of {n}")
 
 
+@pytest.mark.parametrize("height", [16, 32])
 @pytest.mark.parametrize("hq", [7, 8])
 @pytest.mark.parametrize("n", [16384, 32768])
-def test_attention_prefill_over_tens_of_thousands_of_keys(hq, n):
+def test_attention_prefill_over_tens_of_thousands_of_keys(hq, n, height):
     """The last 20 rows of a sequence of n tokens whose earlier keys are cached (what the second
     portion of a long prompt does), and four rows near the start."""
     from sonicboom_amd import ops
@@ -103,7 +104,7 @@ def test_attention_prefill_over_tens_of_thousands_of_keys(hq, n):
     for f in far:
         keys[f, :, 0] = rise
     kc, vc, table = paged(keys, vals, seed=11 + hq)
-    height = ops.attention_row_tile(hq, hkv, hd)
+    assert ops.attention_row_tiles(hq, hkv, hd) == (16, 32)
     pos = torch.tensor(positions, dtype=torch.int32)
     tiles = [(r, 1, 0, 0) for r in range(4)] + [(4 + r0, min(height, 20 - r0), 0, 0) for r0 in range(0, 20, height)]
     tiles = torch.tensor(tiles, dtype=torch.int32)
@@ -154,8 +155,8 @@ def test_rotation_at_positions_of_tens_of_thousands(dtype):
 
 LONG = {
     "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
-    "num_hidden_layers": 2, "hidden_size": 64, "num_attention_heads": 2, "num_key_value_heads": 1,
-    "intermediate_size": 96, "vocab_size": 300, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "num_hidden_layers": 2, "hidden_size": 96, "num_attention_heads": 3, "num_key_value_heads": 1,
+    "intermediate_size": 160, "vocab_size": 300, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
     "max_position_embeddings": 32768, "tie_word_embeddings": False, "use_sliding_window": False,
     "hidden_act": "silu",
 }
@@ -179,11 +180,15 @@ def long_case(tmp_path_factory):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_a_prompt_of_20000_tokens(long_case, dtype):
     """More rows than a step takes at once: two portions, the second over the 16,384 keys the first
-    left; then the last 8 tokens once more one by one on a second slot (decode over 19,992 keys)."""
+    left (in bfloat16 both in tiles of 32 rows, the prefill kernel's form for long prompts); then
+    the last 8 tokens once more one by one on a second slot (decode over 19,992 keys)."""
     from sonicboom_amd.engine import DecoderModel, Engine, StepEntry
     folder, tokens, want = long_case
     eng = Engine(DecoderModel.from_folder(folder, dtype), 64 * 640)
     assert len(tokens) > eng.max_step_rows
+    if dtype == "bfloat16":
+        from sonicboom_amd import ops
+        assert eng.model.row_tiles == [16, 32] and len(tokens) // 32 >= ops.TALL_MIN_BLOCKS
     s = eng.alloc_slot()
     got = eng.step([StepEntry(s, tokens, range(len(tokens) - 8, len(tokens)))]).cpu().numpy()
     assert_logits_close(got, want, dtype, "the last 8 places of 20,000", sharp=True)

@@ -125,7 +125,7 @@ def run_mixer(mixer, rt, h_rows, cuts, width):
     for n in cuts:
         entries = [StepEntry(slot, [0] * n, ())]
         cache.reserve([slot], [n])
-        ctx = StepContext(cache, entries, rt.device, [mixer.row_tile])
+        ctx = StepContext(cache, entries, rt.device, mixer.row_tile)
         x = torch.zeros((n, width), dtype=F32, device=DEV)
         mixer.forward(h_rows[start:start + n].to(DEV).contiguous(), x, ctx, binding)
         cache.advance([slot], [n])
