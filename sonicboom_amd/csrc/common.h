@@ -90,6 +90,20 @@ inline int check_launch(const char *what) {
   return SB_OK;
 }
 
+// Compute units of the current device (256 on an MI355X; fewer when the GPU is partitioned), asked
+// of the runtime once per device: what the launchers spread their blocks over.
+inline int cu_count() {
+  static int counts[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (counts[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    counts[dev] = n;
+  }
+  return counts[dev];
+}
+
 inline bool valid_dtype(int d) { return d == SB_F32 || d == SB_BF16; }
 inline size_t dtype_size(int d) { return d == SB_F32 ? 4 : 2; }
 

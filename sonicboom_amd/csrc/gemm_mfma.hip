@@ -646,7 +646,6 @@ gemm_direct16_kernel(Args a) {
   }
 }
 
-constexpr int kCus = 256;
 
 template <int MT, int NW, int BK, int DEPTH, int GATED, bool PACKED, bool EVEN_K>
 int launch_one(const Args &a, long long blocks, hipStream_t s) {
@@ -748,8 +747,8 @@ int pick_shape(int n_rows, int n_out, int n_in, int gated, bool direct_ok, doubl
     if (v == 3 || (v == 4 && !direct_ok)) continue;
     const int bm = kShapes[v].bm, bn = gated ? kShapes[v].bn / 2 : kShapes[v].bn;
     const long long tiles_m = (n_rows + bm - 1) / bm, tiles_n = (n_out + bn - 1) / bn;
-    const long long tiles = tiles_m * tiles_n, rounds = (tiles + kCus - 1) / kCus;
-    const double score = speed[v] * (double(n_rows) / double(tiles_m * bm)) * (double(tiles) / double(rounds * kCus));
+    const long long tiles = tiles_m * tiles_n, rounds = (tiles + sb::cu_count() - 1) / sb::cu_count();
+    const double score = speed[v] * (double(n_rows) / double(tiles_m * bm)) * (double(tiles) / double(rounds * sb::cu_count()));
     if (score > best) { best = score; pick = v; }
   }
   if (score_out) *score_out = best;
@@ -820,9 +819,9 @@ extern "C" int sb_gemm_mfma_bf16(void *y, int y_dtype, const void *x, const void
     if (variant == 0) rc = launch_direct<4, 2, 64, 2, false>(a, blocks, 0, s);
     else if (variant == 1) rc = launch_direct<8, 2, 64, 2, false>(a, blocks, 0, s);
     else if (variant == 2 && path == 3) rc = launch_direct<8, 4, 64, 2, false>(a, blocks, 0, s);
-    else if (variant == 2) rc = launch_direct<8, 4, 64, 2, true>(a, blocks, kCus, s);     // 128 KB of LDS: a block a CU
+    else if (variant == 2) rc = launch_direct<8, 4, 64, 2, true>(a, blocks, sb::cu_count(), s);     // 128 KB of LDS: a block a CU
     else if (variant == 3) rc = launch_direct<4, 4, 64, 2, false>(a, blocks, 0, s);
-    else rc = launch_direct<6, 4, 64, 2, true>(a, blocks, kCus, s);
+    else rc = launch_direct<6, 4, 64, 2, true>(a, blocks, sb::cu_count(), s);
   } else {
     if (variant == 0) rc = launch<2, 2, 64, 2, true>(a, blocks, packed, s);
     else if (variant == 1) rc = launch<4, 2, 64, 2, false>(a, blocks, packed, s);
@@ -860,21 +859,21 @@ PartialPlan partial_plan(int n_rows, int n_out, int n_in, bool direct_ok) {
   if (s < 1) s = 1;
   const long long big = (long long)((n_rows + 255) / 256) * ((n_out + 255) / 256);
   const long long big_grid = (big + kXcds - 1) / kXcds * kXcds;       // the grid is padded to whole eights
-  if (s == 1 && direct_ok && 2 * big_grid <= kCus) {
-    const double per_cu = 0.93e9 / kCus;                               // flops per microsecond at speed 1
+  if (s == 1 && direct_ok && 2 * big_grid <= sb::cu_count()) {
+    const double per_cu = 0.93e9 / 256.0;                                        // a CU's flops per microsecond at speed 1
     const double speed[5] = {1.0, 1.05, 1.35, 0.0, 1.35 * 0.89};
     double t_whole = 0;
     for (int v = 0; v < 5; ++v) {
       if (v == 3) continue;
       const int bm = kShapes[v].bm, bn = kShapes[v].bn;
       const long long n_tiles = (long long)((n_rows + bm - 1) / bm) * ((n_out + bn - 1) / bn);
-      const long long rounds = (n_tiles + kCus - 1) / kCus, last = n_tiles - (rounds - 1) * kCus;
+      const long long rounds = (n_tiles + sb::cu_count() - 1) / sb::cu_count(), last = n_tiles - (rounds - 1) * sb::cu_count();
       const double t = 2.0 * bm * bn * double(n_in) / (speed[v] * per_cu) * (double(rounds - 1) + load_factor(last)) + 14.0;
       if (v == 0 || t < t_whole) t_whole = t;
     }
     double t_best = 0;
     long long s_best = 0;
-    for (long long s2 = 2; s2 <= 8 && s2 * big_grid <= kCus && s2 <= n_k / 4; ++s2) {
+    for (long long s2 = 2; s2 <= 8 && s2 * big_grid <= sb::cu_count() && s2 <= n_k / 4; ++s2) {
       const int per = int((n_k + s2 - 1) / s2);
       const double t = 2.0 * 256 * 256 * (64.0 * per) / (speed[2] * per_cu) * load_factor(s2 * big_grid) + 14.0 +
                        (2.0 * s2 - 2.0) * n_rows * double(n_out) * 4.0 / 4e6;

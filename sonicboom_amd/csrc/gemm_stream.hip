@@ -208,7 +208,7 @@ inline int hint_slices(int hint) { return (hint >> 8) & 0xff; }
 // Waves per block: the count whose blocks fill whole rounds over the CUs best; more waves on a tie.
 int waves_for(int tiles, int r, int force_waves) {
   if (force_waves >= 4 && force_waves <= 8) return force_waves;
-  constexpr int n_cu = 256;   // MI355X
+  const int n_cu = sb::cu_count();
   int best = 4;
   long long best_cost = -1;
   for (int w = 4; w <= 8; ++w) {
@@ -230,7 +230,7 @@ struct Cut {
 inline int row_tiles(int n_rows) { return n_rows <= 16 ? 1 : (n_rows <= 32 ? 2 : (n_rows <= 64 ? 4 : 8)); }
 Cut cut_for(int tiles, int n_steps, int tt, int hint) {
   const int force_waves = hint_waves(hint), force_slices = hint_slices(hint);
-  constexpr int n_cu = 256;   // MI355X
+  const int n_cu = sb::cu_count();
   Cut best{4, 1, (n_steps + kAhead - 1) / kAhead * kAhead};
   long long best_cost = -1;
   for (int want = 1; want <= 8; ++want) {
