@@ -493,7 +493,7 @@ def main() -> int:
     points = {}
     if not a.no_points:
         for b in (1, 64):
-            dt, _, _, _ = decode_run(b, max(8, a.steps // 2), max(2, a.warmup // 2))
+            dt, _, _, _ = decode_run(b, max(16, a.steps // 2), max(4, a.warmup // 2))
             points[f"decode_b{b}"] = round(b / dt, 1)
             print(f"[bench] decode b{b}: {points[f'decode_b{b}']} tok/s", file=sys.stderr, flush=True)
 
