@@ -72,6 +72,9 @@ class _StaticContext(_Context):
         # the parts that never change for a decode step of this batch size: a row a sequence,
         # every row wanted, and whatever the height a run is that one row
         ar = np.arange(batch, dtype=np.int32)
+        # the tables a step rewrites, as views of each staging buffer (made once)
+        self._views = [{key: layout.view(h.numpy(), key) for key in ("ids", "row_pos", "len_before", "slots")
+                        + tuple(("table", g) for g in range(layout.n_groups))} for h in self._hosts]
         for h in self._hosts:
             n = h.numpy()
             layout.view(n, "row_seq")[:] = ar
@@ -84,22 +87,21 @@ class _StaticContext(_Context):
         """This step's ids, positions and page tables, in one copy to the device.  Fewer
         sequences than the buffers' batch: the rest are rows of token 0 at position 0 with no
         page at all (they store nothing and attend to nothing; their logits are not read)."""
-        host = self._hosts[self._turn]
+        host, views = self._hosts[self._turn], self._views[self._turn]
         self._turn ^= 1
-        n, layout = host.numpy(), self.layout
         live = len(slots)
         lengths = np.zeros(self.batch, dtype=np.int32)
         lengths[:live] = [cache.length(s) for s in slots]
-        ids = layout.view(n, "ids")
+        ids = views["ids"]
         ids[:live] = np.asarray(tokens, dtype=np.int32)
         ids[live:] = 0
-        layout.view(n, "row_pos")[:] = lengths
-        layout.view(n, "len_before")[:] = lengths
-        slot_row = layout.view(n, "slots")
+        views["row_pos"][:] = lengths
+        views["len_before"][:] = lengths
+        slot_row = views["slots"]
         slot_row[:live] = np.asarray(slots, dtype=np.int32)
         slot_row[live:] = slots[0]
-        for g in range(layout.n_groups):
-            table = layout.view(n, ("table", g))
+        for g in range(self.layout.n_groups):
+            table = views[("table", g)]
             table[:live] = cache.page_table(g, slots, min_width=self.width)
             table[live:] = -1
         self.max_len_after = int(lengths.max()) + 1
