@@ -943,30 +943,10 @@ attn_prefill_tall_kernel(bf16_t *__restrict__ out, const bf16_t *__restrict__ q,
 // Partial results, when a row's keys span several chunks, go to
 //   part_o  float [seqs][tiles][n_chunks][HD][16]   (unnormalised sums, column fastest)
 //   part_ml float [seqs][tiles][n_chunks][2][16]    (maximum, sum)
-// and are merged in ascending chunk order by attn_decode_merge_kernel.  (Merging in the block
+// and are merged by attn_decode_merge_kernel (up to 16 chunks, in ascending order) or
+// attn_decode_merge_many_kernel.  (Merging in the block
 // that finishes last was tried and dropped: the device-scope fences it needs write back and
 // invalidate whole L2 caches on this multi-die GPU and cost far more than the second launch.)
-// Element e = d * 16 + column of a (sequence, tile): the chunks' partial sums, rescaled to the
-// common maximum and added in ascending chunk order.
-__device__ __forceinline__ void merge_element(bf16_t *__restrict__ out, const float *__restrict__ po,
-                                              const float *__restrict__ pml, int e, int first, int last,
-                                              int seq, int heads_q, int kvh, int ht, int group) {
-  const int c = e & 15, d = e >> 4;
-  const int hh = ht * 16 + c;
-  if (hh >= group) return;
-  float m = -__builtin_inff();
-#pragma unroll 4
-  for (int ch = first; ch <= last; ++ch) m = fmaxf(m, pml[size_t(ch) * 32 + c]);
-  const float m_use = m == -__builtin_inff() ? 0.f : m;
-  float o = 0.f, l = 0.f;
-#pragma unroll 4
-  for (int ch = first; ch <= last; ++ch) {
-    const float f = __builtin_amdgcn_exp2f(pml[size_t(ch) * 32 + c] - m_use);
-    o += po[size_t(ch) * (HD * 16) + e] * f;
-    l += pml[size_t(ch) * 32 + 16 + c] * f;
-  }
-  out[(size_t(seq) * heads_q + kvh * group + hh) * HD + d] = f32_to_bf16(l > 0.f ? o / l : 0.f);
-}
 
 // Decode grids have one dimension, the block number counting the (kv head x head tile) fastest,
 // then the sequence, the chunk of pages slowest.  Blocks go to the GPU's eight dies in turn by
@@ -1526,8 +1506,8 @@ attn_decode_long_kernel(bf16_t *__restrict__ out, float *__restrict__ part_o, fl
                       seq, kvh, ht, group, heads_q, n_chunks, size_t(seq) * tiles + blk.tile);
 }
 
-// Merge the chunks of a (sequence, tile) in ascending order: one thread per (d, column).
-// Grid (HD * 16 / 256, tiles, sequences).
+// Merge the chunks of a (sequence, tile), at most kAtOnce of them, in ascending order: one thread
+// per element e = d * 16 + column.  Grid (HD * 16 / 256, tiles, sequences).
 __global__ void __launch_bounds__(256)
 attn_decode_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o,
                          const float *__restrict__ part_ml, const int32_t *__restrict__ row_pos,
@@ -1545,8 +1525,7 @@ attn_decode_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ par
   // waiting for the position first costs this short kernel a trip to memory of its two.
   constexpr int kAtOnce = 16;
   float mv[kAtOnce], lv[kAtOnce], ov[kAtOnce];
-  const bool at_once = n_chunks <= kAtOnce && e < HD * 16;
-  if (at_once) {
+  {
     const int c = e & 15;
 #pragma unroll
     for (int ch = 0; ch < kAtOnce; ++ch) {
@@ -1559,12 +1538,7 @@ attn_decode_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ par
   const int key_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
   const int first = key_lo / (SB_PAGE * pages_per_chunk), last = min(pos / (SB_PAGE * pages_per_chunk), n_chunks - 1);
   if (first == last) return;      // the decode kernel has written the result itself
-  if (e >= HD * 16) return;
-  if (!at_once) {
-    merge_element(out, po, pml, e, first, last, seq, heads_q, kvh, ht, group);
-    return;
-  }
-  // as merge_element: rescaled to the common maximum and added in ascending chunk order
+  // rescaled to the common maximum and added in ascending chunk order
   const int c = e & 15, d = e >> 4;
   const int hh = ht * 16 + c;
   if (hh >= group) return;
@@ -1581,6 +1555,79 @@ attn_decode_merge_kernel(bf16_t *__restrict__ out, const float *__restrict__ par
     l = use ? l + lv[ch] * f : l;
   }
   out[(size_t(seq) * heads_q + kvh * group + hh) * HD + d] = f32_to_bf16(l > 0.f ? o / l : 0.f);
+}
+
+// The same for rows of many chunks: a block takes 64 elements, its four waves every fourth
+// chunk each, eight chunks' partial results in flight at a time (one thread walking all chunks
+// waits for memory once per few chunks: 128 chunks took it longer than the decode kernel took to
+// read the keys).  A wave keeps a running maximum of its own; the four meet in LDS and are folded
+// in wave order.  Grid (HD * 16 / 64, tiles, sequences).
+__global__ void __launch_bounds__(256)
+attn_decode_merge_many_kernel(bf16_t *__restrict__ out, const float *__restrict__ part_o,
+                              const float *__restrict__ part_ml, const int32_t *__restrict__ row_pos,
+                              int heads_q, int heads_kv, int n_chunks, int window, int pages_per_chunk) {
+  __shared__ float lds_m[4][64], lds_l[4][64], lds_o[4][64];
+  const int seq = blockIdx.z;
+  const int group = heads_q / heads_kv;
+  const int head_tiles = (group + 15) / 16;
+  const int kvh = blockIdx.y / head_tiles, ht = blockIdx.y - kvh * head_tiles;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int e = blockIdx.x * 64 + lane;                 // < HD * 16: 64 divides it
+  const int c = e & 15, d = e >> 4;
+  const size_t tile_index = size_t(seq) * gridDim.y + blockIdx.y;
+  const float *po = part_o + (tile_index * n_chunks) * (HD * 16), *pml = part_ml + (tile_index * n_chunks) * 32;
+  constexpr int kAtOnce = 8;
+  float mv[kAtOnce], lv[kAtOnce], ov[kAtOnce];
+  auto ask = [&](int base) __attribute__((always_inline)) {
+#pragma unroll
+    for (int i = 0; i < kAtOnce; ++i) {
+      const size_t cc = size_t(min(base + 4 * i, n_chunks - 1));   // (past the end: the last once more, not used)
+      mv[i] = pml[cc * 32 + c];
+      lv[i] = pml[cc * 32 + 16 + c];
+      ov[i] = po[cc * (HD * 16) + e];
+    }
+  };
+  // the first round goes out together with the position, which says which chunks count
+  ask(wave);
+  const int pos = row_pos[seq];
+  const int key_lo = (window > 0 && pos >= window) ? pos - window + 1 : 0;
+  const int first = key_lo / (SB_PAGE * pages_per_chunk), last = min(pos / (SB_PAGE * pages_per_chunk), n_chunks - 1);
+  if (first == last) return;      // the decode kernel has written the result itself
+  float m = -__builtin_inff(), o = 0.f, l = 0.f;
+  for (int base = wave;; base += 4 * kAtOnce) {
+    if (base + 4 * (kAtOnce - 1) >= first) {
+#pragma unroll
+      for (int i = 0; i < kAtOnce; ++i) {
+        const int ch = base + 4 * i;
+        const bool use = ch >= first && ch <= last;
+        const float m_new = use ? fmaxf(m, mv[i]) : m;
+        const float m_use = m_new == -__builtin_inff() ? 0.f : m_new;
+        const float keep = __builtin_amdgcn_exp2f(m - m_use), f = use ? __builtin_amdgcn_exp2f(mv[i] - m_use) : 0.f;
+        o = o * keep + (use ? ov[i] * f : 0.f);
+        l = l * keep + (use ? lv[i] * f : 0.f);
+        m = m_new;
+      }
+    }
+    if (base + 4 * kAtOnce > last) break;
+    ask(base + 4 * kAtOnce);
+  }
+  lds_m[wave][lane] = m;
+  lds_l[wave][lane] = l;
+  lds_o[wave][lane] = o;
+  __syncthreads();
+  if (wave != 0) return;
+  const int hh = ht * 16 + c;
+  if (hh >= group) return;
+  float m_all = fmaxf(fmaxf(lds_m[0][lane], lds_m[1][lane]), fmaxf(lds_m[2][lane], lds_m[3][lane]));
+  if (m_all == -__builtin_inff()) m_all = 0.f;
+  float o_all = 0.f, l_all = 0.f;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const float f = __builtin_amdgcn_exp2f(lds_m[w][lane] - m_all);
+    o_all += lds_o[w][lane] * f;
+    l_all += lds_l[w][lane] * f;
+  }
+  out[(size_t(seq) * heads_q + kvh * group + hh) * HD + d] = f32_to_bf16(l_all > 0.f ? o_all / l_all : 0.f);
 }
 
 int check_common(const void *out, const void *q, const void *k, const void *v, const void *pt,
@@ -1658,7 +1705,10 @@ int decode_launch(const char *who, void *out, const void *q, const RopeArgs &ra,
       // time: 260 equal blocks take as long as 512 (measured: 65 sequences x 4 kv heads x 2,048
       // keys 77 us in one chunk against 45 for 64 sequences, 63 in chunks of eight pages)
       const long long n_busy = per_chunk * full;
-      const double uneven = n_busy > 256 ? double((n_busy + 255) / 256) * 256.0 / double(n_busy) : 1.0;
+      // (blocks of few pages in a row pay less of it, the CU's second block being short: 260
+      // blocks of two pages a wave took 22.7 us where 130 of four took 25.7)
+      const double rounds = n_busy > 256 ? double((n_busy + 255) / 256) * 256.0 / double(n_busy) : 1.0;
+      const double uneven = 1.0 + (rounds - 1.0) * (run < 8 ? run / 8.0 : 1.0);
       const double stream_us =
           double(per_chunk) * pages * page_bytes / rate * (1.0 + 4.0 / (run * 3.3)) * uneven;
       const double in_a_row = run * 3.3 + 4.0;
@@ -1691,8 +1741,12 @@ int decode_launch(const char *who, void *out, const void *q, const RopeArgs &ra,
 #undef SB_ARGS
   int rc = sb::check_launch(who);
   if (rc != SB_OK || n_chunks == 1) return rc;
-  attn_decode_merge_kernel<<<dim3((HD * 16 + 255) / 256, heads_kv * head_tiles, n_seqs), 256, 0, s>>>(
-      (bf16_t *)out, part_o, part_ml, row_pos, heads_q, heads_kv, n_chunks, window, pages_per_chunk);
+  if (n_chunks <= 16)
+    attn_decode_merge_kernel<<<dim3((HD * 16 + 255) / 256, heads_kv * head_tiles, n_seqs), 256, 0, s>>>(
+        (bf16_t *)out, part_o, part_ml, row_pos, heads_q, heads_kv, n_chunks, window, pages_per_chunk);
+  else
+    attn_decode_merge_many_kernel<<<dim3(HD * 16 / 64, heads_kv * head_tiles, n_seqs), 256, 0, s>>>(
+        (bf16_t *)out, part_o, part_ml, row_pos, heads_q, heads_kv, n_chunks, window, pages_per_chunk);
   return sb::check_launch(who);
 }
 

@@ -88,6 +88,36 @@ def test_attention_decode_over_tens_of_thousands_of_keys(hq, n):
               what=f"dominant key at {far} of {n}")
 
 
+@pytest.mark.parametrize("pages", [1, 2])
+@pytest.mark.parametrize("window", [1000, 9000])
+def test_attention_decode_window_edge_in_a_far_chunk(window, pages):
+    """A window over a row of 20,000 keys cut into some eighty to a hundred and sixty chunks: the
+    chunks before the window's first are never written and must not be read as results, the
+    window's first key must count and the key before it must not, and the position lies in a
+    chunk that is not full.  (The second kernel, which merges the chunks, takes them in rounds
+    when they are many; the window starts in a later round than the first.)"""
+    from sonicboom_amd import ops
+    hq, hkv, hd, n = 6, 2, 128, 20000
+    keys, vals, q, rise, scale = looking_along_zero(n, hq, hkv, hd, 1, seed=61)
+    group = hq // hkv
+    for p in (n - 1, 19000):
+        for inside in (False, True):
+            k = keys.clone()
+            edge = p - window + (1 if inside else 0)
+            k[edge, :, 0] = rise
+            kc, vc, table = paged(k, vals, seed=5)
+            pos = torch.tensor([p], dtype=torch.int32, device=DEV)
+            with ops.attention_decode_pages_per_wave(hd, pages):
+                got = ops.attention_decode_mfma(q.to(DEV), kc, vc, table.to(DEV), pos, hq, hkv, hd, scale, window)
+            if inside:
+                want = vals[edge].repeat_interleave(group, dim=0).reshape(1, -1).numpy()
+            else:
+                want = plain.attention(q.float().numpy(), k.reshape(n, -1).numpy(), vals.reshape(n, -1).numpy(), [p],
+                                       np.arange(n), hq, hkv, hd, scale, causal=True, window=window)
+                assert np.abs(want - vals[edge].repeat_interleave(group, dim=0).reshape(1, -1).numpy()).max() > 0.5
+            close(got, want, atol=2e-2, rtol=1e-2, what=f"position {p}, window {window}, key {edge}")
+
+
 @pytest.mark.parametrize("height", [16, 32])
 @pytest.mark.parametrize("hq", [7, 8])
 @pytest.mark.parametrize("n", [16384, 32768])
