@@ -2,7 +2,7 @@
 MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--layers L]
-                    [--sizes 0.5b|1.5b|3b|7b|14b|32b|72b] [--prompt T] [--context C] [--workload steady|mixed]
+                    [--sizes 0.5b|1.5b|3b|7b|14b|32b|72b] [--prompt T] [--context C] [--workload steady|mixed|forms]
 
 A "step" is one decode step: every sequence of the batch goes on by one token (step function,
 greedy choice on the device, the token fed back).
@@ -27,6 +27,10 @@ Beside the JSON line on standard output, every metric goes to standard error as 
 loop itself: ``--sizes 14b``: 16 prompts of seeded lengths uniform in [256, 4096] in a cache of
 8192 tokens a sequence, prompts in one step, then 256 greedy steps; ``--sizes 72b``: 8 prompts of
 512 to 2048 tokens, 128 steps, 4096 tokens a sequence.  Prefill and decode are timed apart.
+
+``--workload forms`` prints a table instead of the line: the decode step (``--batches 1,8``) with
+the qkv, output and down product forced, one at a time, to every form (waves a block x K slices)
+of the kernel that streams the weights, against the launchers' own choices.
 """
 import argparse
 import json
@@ -245,7 +249,8 @@ def main() -> int:
     ap.add_argument("--sizes", choices=sorted(SIZES), default="7b", help="layer sizes (default: the benchmark's)")
     ap.add_argument("--prompt", type=int, default=PROMPT, help="cached prompt tokens per sequence")
     ap.add_argument("--context", type=int, default=CONTEXT, help="cache size per sequence")
-    ap.add_argument("--workload", choices=("steady", "mixed"), default="steady")
+    ap.add_argument("--workload", choices=("steady", "mixed", "forms"), default="steady")
+    ap.add_argument("--batches", default="1,8", help="--workload forms: the batch sizes, comma separated")
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and batch 64 points")
     ap.add_argument("--no-graph", action="store_true", help="launch decode steps kernel by kernel")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel rates")
@@ -320,6 +325,56 @@ def main() -> int:
         return time.perf_counter() - t
 
     # ------------------------------------------------------------------------------------------
+    if a.workload == "forms":
+        # The decode step with one product at a time forced to every form of the weight-streaming
+        # kernel (waves a block x K slices), everything else as the launchers choose: a table on
+        # standard output, no JSON line.  The products are told apart by their packed shapes.
+        d, ff = m["d"], m["ff"]
+        targets = {"qkv": ((m["hq"] + 2 * m["hkv"]) * m["hd"], d), "out": (d, m["hq"] * m["hd"]), "down": (d, ff)}
+        forced = {"shape": None, "form": (0, 0)}
+        launcher_partial = ops.gemm_bf16_partial
+
+        def partial(x, w, packed_shape=None):
+            if packed_shape is not None and tuple(packed_shape) == forced["shape"]:
+                with ops.gemm_few_rows_kernel(None, *forced["form"]):
+                    return launcher_partial(x, w, packed_shape=packed_shape)
+            return launcher_partial(x, w, packed_shape=packed_shape)
+        ops.gemm_bf16_partial = partial
+        layers = cfg["num_hidden_layers"]
+        slice_counts = (1, 2, 3, 4, 5, 6, 8)
+        for batch in (int(b) for b in a.batches.split(",")):
+            eng = Engine(model, ((PROMPT + 511) // 64) * 64 * batch, max_slots=batch)
+            slots = [eng.alloc_slot() for _ in range(batch)]
+            eng.step([StepEntry(s, p, (PROMPT - 1,)) for s, p in zip(slots, random_prompts([PROMPT] * batch))])
+
+            def step_ms(shape, form):
+                forced["shape"], forced["form"] = shape, form
+                loop = DecodeLoop(eng, use_graph=not a.no_graph)
+                loop.start(slots, [1] * batch)
+                for _ in range(4):
+                    loop.step()
+                times = [sync_time(loop.step) for _ in range(24)]
+                loop.close()
+                for s in slots:
+                    eng.cache.truncate(s, PROMPT)
+                return statistics.median(times) * 1e3
+            own = statistics.median(step_ms(None, (0, 0)) for _ in range(3))
+            print(f"{model_name} sizes, batch {batch}, {PROMPT} cached tokens: the launchers' own choices {own:.4f} ms a step")
+            for name, shape in targets.items():
+                print(f"  {name} {shape[0]} x {shape[1]} ({shape[0] * shape[1] * 2 / 1e6:.1f} MB); step in ms (difference a layer "
+                      f"in us) by waves; columns: {', '.join(str(c) for c in slice_counts)} slices", flush=True)
+                for waves in (4, 5, 6, 7, 8):
+                    cells = []
+                    for slices in slice_counts:
+                        t = step_ms(shape, (waves, slices))
+                        cells.append(f"{t:.3f} ({(t - own) * 1e3 / layers:+.2f})")
+                    print(f"    {waves} waves: " + "  ".join(cells), flush=True)
+            for s in slots:
+                eng.free_slot(s)
+            del eng
+        ops.gemm_bf16_partial = launcher_partial
+        return 0
+
     if a.workload == "mixed":
         n_prompts, shortest, longest, n_steps, per_seq = MIXED.get(a.sizes, MIXED_DEFAULT)
         lengths = [int(n) for n in rng.integers(shortest, longest + 1, size=n_prompts)]
