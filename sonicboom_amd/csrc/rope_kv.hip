@@ -143,11 +143,11 @@ rope_kv_kernel(TQ *__restrict__ q_out, const TI *__restrict__ qkv, int row_strid
   }
 }
 
-// Many rows without slices or a bias (a prompt step's qkv rows as the tiled product leaves
-// them), bfloat16 queries and cache, head size and rotary width in 16s: a thread moves eight
-// pairs at a time, 16 bytes per load and store instead of two or four.  One block per row.  The
-// arithmetic is rope_kv_kernel's (every element through float, the same rotate_pair), so the
-// bits are the same.
+// Many rows (a prompt step's qkv rows as the tiled product leaves them, whole or in K slices,
+// with or without a bias still to add), bfloat16 queries and cache, head size and rotary width in
+// 16s: a thread moves eight pairs at a time, 16 bytes per load and store instead of two or four.
+// One block per row.  The arithmetic is rope_kv_kernel's (slices added in ascending order, then
+// the bias, every element through float, the same rotate_pair), so the bits are the same.
 __device__ __forceinline__ void load_eight(float (&f)[8], const float *p) {
   const float4 a = *reinterpret_cast<const float4 *>(p), b = *reinterpret_cast<const float4 *>(p + 4);
   f[0] = a.x; f[1] = a.y; f[2] = a.z; f[3] = a.w; f[4] = b.x; f[5] = b.y; f[6] = b.z; f[7] = b.w;
@@ -161,9 +161,33 @@ __device__ __forceinline__ void load_eight(float (&f)[8], const bf16_t *p) {
     f[2 * e + 1] = bf16_to_f32(bf16_t(w[e] >> 16));
   }
 }
-template <typename TI>
+// Eight elements from e on of a qkv row, as qkv_at gives them one by one.
+template <int SLICES, typename TI>
+__device__ __forceinline__ void qkv_eight(float (&f)[8], const TI *r, size_t e, int n_slices, size_t slice_stride,
+                                          const float *bias) {
+  float part[SLICES][8];
+#pragma unroll
+  for (int s = 0; s < SLICES; ++s)
+    if (s == 0 || s < n_slices) load_eight(part[s], r + s * slice_stride + e);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) f[i] = part[0][i];
+#pragma unroll
+  for (int s = 1; s < SLICES; ++s)
+    if (s < n_slices) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f[i] += part[s][i];
+    }
+  if (bias) {
+    float b[8];
+    load_eight(b, bias + e);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = f[i] + b[i];
+  }
+}
+template <typename TI, int SLICES>
 __global__ void __launch_bounds__(256)
-rope_kv_rows_kernel(bf16_t *__restrict__ q_out, const TI *__restrict__ qkv, int row_stride,
+rope_kv_rows_kernel(bf16_t *__restrict__ q_out, const TI *__restrict__ qkv, int row_stride, int n_slices,
+                    size_t slice_stride, const float *__restrict__ bias,
                     const float *__restrict__ inv_freq, const float *__restrict__ freq_factors, int rot_dims,
                     const int32_t *__restrict__ row_pos, const int32_t *__restrict__ row_seq,
                     bf16_t *__restrict__ k_cache, bf16_t *__restrict__ v_cache,
@@ -207,7 +231,7 @@ rope_kv_rows_kernel(bf16_t *__restrict__ q_out, const TI *__restrict__ qkv, int 
   const int n_qk = (heads_q + (store ? heads_kv : 0)) * per_head;
   for (int it = threadIdx.x; it < n_qk; it += blockDim.x) {
     const int head = it / per_head, w = it % per_head;
-    const TI *src = r + size_t(head) * head_dim;
+    const size_t src = size_t(head) * head_dim;           // where the head starts in the row
     // a group of eight (d0 a multiple of 8) goes to the query row as it is, into the cache at the
     // group's place in the cache's order
     const bool is_q = head < heads_q;
@@ -216,8 +240,8 @@ rope_kv_rows_kernel(bf16_t *__restrict__ q_out, const TI *__restrict__ qkv, int 
     if (w < pair_groups) {
       const int i0 = w * 8;
       float lo[8], hi[8], y0[8], y1[8];
-      load_eight(lo, src + i0);
-      load_eight(hi, src + i0 + half);
+      qkv_eight<SLICES>(lo, r, src + i0, n_slices, slice_stride, bias);
+      qkv_eight<SLICES>(hi, r, src + i0 + half, n_slices, slice_stride, bias);
 #pragma unroll
       for (int e = 0; e < 8; ++e) rotate_pair(lo[e], hi[e], cs[i0 + e], sn[i0 + e], y0[e], y1[e]);
       *reinterpret_cast<uint4 *>(dst + at(i0)) = pack(y0);
@@ -225,7 +249,7 @@ rope_kv_rows_kernel(bf16_t *__restrict__ q_out, const TI *__restrict__ qkv, int 
     } else {
       const int d0 = 2 * half + (w - pair_groups) * 8;
       float v[8];
-      load_eight(v, src + d0);
+      qkv_eight<SLICES>(v, r, src + d0, n_slices, slice_stride, bias);
       *reinterpret_cast<uint4 *>(dst + at(d0)) = pack(v);
     }
   }
@@ -235,7 +259,7 @@ rope_kv_rows_kernel(bf16_t *__restrict__ q_out, const TI *__restrict__ qkv, int 
   for (int it = threadIdx.x; it < heads_kv * groups; it += blockDim.x) {
     const int kh = it / groups, d0 = (it % groups) * 8;
     float v[8];
-    load_eight(v, r + size_t(heads_q + heads_kv + kh) * head_dim + d0);
+    qkv_eight<SLICES>(v, r, size_t(heads_q + heads_kv + kh) * head_dim + d0, n_slices, slice_stride, bias);
 #pragma unroll
     for (int e = 0; e < 8; ++e) v_cache[page_base + kh * head_step + sb_value_index(d0 + e, slot)] = f32_to_bf16(v[e]);
   }
@@ -276,16 +300,24 @@ extern "C" int sb_rope_kv_store(void *q_out, int q_dtype, const void *qkv, int q
   const int n_heads = heads_q + 2 * heads_kv;
   const uintptr_t addresses = reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(q_out) |
                               reinterpret_cast<uintptr_t>(k_cache);
-  if (n_rows >= 512 && q_dtype == SB_BF16 && cache_dtype == SB_BF16 && n_slices == 1 && !bias && head_dim % 8 == 0 &&
-      row_stride % 8 == 0 && (!inv_freq || rot_dims % 16 == 0) && addresses % 16 == 0) {
-    if (qkv_dtype == SB_BF16)
-      rope_kv_rows_kernel<bf16_t><<<n_rows, 256, 0, s>>>(
-          (bf16_t *)q_out, (const bf16_t *)qkv, row_stride, inv_freq, freq_factors, rot_dims, row_pos, row_seq,
-          (bf16_t *)k_cache, (bf16_t *)v_cache, page_table, max_pages, n_pages_total, heads_q, heads_kv, head_dim);
-    else
-      rope_kv_rows_kernel<float><<<n_rows, 256, 0, s>>>(
-          (bf16_t *)q_out, (const float *)qkv, row_stride, inv_freq, freq_factors, rot_dims, row_pos, row_seq,
-          (bf16_t *)k_cache, (bf16_t *)v_cache, page_table, max_pages, n_pages_total, heads_q, heads_kv, head_dim);
+  const uintptr_t bias_address = reinterpret_cast<uintptr_t>(bias);
+  if (n_rows >= 512 && q_dtype == SB_BF16 && cache_dtype == SB_BF16 && head_dim % 8 == 0 && row_stride % 8 == 0 &&
+      (!inv_freq || rot_dims % 16 == 0) && (addresses | bias_address) % 16 == 0) {
+#define SB_ROWS(TI, SLICES)                                                                              \
+  rope_kv_rows_kernel<TI, SLICES><<<n_rows, 256, 0, s>>>(                                                \
+      (bf16_t *)q_out, (const TI *)qkv, row_stride, n_slices, slice_stride, bias, inv_freq, freq_factors, \
+      rot_dims, row_pos, row_seq, (bf16_t *)k_cache, (bf16_t *)v_cache, page_table, max_pages,           \
+      n_pages_total, heads_q, heads_kv, head_dim)
+    if (qkv_dtype == SB_BF16) {
+      if (n_slices == 1) SB_ROWS(bf16_t, 1);
+      else if (n_slices <= 4) SB_ROWS(bf16_t, 4);
+      else SB_ROWS(bf16_t, kMaxSlices);
+    } else {
+      if (n_slices == 1) SB_ROWS(float, 1);
+      else if (n_slices <= 4) SB_ROWS(float, 4);
+      else SB_ROWS(float, kMaxSlices);
+    }
+#undef SB_ROWS
     return sb::check_launch("sb_rope_kv_store");
   }
   const int heads_per_block = n_rows >= 512 ? n_heads : 4;

@@ -524,6 +524,39 @@ def test_rope_kv_store_rows_eight_pairs_at_a_time(hq, hkv, hd, rot, rotate, in_d
         assert torch.equal(results[0][0], qkv[:, :hq * hd].to(BF16))
 
 
+@pytest.mark.parametrize("hq, hkv, hd, rot", [(28, 4, 128, 0), (3, 3, 64, 32), (5, 2, 80, 0)])
+@pytest.mark.parametrize("slices", [2, 3, 5])
+@pytest.mark.parametrize("in_dtype", [F32, BF16])
+def test_rope_kv_store_rows_in_slices_with_a_bias(hq, hkv, hd, rot, slices, in_dtype):
+    """The same kernel takes a prompt's qkv rows as K slices of the product with the bias still to
+    add (what the sliced product of a few hundred rows leaves): slices added in ascending order,
+    then the bias, bitwise as the element-wise kernel does it in calls of 100 rows, and the sum is
+    the plain rotation of the summed rows."""
+    from sonicboom_amd import ops
+    n, w = 700, (hq + 2 * hkv) * hd
+    parts = randn(slices, n, w, dtype=in_dtype).to(DEV)
+    bias = randn(w, scale=0.1, seed=3).to(DEV)
+    pos = (torch.arange(n, dtype=torch.int32) * 3 % 701).to(DEV)
+    seq = torch.zeros(n, dtype=torch.int32, device=DEV)
+    table = torch.tensor([[4, 9, 1, 7, 3, 10, 0, 6, 2, 8, 5]], dtype=torch.int32, device=DEV)
+    dims = rot or hd
+    inv = torch.exp(-2.0 * torch.arange(dims // 2, dtype=F32) / dims * math.log(1e6)).to(DEV)
+    results = []
+    for step in (n, 100):
+        kc, vc = make_cache(11, hkv, hd, BF16, fill=0.0)
+        qs = [ops.rope_kv_store(parts[:, r0:r0 + step].contiguous(), BF16, inv, None, dims, pos[r0:r0 + step],
+                                seq[r0:r0 + step], kc, vc, table, hq, hkv, hd, bias=bias) for r0 in range(0, n, step)]
+        results.append((torch.cat(qs), kc, vc))
+    for a, b in zip(*results):
+        assert torch.equal(a, b)
+    rows = parts.float().sum(dim=0).cpu() + bias.cpu()
+    want_q = plain.rope_neox(rows[:, :hq * hd].numpy(), pos.cpu().numpy(), hd, 1e6, rot, None)
+    close(results[0][0], want_q, atol=3e-2, rtol=8e-3, what="q of the long prompt")
+    page, slot = int(table[0, int(pos[650]) // 64]), int(pos[650]) % 64
+    close(layout.get_value(results[0][2], page, slot).reshape(-1), rows[650, (hq + hkv) * hd:].to(BF16).float(),
+          atol=2e-2, rtol=8e-3, what="a value row")
+
+
 def test_rope_reference_vectors():
     """/root/reference/tests/core/test_nn.cpp:221-290: position 0 is the identity; with
     head size 2 and an angle of pi/2, [1,0] turns into [0,1]; pairs are (i, i+half)."""
