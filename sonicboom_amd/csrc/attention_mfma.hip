@@ -1685,7 +1685,8 @@ int decode_launch(const char *who, void *out, const void *q, const RopeArgs &ra,
     // How many pages in a row: the count with the least estimated time, in microseconds, from
     // what was measured (MI355X, cold caches).  A wave gets through a page in about 3.3 us
     // whatever the head size (two round trips to memory); a CU streams about 27 GB/s, all of
-    // them together 5.3 TB/s; a block costs about 4 us besides; more than one chunk costs the
+    // them together 5.3 TB/s; a block costs about 2 us besides (fitted: with 4 the choices lost 42 us over
+    // 29 measured cases of 1 to 128 sequences and 2,000 to 131,000 keys, with 2 they lose 5); more than one chunk costs the
     // partial results and the second kernel, about 8 us.  The table's width is taken for the rows' length less half of the 16
     // pages it is rounded up by.  One chunk (a quarter of the width per wave) is among the
     // candidates: it wins when sequences x kv heads alone fill most of the GPU.
@@ -1700,7 +1701,7 @@ int decode_launch(const char *who, void *out, const void *q, const RopeArgs &ra,
       const double busy = double(per_chunk) * full < 256.0 ? double(per_chunk) * full : 256.0;
       const double rate = busy * 27e3 < 5.3e6 ? busy * 27e3 : 5.3e6;            // bytes per us
       const int run = c < pages ? c : pages;
-      // a block spends about 4 us on what is not streaming (look-ups, queries, the merge)
+      // a block spends about 2 us on what is not streaming (look-ups, queries, the merge)
       // blocks that a CU holds together share its rate, so the CU with the most blocks sets the
       // time: 260 equal blocks take as long as 512 (measured: 65 sequences x 4 kv heads x 2,048
       // keys 77 us in one chunk against 45 for 64 sequences, 63 in chunks of eight pages)
@@ -1710,8 +1711,8 @@ int decode_launch(const char *who, void *out, const void *q, const RopeArgs &ra,
       const double rounds = n_busy > 256 ? double((n_busy + 255) / 256) * 256.0 / double(n_busy) : 1.0;
       const double uneven = 1.0 + (rounds - 1.0) * (run < 8 ? run / 8.0 : 1.0);
       const double stream_us =
-          double(per_chunk) * pages * page_bytes / rate * (1.0 + 4.0 / (run * 3.3)) * uneven;
-      const double in_a_row = run * 3.3 + 4.0;
+          double(per_chunk) * pages * page_bytes / rate * (1.0 + 2.0 / (run * 3.3)) * uneven;
+      const double in_a_row = run * 3.3 + 2.0;
       const double t = (stream_us > in_a_row ? stream_us : in_a_row) + (chunks > 1 ? 8.0 : 0.0);
       if (best < 0.0 || t < best) best = t, ppw = c;
     }
