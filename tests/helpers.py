@@ -47,8 +47,9 @@ def forget_plain(folder):
 # a fraction of the spread plus a fraction of itself, and the root mean square of all differences,
 # which rounding keeps small and a systematic mistake does not, has a tighter bound of its own.
 # On the "sharp" models (conftest.SHARP_QK) scores of ten and more make the softmax amplify the
-# rounding of queries and keys: measured on the GPU the largest difference was 0.23 spreads and
-# the root mean square 0.022, against 0.018 and 0.004 on the tiny models of plain random weights.
+# rounding of queries and keys: measured on the GPU over the whole suite the largest difference
+# was 0.287 spreads and the root mean square 0.0233, against 0.0257 and 0.0055 on the tiny models
+# of plain random weights; the bounds of both kinds are what was measured times 1.4.
 # "wide" is for models of real layer sizes, where a row of 3,584 and a sum over 18,944 products
 # round more often: measured 0.066 and 0.013 there (the largest over two layers of the 7B, 14B and
 # 72B sizes; the 7B sizes alone 0.058 and 0.0095), where the smallest of the mistakes that
@@ -56,8 +57,8 @@ def forget_plain(folder):
 # moves the plain logits by 0.20 and 0.031 (a wrong scale by 4.6 and 0.88): the bounds are what
 # was measured times 1.4, and that mistake is 2.2 and 1.7 times beyond them.
 F32_TOL = dict(atol=5e-5, rtol=5e-5)
-BF16_MAX = {"tiny": 0.04, "wide": 0.09, "sharp": 0.5}     # largest difference, in spreads (plus BF16_REL * |logit|)
-BF16_RMS = {"tiny": 0.01, "wide": 0.018, "sharp": 0.05}   # root mean square of the differences, in spreads
+BF16_MAX = {"tiny": 0.036, "wide": 0.09, "sharp": 0.4}     # largest difference, in spreads (plus BF16_REL * |logit|)
+BF16_RMS = {"tiny": 0.008, "wide": 0.018, "sharp": 0.033}   # root mean square of the differences, in spreads
 BF16_REL = 0.02
 # the largest of both that the bfloat16 comparisons of this run have seen, by kind (the summary
 # at the end of a test run prints them: what the bounds above are set from)
