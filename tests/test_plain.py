@@ -336,7 +336,7 @@ def test_sharp_models_show_attention_mistakes(models, sharp_folders):
         tokens = [int(t) for t in rng(14).integers(0, cfg["vocab_size"], size=65)]
         for what in mistakes:
             by_max, by_rms = moved(cfg, w, tokens, what, True)
-            assert by_max > 2.0 and by_rms > 3.0, \
+            assert by_max > 4.0 and by_rms > 5.0, \
                 f"sharp {name}: a wrong {what} is {by_max:.2f} bounds at its largest, {by_rms:.2f} in the mean"
         soft_cfg, soft_w = models[name]
         hidden = [what for what in mistakes if max(moved(soft_cfg, soft_w, tokens, what, False)) < 1.0]
